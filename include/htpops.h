@@ -1,0 +1,161 @@
+/*
+ * htpops.h -- C ABI of the MI355X (gfx950) op backend.
+ *
+ * One context owns one HIP stream; ops are enqueued in order on that stream
+ * (the reference executes requests strictly in order on one poller thread,
+ * src/dsp/commu.c:43, :91-114). A context is not thread-safe; several
+ * contexts may coexist.
+ *
+ * Return codes: 0 success, -1 rejected request (same meaning as the
+ * reference's ops: bad sizes, null/unknown buffers, misalignment), other
+ * negative values below.
+ */
+#ifndef HTPOPS_H
+#define HTPOPS_H
+
+#include "htpops_abi.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HTPOPS_OK            0
+#define HTPOPS_ERR_REJECTED  (-1) /* the reference's "return -1" */
+#define HTPOPS_ERR_NO_DEVICE (-2) /* compute requested from a context created without a GPU */
+#define HTPOPS_ERR_HIP       (-3) /* a HIP runtime call failed; see htpops_last_error() */
+#define HTPOPS_ERR_NOMEM     (-4)
+#define HTPOPS_ERR_BUSY      (-5) /* channel already active (AEE_EALREADY in the reference) */
+
+#define HTPOPS_DEVICE_NONE (-1)
+
+typedef struct htpops_context htpops_context;
+
+/* ---- session ----------------------------------------------------------- */
+
+/* Replaces open_dsp_session + htp_ops_init_backend (reference: src/host/session.c:14-96,
+ * src/dsp/commu.c:239-249). device >= 0 selects a GPU and creates the context's stream.
+ * device == HTPOPS_DEVICE_NONE creates a context that can register buffers and validate /
+ * frame requests but refuses every compute op with HTPOPS_ERR_NO_DEVICE. */
+int htpops_init_backend(htpops_context **out_ctx, int device);
+
+/* Replaces htp_ops_close (reference: src/dsp/commu.c:226-235): stops the channel, releases
+ * every buffer the context allocated, destroys the stream. */
+int htpops_close(htpops_context *ctx);
+
+/* Text of the most recent failure on this context (never NULL). */
+const char *htpops_last_error(const htpops_context *ctx);
+
+/* Blocks until everything enqueued on the context's stream has finished. */
+int htpops_synchronize(htpops_context *ctx);
+
+/* The context's hipStream_t, for callers that order their own HIP work against it. */
+void *htpops_get_stream(htpops_context *ctx);
+
+/* ---- buffer registry ---------------------------------------------------
+ * Replaces rpcmem_alloc + fastrpc_mmap on the host (reference: src/host/test.c:30-58) and the
+ * fd -> address table on the device (reference: src/dsp/mmap_mgr.cc:15-43). Handles are small
+ * positive integers that go into RpcmemBufAddr.fd. */
+
+/* Allocates `bytes` of device memory (256-byte aligned); returns a handle > 0 or a negative error. */
+int htpops_buffer_alloc(htpops_context *ctx, size_t bytes);
+
+/* Registers caller-owned device memory (e.g. a framework tensor); not freed on release. */
+int htpops_buffer_register(htpops_context *ctx, void *device_ptr, size_t bytes);
+
+/* mmap_manager_put_map: forgets the handle, frees the memory if the context allocated it.
+ * Unknown handles are ignored and return 0, as in the reference (mmap_mgr.cc:29-37). */
+int htpops_buffer_release(htpops_context *ctx, int handle);
+
+/* Device address and size of a handle (NULL / 0 if unknown). */
+void  *htpops_buffer_device_ptr(htpops_context *ctx, int handle);
+size_t htpops_buffer_size(htpops_context *ctx, int handle);
+
+/* Host <-> device copies ordered on the context's stream; both return after the copy is done. */
+int htpops_buffer_write(htpops_context *ctx, int handle, size_t offset, const void *src, size_t bytes);
+int htpops_buffer_read(htpops_context *ctx, int handle, size_t offset, void *dst, size_t bytes);
+
+/* ---- op execution ------------------------------------------------------ */
+
+/* Replaces execute_op_simple (reference: include/dsp/op_executor.h:9, src/dsp/op_executor.cc:52-204).
+ * Validates the request, resolves handles, enqueues the kernels on the context's stream and returns
+ * without waiting. Unknown op ids return -1 (the reference silently returns 0 there). */
+int htpops_execute_op(htpops_context *ctx, const struct OpComputeRequest *req);
+
+/* One pass of the reference's consumer loop over a message (src/dsp/commu.c:91-126): runs every
+ * request in order, stores each op's return code in RequestHeader.state, honours
+ * RPCMEM_MAP.n_puts as handle releases, waits for the stream, then publishes completion by
+ * storing state.d = v[0] | (1 << 8). Returns 0, or a negative error if the message is malformed
+ * (offsets outside `msg_bytes`; pass 0 to skip the bound check). The go byte v[0] is not
+ * required to be set. */
+int htpops_process_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes);
+
+/* Replaces htp_ops_create_channel / htp_ops_destroy_channel (reference: include/htp_ops.idl:11-12,
+ * src/dsp/commu.c:151-212): starts a consumer thread that polls msg->state exactly as
+ * msg_receiver_loop does (run when v[0] != 0 && v[1] == 0) and calls htpops_process_message.
+ * `msg` is ordinary host memory of `max_msg_size` bytes owned by the caller; it is zeroed here. */
+int htpops_create_channel(htpops_context *ctx, void *msg, size_t max_msg_size);
+int htpops_destroy_channel(htpops_context *ctx);
+
+/* Direct entries with the argument order of the FastRPC interface (reference: include/htp_ops.idl:15-17,
+ * include/host/op_export.h:3-5). Both enqueue and then wait, like an RPC. */
+int htpops_rms_norm_f32(htpops_context *ctx, int dst_fd, int dst_offset, int src_fd, int src_offset, int ne0,
+                        int ne1);
+int htpops_mat_mul_permuted_w16a32(htpops_context *ctx, int output_fd, int output_offset, int activation_fd,
+                                   int activation_offset, int weight_fd, int weight_offset, int m, int k, int n);
+
+/* ---- raw-pointer op entries ---------------------------------------------
+ * Same kernels as htpops_execute_op, for callers that hold device pointers. All pointers are
+ * device addresses; all calls enqueue on the context's stream and return without waiting.
+ * Each replaces the L1 function named beside it (reference: include/dsp/ops.h:15-26). */
+
+/* hvx_rms_norm_f32 (src/dsp/ops/rms_norm.c:68-84): weight may be NULL (all ones). The reference op
+ * is eps = 1e-5f, weight = NULL. Pointers must be 16-byte aligned. */
+int htpops_rms_norm_f32_ex_ptr(htpops_context *ctx, float *dst, const float *src, const float *weight, float eps,
+                               int ne0, int ne1);
+
+/* Activation quantizer (replaces transfer_activation_chunk_fp32_to_fp16, src/dsp/ops/mat_mul.c:89-128,
+ * with ggml's Q8_0 arithmetic): src fp32 [m][k] -> dst block_q8_0 [m][k/32]. k % 32 == 0. */
+int htpops_quantize_q8_0_ptr(htpops_context *ctx, void *dst, const float *src, int k, int m);
+
+/* RMSNorm fused with the quantizer: dst block_q8_0 [ne1][ne0/32]. Same result as the two ops in a row. */
+int htpops_rms_norm_quantize_q8_0_ptr(htpops_context *ctx, void *dst, const float *src, const float *weight,
+                                      float eps, int ne0, int ne1);
+
+/* hmx_mat_mul_permuted_qk_0_d16a32 (src/dsp/ops/mat_mul.c:875-1153) with integer block dots:
+ * dst fp32 [m][n]; act block_q8_0 [m][k/32]; weight block_q4_0 or block_q8_0 [n][k/32].
+ * weight_type is GGML_TYPE_Q4_0 (2) or GGML_TYPE_Q8_0 (8). k % 32 == 0. */
+int htpops_mat_mul_q8_0_act_ptr(htpops_context *ctx, float *dst, const void *act_q8_0, const void *weight, int m,
+                                int k, int n, int weight_type);
+
+/* Same with fp32 activations [m][k]; they are quantized into a workspace owned by the context. */
+int htpops_mat_mul_f32_act_ptr(htpops_context *ctx, float *dst, const float *act, const void *weight, int m, int k,
+                               int n, int weight_type);
+
+/* simple_flash_attn (src/dsp/ops/flash_attn.c:1368-1420). Q/O [qo_len][n_heads][head_dim] as fp32
+ * (qo_is_f32 = 1, the reference op) or fp16; K/V fp16 [kv_len][n_kv_heads][head_dim]; mask fp16
+ * [qo_len][align_up(kv_len, 64)] added to the scaled scores, or NULL; causal as in FlashAttnExParams. */
+int htpops_flash_attn_ptr(htpops_context *ctx, void *o, const void *q, const void *k, const void *v,
+                          const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
+                          int qo_is_f32, int causal);
+
+/* ---- measurement helpers (bench harness; no counterpart in the reference) ---- */
+
+/* Records an event on the context's stream / returns elapsed milliseconds between the two most
+ * recent start and stop marks after waiting for the stop mark. */
+int htpops_timer_start(htpops_context *ctx);
+int htpops_timer_stop(htpops_context *ctx);
+int htpops_timer_elapsed_ms(htpops_context *ctx, float *ms);
+
+/* Runs `iters` back-to-back v_mfma_i32_32x32x32_i8 (kind 0), v_mfma_i32_16x16x64_i8 (kind 1) or
+ * v_mfma_f32_32x32x16_f16 (kind 2) loops on every CU and reports the achieved op rate in Tera-ops/s. */
+int htpops_measure_mfma_peak(htpops_context *ctx, int kind, int iters, double *tera_ops);
+
+/* Plain device-to-device copy kernel (16 B per lane, grid-stride) used to calibrate HBM counters and to
+ * measure the attainable copy bandwidth; reports bytes read + written per second in GB/s. */
+int htpops_measure_copy_bandwidth(htpops_context *ctx, size_t bytes, int iters, double *gbps);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* HTPOPS_H */
