@@ -1,0 +1,569 @@
+// Decode-path matrix-vector product for gfx950: Q4_0 or Q8_0 weight rows times one Q8_0 activation row.
+//
+// Replaces hmx_mat_mul_permuted_qk_0_d16a32 at m = 1 (reference: src/dsp/ops/mat_mul.c:875-1153), which dequantizes
+// every weight to fp16 in on-chip memory and runs a 32-row matrix tile for one useful row. Here the op is what it
+// is on this machine: a stream over the weight bytes (18 or 34 bytes per 32 weights, each read once) with the
+// integer block dots done in registers.
+//
+// Unit of work: a PAIR of blocks (64 weights). A pair is 36 bytes (Q4_0) or 68 bytes (Q8_0), i.e. a whole number
+// of dwords, and every row starts on a pair boundary when k % 64 == 0, so lanes load pairs as dwords with no byte
+// realignment. Inside a pair the first block's quants sit two bytes off a dword boundary, behind its fp16 scale.
+// Instead of shifting weight bytes, the activation pair (which has the same skew in its own wire layout) is masked
+// once per wave so that its bytes line up with the weight dwords and carry zeros under the scale bytes; the
+// integer dot is order independent, so v_dot4_i32_i8 over the skewed dwords gives the exact block sums.
+// Q4_0 nibbles stay unsigned (0..15): sum (q - 8) a = sum q a - 8 sum a, and sum a is per activation block.
+//
+// Mapping: G lanes (16, 32 or 64) share a row and stride over its pairs; a wave works on 64 / G rows at once and
+// R such row sets, with every weight load issued before the first use (the whole matrix is a few tens of KB per
+// CU, so the kernel is latency bound and wants all bytes in flight). fp32 partial sums are reduced over the G lanes.
+#include "device_utils.h"
+#include "kernels.h"
+
+#include <stdlib.h>
+
+#include <type_traits>
+
+namespace htpops {
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves   = kThreads / kWave;
+
+template <int WT>
+struct Pair;
+template <>
+struct Pair<kQ4_0> {
+  static constexpr int kDwords = 9;
+};
+template <>
+struct Pair<kQ8_0> {
+  static constexpr int kDwords = 17;
+};
+constexpr int kActPairDwords = 17;
+
+// Activation pair prepared for dotting against raw weight dwords.
+template <int WT>
+struct ActPair;
+
+template <>
+struct ActPair<kQ4_0> {
+  uint32_t lo[9];  // bytes that meet the low nibbles of weight dword i
+  uint32_t hi[9];  // bytes that meet the high nibbles of weight dword i
+  float    d0, d1; // activation scales of the two blocks
+  int      off0, off1;  // 8 * (sum of the block's activation bytes)
+};
+
+template <>
+struct ActPair<kQ8_0> {
+  uint32_t a[17];
+  float    d0, d1;
+};
+
+template <int N>
+__device__ __forceinline__ void load_dwords(uint32_t (&dst)[N], const uint32_t *__restrict__ p) {
+  constexpr int n4 = N / 4;
+#pragma unroll
+  for (int i = 0; i < n4; ++i) {
+    const u32x4_a4 v = *reinterpret_cast<const u32x4_a4 *>(p + 4 * i);
+    dst[4 * i + 0]   = v.x;
+    dst[4 * i + 1]   = v.y;
+    dst[4 * i + 2]   = v.z;
+    dst[4 * i + 3]   = v.w;
+  }
+#pragma unroll
+  for (int i = 4 * n4; i < N; ++i) {
+    dst[i] = p[i];
+  }
+}
+
+template <int N>
+__device__ __forceinline__ void zero_dwords(uint32_t (&dst)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    dst[i] = 0u;
+  }
+}
+
+__device__ __forceinline__ void prepare(ActPair<kQ4_0> &ap, const uint32_t (&a)[17]) {
+  ap.lo[0] = a[0] & 0xffff0000u;  // elements 0,1 of block 0 (under weight bytes 2,3); scale bytes -> 0
+  ap.lo[1] = a[1];
+  ap.lo[2] = a[2];
+  ap.lo[3] = a[3];
+  ap.lo[4] = a[4] & 0x0000ffffu;  // elements 14,15; the next two weight bytes are block 1's scale
+  ap.hi[0] = a[4] & 0xffff0000u;  // elements 16,17
+  ap.hi[1] = a[5];
+  ap.hi[2] = a[6];
+  ap.hi[3] = a[7];
+  ap.hi[4] = a[8] & 0x0000ffffu;  // elements 30,31
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    ap.lo[5 + i] = a[9 + i];   // block 1, elements 0..15
+    ap.hi[5 + i] = a[13 + i];  // block 1, elements 16..31
+  }
+  ap.d0 = half_bits_to_float(a[0]);
+  ap.d1 = half_bits_to_float(a[8] >> 16);
+  int s0 = 0, s1 = 0;
+#pragma unroll
+  for (int i = 0; i < 5; ++i) {
+    s0 = dot4_i8(ap.lo[i], 0x01010101u, s0);
+    s0 = dot4_i8(ap.hi[i], 0x01010101u, s0);
+  }
+#pragma unroll
+  for (int i = 5; i < 9; ++i) {
+    s1 = dot4_i8(ap.lo[i], 0x01010101u, s1);
+    s1 = dot4_i8(ap.hi[i], 0x01010101u, s1);
+  }
+  ap.off0 = 8 * s0;
+  ap.off1 = 8 * s1;
+}
+
+__device__ __forceinline__ void prepare(ActPair<kQ8_0> &ap, const uint32_t (&a)[17]) {
+#pragma unroll
+  for (int i = 0; i < 17; ++i) {
+    ap.a[i] = a[i];
+  }
+  ap.d0 = half_bits_to_float(a[0]);
+  ap.d1 = half_bits_to_float(a[8] >> 16);
+}
+
+// fp32 contribution of one weight pair: ((float) sumi0 * d_w0) * d_a0 + ((float) sumi1 * d_w1) * d_a1
+__device__ __forceinline__ float pair_dot(const uint32_t (&w)[9], const ActPair<kQ4_0> &ap) {
+  int s0 = -ap.off0, s1 = -ap.off1;
+#pragma unroll
+  for (int i = 0; i < 5; ++i) {
+    s0 = dot4_i8(w[i] & 0x0f0f0f0fu, ap.lo[i], s0);
+    s0 = dot4_i8((w[i] >> 4) & 0x0f0f0f0fu, ap.hi[i], s0);
+  }
+#pragma unroll
+  for (int i = 5; i < 9; ++i) {
+    s1 = dot4_i8(w[i] & 0x0f0f0f0fu, ap.lo[i], s1);
+    s1 = dot4_i8((w[i] >> 4) & 0x0f0f0f0fu, ap.hi[i], s1);
+  }
+  const float dw0 = half_bits_to_float(w[0]);
+  const float dw1 = half_bits_to_float(w[4] >> 16);
+  float       t   = ((float) s0 * dw0) * ap.d0;
+  t += ((float) s1 * dw1) * ap.d1;
+  return t;
+}
+
+__device__ __forceinline__ float pair_dot(const uint32_t (&w)[17], const ActPair<kQ8_0> &ap) {
+  int s0 = 0, s1 = 0;
+  s0 = dot4_i8(w[0], ap.a[0] & 0xffff0000u, s0);
+#pragma unroll
+  for (int i = 1; i < 8; ++i) {
+    s0 = dot4_i8(w[i], ap.a[i], s0);
+  }
+  s0 = dot4_i8(w[8], ap.a[8] & 0x0000ffffu, s0);
+#pragma unroll
+  for (int i = 9; i < 17; ++i) {
+    s1 = dot4_i8(w[i], ap.a[i], s1);
+  }
+  const float dw0 = half_bits_to_float(w[0]);
+  const float dw1 = half_bits_to_float(w[8] >> 16);
+  float       t   = ((float) s0 * dw0) * ap.d0;
+  t += ((float) s1 * dw1) * ap.d1;
+  return t;
+}
+
+// ITERS > 0: every lane handles exactly ITERS pairs per row (pairs <= G * ITERS), all loads up front.
+template <int WT, int G, int ITERS, int R>
+__global__ __launch_bounds__(kThreads) void gemv_pairs_kernel(float *__restrict__ out,
+                                                              const uint32_t *__restrict__ act,
+                                                              const uint32_t *__restrict__ w, int n, int pairs) {
+  constexpr int PD    = Pair<WT>::kDwords;
+  constexpr int SLOTS = kWave / G;
+  const int     lane  = threadIdx.x & (kWave - 1);
+  const int     wave  = threadIdx.x / kWave;
+  const int     g     = lane % G;
+  const int     slot  = lane / G;
+  const int     row0  = (blockIdx.x * kWaves + wave) * (SLOTS * R);
+  if (row0 >= n) {
+    return;
+  }
+  const size_t row_dwords = (size_t) pairs * PD;
+
+  uint32_t wreg[R][ITERS][PD];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int row = row0 + r * SLOTS + slot;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int p = g + i * G;
+      if (row < n && p < pairs) {
+        load_dwords<PD>(wreg[r][i], w + (size_t) row * row_dwords + (size_t) p * PD);
+      } else {
+        zero_dwords<PD>(wreg[r][i]);  // zero scales: the pair contributes exactly 0
+      }
+    }
+  }
+
+  ActPair<WT> ap[ITERS];
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int p = g + i * G;
+    uint32_t  a[kActPairDwords];
+    if (p < pairs) {
+      load_dwords<kActPairDwords>(a, act + (size_t) p * kActPairDwords);
+    } else {
+      zero_dwords<kActPairDwords>(a);
+    }
+    prepare(ap[i], a);
+  }
+
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      acc += pair_dot(wreg[r][i], ap[i]);
+    }
+    acc           = group_sum<G>(acc);
+    const int row = row0 + r * SLOTS + slot;
+    if (g == 0 && row < n) {
+      out[row] = acc;
+    }
+  }
+}
+
+// Any number of pairs per row: lanes loop over the row, activations are re-read (L2) for every row set.
+template <int WT, int R>
+__global__ __launch_bounds__(kThreads) void gemv_pairs_loop_kernel(float *__restrict__ out,
+                                                                   const uint32_t *__restrict__ act,
+                                                                   const uint32_t *__restrict__ w, int n, int pairs) {
+  constexpr int PD   = Pair<WT>::kDwords;
+  const int     lane = threadIdx.x & (kWave - 1);
+  const int     wave = threadIdx.x / kWave;
+  const int     row0 = (blockIdx.x * kWaves + wave) * R;
+  if (row0 >= n) {
+    return;
+  }
+  const size_t row_dwords = (size_t) pairs * PD;
+  float        acc[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    acc[r] = 0.0f;
+  }
+  for (int p = lane; p < pairs; p += kWave) {
+    uint32_t wreg[R][PD];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      if (row0 + r < n) {
+        load_dwords<PD>(wreg[r], w + (size_t) (row0 + r) * row_dwords + (size_t) p * PD);
+      } else {
+        zero_dwords<PD>(wreg[r]);
+      }
+    }
+    uint32_t a[kActPairDwords];
+    load_dwords<kActPairDwords>(a, act + (size_t) p * kActPairDwords);
+    ActPair<WT> ap;
+    prepare(ap, a);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      acc[r] += pair_dot(wreg[r], ap);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const float s = group_sum<kWave>(acc[r]);
+    if (lane == 0 && row0 + r < n) {
+      out[row0 + r] = s;
+    }
+  }
+}
+
+// sum over the G consecutive lanes of a group; valid in the group's last lane
+template <int G>
+__device__ __forceinline__ float group_sum_dpp(float v) {
+#define HTPOPS_DPP_ADD(ctrl, row_mask) \
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, row_mask, 0xf, false))
+  HTPOPS_DPP_ADD(0xB1, 0xf);   // quad_perm [1,0,3,2]
+  HTPOPS_DPP_ADD(0x4E, 0xf);   // quad_perm [2,3,0,1]
+  HTPOPS_DPP_ADD(0x141, 0xf);  // row_half_mirror
+  HTPOPS_DPP_ADD(0x140, 0xf);  // row_mirror: every lane of a 16-lane row holds the row sum
+  if (G >= 32) {
+    HTPOPS_DPP_ADD(0x142, 0xa);  // row_bcast15 into rows 1 and 3
+  }
+  if (G >= 64) {
+    HTPOPS_DPP_ADD(0x143, 0xc);  // row_bcast31 into rows 2 and 3
+  }
+#undef HTPOPS_DPP_ADD
+  return v;
+}
+
+// ---- shared-activation variant --------------------------------------------------------------------------------
+// Same arithmetic and lane mapping as gemv_pairs_kernel, but the activation row is staged in LDS once per
+// workgroup instead of being fetched by every wave: the texture path then carries (almost) only weight bytes.
+// Weight loads are issued first, the cooperative activation copy second, so the weights are in flight while the
+// workgroup synchronises. Partial sums are reduced with DPP row operations instead of LDS permutes.
+template <int WT, int G, int ITERS, int R, int THREADS>
+__global__ __launch_bounds__(THREADS) void gemv_shared_act_kernel(float *__restrict__ out,
+                                                                  const uint32_t *__restrict__ act,
+                                                                  const uint32_t *__restrict__ w, int n, int pairs) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t act_lds[];
+  constexpr int PD    = Pair<WT>::kDwords;
+  constexpr int SLOTS = kWave / G;
+  constexpr int WAVES = THREADS / kWave;
+  const int     lane  = threadIdx.x & (kWave - 1);
+  const int     wave  = threadIdx.x / kWave;
+  const int     g     = lane % G;
+  const int     slot  = lane / G;
+  const int     row0  = (blockIdx.x * WAVES + wave) * (SLOTS * R);
+  const size_t  row_dwords = (size_t) pairs * PD;
+
+  // The activation row is requested FIRST and the weights right behind it: loads retire in order, so the (L2
+  // resident, quickly served) activations never wait behind the HBM stream, while the weights are already in
+  // flight during the workgroup's LDS exchange. A row is at most 192 pairs = 13056 bytes: ACT_SLOTS 16-byte
+  // pieces per thread cover it; pieces at or across the end of the row are slid back to end - 16.
+  constexpr int ACT_SLOTS = (192 * kActPairDwords * 4 + THREADS * 16 - 1) / (THREADS * 16);
+  const int     act_bytes = pairs * kActPairDwords * 4;
+  uint4         areg[ACT_SLOTS];
+  int           aoff[ACT_SLOTS];
+#pragma unroll
+  for (int j = 0; j < ACT_SLOTS; ++j) {
+    const int off = (threadIdx.x + j * THREADS) * 16;
+    aoff[j]       = min(off, act_bytes - 16);
+    const u32x4_a4 v = *reinterpret_cast<const u32x4_a4 *>(reinterpret_cast<const uint8_t *>(act) + aoff[j]);
+    areg[j]       = make_uint4(v.x, v.y, v.z, v.w);
+  }
+
+  // Branch-free weight loads (so that the compiler can count them and wait per use): lanes without work read a
+  // clamped, valid address and get their two scale fields zeroed afterwards, which makes the pair contribute 0.
+  uint32_t wreg[R][ITERS][PD];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int row = min(row0 + r * SLOTS + slot, n - 1);
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const int p = min(g + i * G, pairs - 1);
+      load_dwords<PD>(wreg[r][i], w + (size_t) row * row_dwords + (size_t) p * PD);
+    }
+  }
+
+  // every thread stores its pieces, without a branch: pieces clamped to the end of the row rewrite the same
+  // bytes with the same values, which is harmless and keeps the loads above where they were issued
+#pragma unroll
+  for (int j = 0; j < ACT_SLOTS; ++j) {
+    uint32_t *dst = act_lds + aoff[j] / 4;  // only dword aligned when the piece was slid back
+    dst[0] = areg[j].x, dst[1] = areg[j].y, dst[2] = areg[j].z, dst[3] = areg[j].w;
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the LDS writes have landed; vmcnt is left alone
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+
+  ActPair<WT> ap[ITERS];
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int p = g + i * G;
+    uint32_t  a[kActPairDwords];
+    if (p < pairs) {
+#pragma unroll
+      for (int e = 0; e < kActPairDwords; ++e) {
+        a[e] = act_lds[p * kActPairDwords + e];
+      }
+    } else {
+      zero_dwords<kActPairDwords>(a);
+    }
+    prepare(ap[i], a);
+  }
+
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int row = row0 + r * SLOTS + slot;
+    float     acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < ITERS; ++i) {
+      const bool live = row < n && g + i * G < pairs;
+      constexpr int kScale1 = WT == kQ4_0 ? 4 : 8;  // dword holding the second block's scale (upper half)
+      wreg[r][i][0]         = live ? wreg[r][i][0] : 0u;
+      wreg[r][i][kScale1]   = live ? wreg[r][i][kScale1] : 0u;
+      acc += pair_dot(wreg[r][i], ap[i]);
+    }
+    acc = group_sum_dpp<G>(acc);
+    if (g == G - 1 && row < n) {
+      out[row] = acc;
+    }
+  }
+}
+
+template <int WT, int G, int ITERS, int R, int THREADS>
+hipError_t launch_shared_act_instance(hipStream_t stream, float *out, const uint32_t *act, const uint32_t *w, int n,
+                                      int pairs) {
+  constexpr int rows_per_group = (THREADS / kWave) * (kWave / G) * R;
+  const dim3    grid((unsigned) ((n + rows_per_group - 1) / rows_per_group));
+  hipLaunchKernelGGL((gemv_shared_act_kernel<WT, G, ITERS, R, THREADS>), grid, dim3(THREADS),
+                     (size_t) pairs * kActPairDwords * 4, stream, out, act, w, n, pairs);
+  return hipGetLastError();
+}
+
+template <int WT, int G, int ITERS>
+hipError_t launch_shared_act(hipStream_t stream, float *out, const uint32_t *act, const uint32_t *w, int n, int pairs,
+                             int r, int threads) {
+#define HTPOPS_CASE(R, T)                                                                         \
+  if (r == R && threads == T) {                                                                   \
+    return launch_shared_act_instance<WT, G, ITERS, R, T>(stream, out, act, w, n, pairs);        \
+  }
+  HTPOPS_CASE(1, 256)
+  HTPOPS_CASE(2, 256)
+  HTPOPS_CASE(1, 512)
+  HTPOPS_CASE(2, 512)
+  HTPOPS_CASE(4, 256)
+  HTPOPS_CASE(1, 1024)
+#undef HTPOPS_CASE
+  return hipErrorInvalidValue;
+}
+
+// Catch-all (odd block counts, any m): one wave per weight row, 16-bit loads, scalar integer arithmetic.
+template <int WT>
+__global__ __launch_bounds__(kThreads) void gemv_blocks_generic_kernel(float *__restrict__ out,
+                                                                       const uint16_t *__restrict__ act,
+                                                                       const uint16_t *__restrict__ w, int m, int n,
+                                                                       int nblk) {
+  constexpr int WH   = WT == kQ4_0 ? 9 : 17;  // halfwords per weight block
+  const int     lane = threadIdx.x & (kWave - 1);
+  const int     row  = blockIdx.x * kWaves + threadIdx.x / kWave;
+  if (row >= n) {
+    return;
+  }
+  for (int mi = 0; mi < m; ++mi) {
+    float acc = 0.0f;
+    for (int b = lane; b < nblk; b += kWave) {
+      const uint16_t *wb   = w + ((size_t) row * nblk + b) * WH;
+      const uint16_t *ab   = act + ((size_t) mi * nblk + b) * 17;
+      int             sumi = 0;
+      if (WT == kQ4_0) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int wq = wb[1 + j], al = ab[1 + j], ah = ab[9 + j];
+          sumi += ((wq & 15) - 8) * (int) (int8_t) (al & 0xff) + (((wq >> 8) & 15) - 8) * (int) (int8_t) (al >> 8);
+          sumi += (((wq >> 4) & 15) - 8) * (int) (int8_t) (ah & 0xff) + (((wq >> 12) & 15) - 8) * (int) (int8_t) (ah >> 8);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int wq = wb[1 + j], aq = ab[1 + j];
+          sumi += (int) (int8_t) (wq & 0xff) * (int) (int8_t) (aq & 0xff) + (int) (int8_t) (wq >> 8) * (int) (int8_t) (aq >> 8);
+        }
+      }
+      acc += ((float) sumi * half_bits_to_float(wb[0])) * half_bits_to_float(ab[0]);
+    }
+    acc = group_sum<kWave>(acc);
+    if (lane == 0) {
+      out[(size_t) mi * n + row] = acc;
+    }
+  }
+}
+
+template <int WT, int G, int ITERS>
+hipError_t launch_pairs(hipStream_t stream, float *out, const uint32_t *act, const uint32_t *w, int n, int pairs,
+                        int rows_per_slot) {
+  constexpr int SLOTS = kWave / G;
+  auto          grid  = [&](int r) { return dim3((unsigned) ((n + kWaves * SLOTS * r - 1) / (kWaves * SLOTS * r))); };
+  switch (rows_per_slot) {
+    case 1:
+      hipLaunchKernelGGL((gemv_pairs_kernel<WT, G, ITERS, 1>), grid(1), dim3(kThreads), 0, stream, out, act, w, n, pairs);
+      break;
+    case 2:
+      hipLaunchKernelGGL((gemv_pairs_kernel<WT, G, ITERS, 2>), grid(2), dim3(kThreads), 0, stream, out, act, w, n, pairs);
+      break;
+    default:
+      hipLaunchKernelGGL((gemv_pairs_kernel<WT, G, ITERS, 4>), grid(4), dim3(kThreads), 0, stream, out, act, w, n, pairs);
+      break;
+  }
+  return hipGetLastError();
+}
+
+template <int WT>
+hipError_t launch_gemv_row(hipStream_t stream, float *out, const uint32_t *act, const uint32_t *w, int n, int pairs) {
+  static const int forced_r       = env_int("HTPOPS_GEMV_ROWS", 0);
+  static const int forced_threads = env_int("HTPOPS_GEMV_THREADS", 0);
+  static const int use_shared     = env_int("HTPOPS_GEMV_SHARED", 1);
+  constexpr int    PD             = Pair<WT>::kDwords;
+  if (use_shared && pairs <= 192) {
+    int r = 2, threads = 256;
+    if (pairs > 64) {
+      r = 1, threads = 512;
+    }
+    if (forced_r) {
+      r = forced_r;
+    }
+    if (forced_threads) {
+      threads = forced_threads;
+    }
+    if (pairs <= 16) {
+      return launch_shared_act<WT, 16, 1>(stream, out, act, w, n, pairs, r, threads);
+    }
+    if (pairs <= 32) {
+      return launch_shared_act<WT, 32, 1>(stream, out, act, w, n, pairs, r, threads);
+    }
+    if (pairs <= 64) {
+      return launch_shared_act<WT, 64, 1>(stream, out, act, w, n, pairs, r, threads);
+    }
+    if (pairs <= 128) {
+      return launch_shared_act<WT, 64, 2>(stream, out, act, w, n, pairs, r, threads);
+    }
+    return launch_shared_act<WT, 64, 3>(stream, out, act, w, n, pairs, r, threads);
+  }
+  // rows in flight per lane group: fewer for long rows (register budget), more for short ones
+  auto pick_r = [&](int regs_per_row, int slots) {
+    if (forced_r == 1 || forced_r == 2 || forced_r == 4) {
+      return forced_r;
+    }
+    int r = 4;
+    while (r > 1 && (regs_per_row * r > 72 || (long long) n / (slots * r) < 2048)) {
+      r >>= 1;
+    }
+    return r;
+  };
+  if (pairs <= 16) {
+    return launch_pairs<WT, 16, 1>(stream, out, act, w, n, pairs, pick_r(PD, 4));
+  }
+  if (pairs <= 32) {
+    return launch_pairs<WT, 32, 1>(stream, out, act, w, n, pairs, pick_r(PD, 2));
+  }
+  if (pairs <= 64) {
+    return launch_pairs<WT, 64, 1>(stream, out, act, w, n, pairs, pick_r(PD, 1));
+  }
+  if (pairs <= 128) {
+    return launch_pairs<WT, 64, 2>(stream, out, act, w, n, pairs, pick_r(2 * PD, 1));
+  }
+  if (pairs <= 192) {
+    return launch_pairs<WT, 64, 3>(stream, out, act, w, n, pairs, pick_r(3 * PD, 1));
+  }
+  hipLaunchKernelGGL((gemv_pairs_loop_kernel<WT, 2>), dim3((unsigned) ((n + kWaves * 2 - 1) / (kWaves * 2))),
+                     dim3(kThreads), 0, stream, out, act, w, n, pairs);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+// m rows of activations, one pass over the weights per activation row. The caller routes larger m to the MFMA path.
+hipError_t launch_gemv_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
+                                int n, WeightType wt) {
+  const int  nblk       = k / kQK;
+  const bool pair_path  = (nblk % 2 == 0) && ((reinterpret_cast<uintptr_t>(act) | reinterpret_cast<uintptr_t>(weight)) & 3) == 0;
+  if (!pair_path) {
+    dim3 grid((unsigned) ((n + kWaves - 1) / kWaves));
+    if (wt == kQ4_0) {
+      hipLaunchKernelGGL(gemv_blocks_generic_kernel<kQ4_0>, grid, dim3(kThreads), 0, stream, out,
+                         (const uint16_t *) act, (const uint16_t *) weight, m, n, nblk);
+    } else {
+      hipLaunchKernelGGL(gemv_blocks_generic_kernel<kQ8_0>, grid, dim3(kThreads), 0, stream, out,
+                         (const uint16_t *) act, (const uint16_t *) weight, m, n, nblk);
+    }
+    return hipGetLastError();
+  }
+  const int pairs = nblk / 2;
+  for (int mi = 0; mi < m; ++mi) {
+    const uint32_t *a = reinterpret_cast<const uint32_t *>(act) + (size_t) mi * pairs * kActPairDwords;
+    float          *o = out + (size_t) mi * n;
+    hipError_t      e = wt == kQ4_0 ? launch_gemv_row<kQ4_0>(stream, o, a, (const uint32_t *) weight, n, pairs) :
+                                      launch_gemv_row<kQ8_0>(stream, o, a, (const uint32_t *) weight, n, pairs);
+    if (e != hipSuccess) {
+      return e;
+    }
+  }
+  return hipSuccess;
+}
+
+}  // namespace htpops

@@ -1,0 +1,938 @@
+// C ABI of the MI355X op backend: context, buffer registry, request decoding, mailbox protocol.
+//
+// This file is the replacement for the reference's dispatch layer: execute_op_simple (src/dsp/op_executor.cc:52-204),
+// the fd -> address table (src/dsp/mmap_mgr.cc:15-43) and the consumer side of the shared-memory mailbox
+// (src/dsp/commu.c:37-136, :151-212). FastRPC, VTCM/HMX set-up and cache maintenance have no counterpart: a request
+// is validated on the host and its kernels are enqueued on the context's HIP stream.
+#include "htpops.h"
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <chrono>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "kernels.h"
+
+namespace {
+
+struct Buffer {
+  void  *ptr   = nullptr;
+  size_t size  = 0;
+  bool   owned = false;  // allocated by the context (freed on release)
+  bool   live  = false;
+};
+
+constexpr int kMaxHandles = 1 << 20;
+
+}  // namespace
+
+struct htpops_context {
+  int                 device     = HTPOPS_DEVICE_NONE;
+  bool                has_device = false;
+  hipStream_t         stream     = nullptr;
+  std::vector<Buffer> buffers;  // index = handle; slot 0 unused
+  std::vector<int>    free_slots;
+  std::string         last_error;
+
+  // scratch owned by the context: quantized activations of the fp32-activation matmul, attention partials
+  void  *workspace       = nullptr;
+  size_t workspace_bytes = 0;
+
+  hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+
+  // mailbox channel
+  std::thread           poller;
+  std::atomic<bool>     poller_stop{ false };
+  struct MessageHeader *chan_msg   = nullptr;
+  size_t                chan_bytes = 0;
+};
+
+namespace {
+
+int fail(htpops_context *ctx, int code, const char *fmt, ...) {
+  char    buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  if (ctx) {
+    ctx->last_error = buf;
+  }
+  if (getenv("HTPOPS_LOG")) {
+    fprintf(stderr, "[htpops] error %d: %s\n", code, buf);
+  }
+  return code;
+}
+
+int hip_fail(htpops_context *ctx, hipError_t e, const char *what) {
+  return fail(ctx, HTPOPS_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define HTPOPS_HIP(ctx, expr)                    \
+  do {                                           \
+    hipError_t e_ = (expr);                      \
+    if (e_ != hipSuccess) {                      \
+      return hip_fail((ctx), e_, #expr);         \
+    }                                            \
+  } while (0)
+
+Buffer *lookup(htpops_context *ctx, int handle) {
+  if (handle <= 0 || (size_t) handle >= ctx->buffers.size() || !ctx->buffers[handle].live) {
+    return nullptr;
+  }
+  return &ctx->buffers[handle];
+}
+
+int new_handle(htpops_context *ctx, void *ptr, size_t size, bool owned) {
+  int h;
+  if (!ctx->free_slots.empty()) {
+    h = ctx->free_slots.back();
+    ctx->free_slots.pop_back();
+  } else {
+    if (ctx->buffers.size() >= (size_t) kMaxHandles) {
+      return fail(ctx, HTPOPS_ERR_NOMEM, "handle table full");
+    }
+    if (ctx->buffers.empty()) {
+      ctx->buffers.emplace_back();  // slot 0: never a valid handle
+    }
+    h = (int) ctx->buffers.size();
+    ctx->buffers.emplace_back();
+  }
+  Buffer &b = ctx->buffers[h];
+  b.ptr     = ptr;
+  b.size    = size;
+  b.owned   = owned;
+  b.live    = true;
+  return h;
+}
+
+// Resolves (handle, offset) to an address with `need` readable/writable bytes, or null (the reference's
+// "mmap_manager_get_map returned NULL" case, op_executor.cc:57-61, extended with range checks).
+void *resolve(htpops_context *ctx, const struct RpcmemBufAddr &addr, size_t need) {
+  Buffer *b = lookup(ctx, addr.fd);
+  if (!b || addr.offset < 0) {
+    return nullptr;
+  }
+  const size_t off = (size_t) addr.offset;
+  if (off > b->size || need > b->size - off) {
+    return nullptr;
+  }
+  return static_cast<uint8_t *>(b->ptr) + off;
+}
+
+bool aligned(const void *p, size_t a) {
+  return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0;
+}
+
+// The 8-byte mailbox state is declared packed (alignment 1) but lives at the start of the message buffer, which
+// callers allocate at least 8-byte aligned; an unaligned buffer falls back to byte accesses between fences.
+uint64_t load_state(struct MessageHeader *msg) {
+  void *p = static_cast<void *>(msg);
+  if (aligned(p, 8)) {
+    return __atomic_load_n(static_cast<uint64_t *>(__builtin_assume_aligned(p, 8)), __ATOMIC_ACQUIRE);
+  }
+  uint64_t d;
+  memcpy(&d, p, 8);
+  __atomic_thread_fence(__ATOMIC_ACQUIRE);
+  return d;
+}
+
+void store_state(struct MessageHeader *msg, uint64_t d) {
+  void *p = static_cast<void *>(msg);
+  if (aligned(p, 8)) {
+    __atomic_store_n(static_cast<uint64_t *>(__builtin_assume_aligned(p, 8)), d, __ATOMIC_RELEASE);
+    return;
+  }
+  __atomic_thread_fence(__ATOMIC_RELEASE);
+  memcpy(p, &d, 8);
+}
+
+// size helpers with overflow checks; return false on overflow or non-positive dims
+bool mul3(size_t a, size_t b, size_t c, size_t *out) {
+  if (a == 0 || b == 0 || c == 0) {
+    *out = 0;
+    return true;
+  }
+  if (a > SIZE_MAX / b) {
+    return false;
+  }
+  size_t ab = a * b;
+  if (ab > SIZE_MAX / c) {
+    return false;
+  }
+  *out = ab * c;
+  return true;
+}
+
+int ensure_workspace(htpops_context *ctx, size_t bytes) {
+  if (bytes <= ctx->workspace_bytes) {
+    return HTPOPS_OK;
+  }
+  if (ctx->workspace) {
+    // kernels already enqueued may still use the old block
+    HTPOPS_HIP(ctx, hipStreamSynchronize(ctx->stream));
+    HTPOPS_HIP(ctx, hipFree(ctx->workspace));
+    ctx->workspace       = nullptr;
+    ctx->workspace_bytes = 0;
+  }
+  size_t rounded = (bytes + ((size_t) 1 << 20) - 1) & ~(((size_t) 1 << 20) - 1);
+  HTPOPS_HIP(ctx, hipMalloc(&ctx->workspace, rounded));
+  ctx->workspace_bytes = rounded;
+  return HTPOPS_OK;
+}
+
+size_t q8_0_bytes(size_t rows, size_t k) {
+  return rows * (k / 32) * 34;
+}
+
+size_t weight_bytes(size_t n, size_t k, int weight_type) {
+  return n * (k / 32) * (weight_type == htpops::kQ4_0 ? 18 : 34);
+}
+
+int need_device(htpops_context *ctx) {
+  if (!ctx->has_device) {
+    return fail(ctx, HTPOPS_ERR_NO_DEVICE, "context was created without a GPU; compute ops are unavailable");
+  }
+  return HTPOPS_OK;
+}
+
+// ---- op bodies on raw device pointers (validation that both the handle and the pointer entries share) ----
+
+int op_rms_norm(htpops_context *ctx, float *dst, const float *src, const float *weight, float eps, int ne0, int ne1) {
+  // reference: rms_norm.c:69-74 rejects null pointers, zero sizes and misaligned rows
+  if (!dst || !src || ne0 <= 0 || ne1 <= 0) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "rms_norm: null buffer or non-positive size (ne0=%d ne1=%d)", ne0, ne1);
+  }
+  if (!aligned(dst, 4) || !aligned(src, 4) || (weight && !aligned(weight, 4))) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "rms_norm: buffers must be 4-byte aligned");
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, htpops::launch_rms_norm_f32(ctx->stream, dst, src, weight, eps, ne0, ne1));
+  return HTPOPS_OK;
+}
+
+int op_quantize(htpops_context *ctx, void *dst, const float *src, int k, int m) {
+  if (!dst || !src || k <= 0 || m <= 0 || k % 32 != 0) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "quantize_q8_0: null buffer or bad size (k=%d m=%d, k %% 32 must be 0)", k, m);
+  }
+  if (!aligned(dst, 4) || !aligned(src, 16)) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "quantize_q8_0: src must be 16-byte and dst 4-byte aligned");
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, htpops::launch_quantize_q8_0(ctx->stream, dst, src, k, m));
+  return HTPOPS_OK;
+}
+
+int op_rms_norm_quantize(htpops_context *ctx, void *dst, const float *src, const float *weight, float eps, int ne0,
+                         int ne1) {
+  if (!dst || !src || ne0 <= 0 || ne1 <= 0 || ne0 % 32 != 0) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "rms_norm_quantize: null buffer or bad size (ne0=%d ne1=%d)", ne0, ne1);
+  }
+  if (!aligned(dst, 4) || !aligned(src, 16) || (weight && !aligned(weight, 16))) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "rms_norm_quantize: src/weight must be 16-byte and dst 4-byte aligned");
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  if (ne0 <= 16384) {
+    HTPOPS_HIP(ctx, htpops::launch_rms_norm_quantize_q8_0(ctx->stream, dst, src, weight, eps, ne0, ne1));
+    return HTPOPS_OK;
+  }
+  // very long rows: normalize into the workspace, then quantize
+  size_t bytes;
+  if (!mul3((size_t) ne0, (size_t) ne1, 4, &bytes)) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "rms_norm_quantize: size overflow");
+  }
+  if (int r = ensure_workspace(ctx, bytes)) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, htpops::launch_rms_norm_f32(ctx->stream, (float *) ctx->workspace, src, weight, eps, ne0, ne1));
+  HTPOPS_HIP(ctx, htpops::launch_quantize_q8_0(ctx->stream, dst, (const float *) ctx->workspace, ne0, ne1));
+  return HTPOPS_OK;
+}
+
+int check_mat_mul(htpops_context *ctx, const void *dst, const void *act, const void *weight, int m, int k, int n,
+                  int weight_type) {
+  // reference: mat_mul.c:878-892
+  if (!dst || !act || !weight || m <= 0 || k <= 0 || n <= 0) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "mat_mul: null buffer or non-positive size (m=%d k=%d n=%d)", m, k, n);
+  }
+  if (k % 32 != 0) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "mat_mul: k=%d is not a multiple of 32", k);
+  }
+  if (weight_type != htpops::kQ4_0 && weight_type != htpops::kQ8_0) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "mat_mul: unsupported weight type %d", weight_type);
+  }
+  if (!aligned(dst, 4) || !aligned(act, 2) || !aligned(weight, 2)) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "mat_mul: misaligned buffer");
+  }
+  return HTPOPS_OK;
+}
+
+int op_mat_mul_q8(htpops_context *ctx, float *dst, const void *act, const void *weight, int m, int k, int n,
+                  int weight_type) {
+  if (int r = check_mat_mul(ctx, dst, act, weight, m, k, n, weight_type)) {
+    return r;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, act, weight, m, k, n,
+                                                  (htpops::WeightType) weight_type));
+  return HTPOPS_OK;
+}
+
+int op_mat_mul_f32(htpops_context *ctx, float *dst, const float *act, const void *weight, int m, int k, int n,
+                   int weight_type) {
+  if (int r = check_mat_mul(ctx, dst, act, weight, m, k, n, weight_type)) {
+    return r;
+  }
+  if (!aligned(act, 16)) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "mat_mul: fp32 activations must be 16-byte aligned");
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  if (int r = ensure_workspace(ctx, q8_0_bytes((size_t) m, (size_t) k))) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, htpops::launch_quantize_q8_0(ctx->stream, ctx->workspace, act, k, m));
+  HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, ctx->workspace, weight, m, k, n,
+                                                  (htpops::WeightType) weight_type));
+  return HTPOPS_OK;
+}
+
+int op_flash_attn(htpops_context *ctx, void *o, const void *q, const void *k, const void *v, const void *mask,
+                  int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim, int qo_is_f32, int causal) {
+  if (!o || !q || !k || !v || qo_len <= 0 || kv_len <= 0 || n_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: null buffer or non-positive size");
+  }
+  // reference: flash_attn.c:1373-1376
+  if (n_heads % n_kv_heads != 0) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: n_heads=%d is not a multiple of n_kv_heads=%d", n_heads,
+                n_kv_heads);
+  }
+  if (head_dim != 64 && head_dim != 128) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: head_dim=%d (64 and 128 are built)", head_dim);
+  }
+  if (!aligned(o, 16) || !aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || (mask && !aligned(mask, 2))) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: q/k/v/o must be 16-byte aligned");
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  if (int r = ensure_workspace(ctx, htpops::flash_attn_workspace_bytes(qo_len, kv_len, n_heads, head_dim))) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, htpops::launch_flash_attn(ctx->stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads,
+                                            head_dim, qo_is_f32 != 0, causal != 0, ctx->workspace));
+  return HTPOPS_OK;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------------ session
+
+extern "C" int htpops_init_backend(htpops_context **out_ctx, int device) {
+  if (!out_ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  *out_ctx            = nullptr;
+  htpops_context *ctx = new (std::nothrow) htpops_context();
+  if (!ctx) {
+    return HTPOPS_ERR_NOMEM;
+  }
+  ctx->buffers.emplace_back();  // handle 0 is never valid
+  if (device != HTPOPS_DEVICE_NONE) {
+    int        count = 0;
+    hipError_t e     = hipGetDeviceCount(&count);
+    if (e != hipSuccess || device < 0 || device >= count) {
+      if (getenv("HTPOPS_LOG")) {
+        fprintf(stderr, "[htpops] init_backend: device %d unavailable (%s, %d devices)\n", device,
+                hipGetErrorString(e), count);
+      }
+      delete ctx;
+      return HTPOPS_ERR_NO_DEVICE;
+    }
+    if (hipSetDevice(device) != hipSuccess || hipStreamCreate(&ctx->stream) != hipSuccess ||
+        hipEventCreate(&ctx->ev_start) != hipSuccess || hipEventCreate(&ctx->ev_stop) != hipSuccess) {
+      delete ctx;
+      return HTPOPS_ERR_HIP;
+    }
+    ctx->device     = device;
+    ctx->has_device = true;
+  }
+  *out_ctx = ctx;
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_close(htpops_context *ctx) {
+  if (!ctx) {
+    return HTPOPS_OK;
+  }
+  htpops_destroy_channel(ctx);
+  if (ctx->has_device) {
+    (void) hipSetDevice(ctx->device);
+    (void) hipStreamSynchronize(ctx->stream);
+  }
+  for (size_t h = 1; h < ctx->buffers.size(); ++h) {
+    Buffer &b = ctx->buffers[h];
+    if (b.live && b.owned) {
+      if (ctx->has_device) {
+        (void) hipFree(b.ptr);
+      } else {
+        free(b.ptr);
+      }
+    }
+  }
+  if (ctx->has_device) {
+    if (ctx->workspace) {
+      (void) hipFree(ctx->workspace);
+    }
+    (void) hipEventDestroy(ctx->ev_start);
+    (void) hipEventDestroy(ctx->ev_stop);
+    (void) hipStreamDestroy(ctx->stream);
+  }
+  delete ctx;
+  return HTPOPS_OK;
+}
+
+extern "C" const char *htpops_last_error(const htpops_context *ctx) {
+  return ctx ? ctx->last_error.c_str() : "null context";
+}
+
+extern "C" int htpops_synchronize(htpops_context *ctx) {
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (!ctx->has_device) {
+    return HTPOPS_OK;
+  }
+  HTPOPS_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  return HTPOPS_OK;
+}
+
+extern "C" void *htpops_get_stream(htpops_context *ctx) {
+  return ctx ? (void *) ctx->stream : nullptr;
+}
+
+// ------------------------------------------------------------------------------------------------ buffers
+
+extern "C" int htpops_buffer_alloc(htpops_context *ctx, size_t bytes) {
+  if (!ctx || bytes == 0) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "buffer_alloc: zero size");
+  }
+  void *p = nullptr;
+  if (ctx->has_device) {
+    HTPOPS_HIP(ctx, hipMalloc(&p, bytes));
+  } else {
+    p = aligned_alloc(256, (bytes + 255) & ~(size_t) 255);
+    if (!p) {
+      return fail(ctx, HTPOPS_ERR_NOMEM, "buffer_alloc: out of host memory");
+    }
+  }
+  int h = new_handle(ctx, p, bytes, true);
+  if (h < 0) {
+    if (ctx->has_device) {
+      (void) hipFree(p);
+    } else {
+      free(p);
+    }
+  }
+  return h;
+}
+
+extern "C" int htpops_buffer_register(htpops_context *ctx, void *device_ptr, size_t bytes) {
+  if (!ctx || !device_ptr || bytes == 0) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "buffer_register: null pointer or zero size");
+  }
+  return new_handle(ctx, device_ptr, bytes, false);
+}
+
+extern "C" int htpops_buffer_release(htpops_context *ctx, int handle) {
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  Buffer *b = lookup(ctx, handle);
+  if (!b) {
+    return HTPOPS_OK;  // unknown handles are ignored (reference: mmap_mgr.cc:29-37)
+  }
+  int ret = HTPOPS_OK;
+  if (b->owned) {
+    if (ctx->has_device) {
+      hipError_t e = hipFree(b->ptr);  // waits for work that may still use the block
+      if (e != hipSuccess) {
+        ret = hip_fail(ctx, e, "hipFree");
+      }
+    } else {
+      free(b->ptr);
+    }
+  }
+  *b = Buffer();
+  ctx->free_slots.push_back(handle);
+  return ret;
+}
+
+extern "C" void *htpops_buffer_device_ptr(htpops_context *ctx, int handle) {
+  Buffer *b = ctx ? lookup(ctx, handle) : nullptr;
+  return b ? b->ptr : nullptr;
+}
+
+extern "C" size_t htpops_buffer_size(htpops_context *ctx, int handle) {
+  Buffer *b = ctx ? lookup(ctx, handle) : nullptr;
+  return b ? b->size : 0;
+}
+
+extern "C" int htpops_buffer_write(htpops_context *ctx, int handle, size_t offset, const void *src, size_t bytes) {
+  Buffer *b = ctx ? lookup(ctx, handle) : nullptr;
+  if (!b || !src || offset > b->size || bytes > b->size - offset) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "buffer_write: unknown handle or range outside the buffer");
+  }
+  uint8_t *dst = static_cast<uint8_t *>(b->ptr) + offset;
+  if (!ctx->has_device) {
+    memcpy(dst, src, bytes);
+    return HTPOPS_OK;
+  }
+  HTPOPS_HIP(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+  HTPOPS_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_buffer_read(htpops_context *ctx, int handle, size_t offset, void *dst, size_t bytes) {
+  Buffer *b = ctx ? lookup(ctx, handle) : nullptr;
+  if (!b || !dst || offset > b->size || bytes > b->size - offset) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "buffer_read: unknown handle or range outside the buffer");
+  }
+  const uint8_t *src = static_cast<const uint8_t *>(b->ptr) + offset;
+  if (!ctx->has_device) {
+    memcpy(dst, src, bytes);
+    return HTPOPS_OK;
+  }
+  HTPOPS_HIP(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+  HTPOPS_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  return HTPOPS_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ ops
+
+extern "C" int htpops_execute_op(htpops_context *ctx, const struct OpComputeRequest *req) {
+  if (!ctx || !req) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  switch (req->op) {
+    case HTP_OPS_RMS_NORM_F32:
+      {
+        // reference: op_executor.cc:82-94
+        const auto *p = reinterpret_cast<const RmsNormF32Params *>(req->payload);
+        size_t      bytes;
+        if (p->ne0 <= 0 || p->ne1 <= 0 || !mul3((size_t) p->ne0, (size_t) p->ne1, 4, &bytes)) {
+          return fail(ctx, HTPOPS_ERR_REJECTED, "rms_norm: bad size (ne0=%d ne1=%d)", p->ne0, p->ne1);
+        }
+        return op_rms_norm(ctx, (float *) resolve(ctx, p->dst, bytes), (const float *) resolve(ctx, p->src, bytes),
+                           nullptr, 1e-5f, p->ne0, p->ne1);
+      }
+    case HTP_OPS_RMS_NORM_F32_EX:
+    case HTP_OPS_RMS_NORM_QUANTIZE_Q8_0:
+      {
+        const auto *p = reinterpret_cast<const RmsNormExParams *>(req->payload);
+        size_t      bytes;
+        if (p->ne0 <= 0 || p->ne1 <= 0 || !mul3((size_t) p->ne0, (size_t) p->ne1, 4, &bytes)) {
+          return fail(ctx, HTPOPS_ERR_REJECTED, "rms_norm: bad size (ne0=%d ne1=%d)", p->ne0, p->ne1);
+        }
+        const float *w = nullptr;
+        if (p->weight.fd >= 0) {
+          w = (const float *) resolve(ctx, p->weight, (size_t) p->ne0 * 4);
+          if (!w) {
+            return fail(ctx, HTPOPS_ERR_REJECTED, "rms_norm: unknown weight buffer");
+          }
+        }
+        const float *src = (const float *) resolve(ctx, p->src, bytes);
+        if (req->op == HTP_OPS_RMS_NORM_F32_EX) {
+          return op_rms_norm(ctx, (float *) resolve(ctx, p->dst, bytes), src, w, p->eps, p->ne0, p->ne1);
+        }
+        if (p->ne0 % 32 != 0) {
+          return fail(ctx, HTPOPS_ERR_REJECTED, "rms_norm_quantize: ne0=%d is not a multiple of 32", p->ne0);
+        }
+        return op_rms_norm_quantize(ctx, resolve(ctx, p->dst, q8_0_bytes((size_t) p->ne1, (size_t) p->ne0)), src, w,
+                                    p->eps, p->ne0, p->ne1);
+      }
+    case HTP_OPS_QUANTIZE_Q8_0:
+      {
+        const auto *p = reinterpret_cast<const RmsNormF32Params *>(req->payload);
+        size_t      bytes;
+        if (p->ne0 <= 0 || p->ne1 <= 0 || p->ne0 % 32 != 0 || !mul3((size_t) p->ne0, (size_t) p->ne1, 4, &bytes)) {
+          return fail(ctx, HTPOPS_ERR_REJECTED, "quantize_q8_0: bad size (ne0=%d ne1=%d)", p->ne0, p->ne1);
+        }
+        return op_quantize(ctx, resolve(ctx, p->dst, q8_0_bytes((size_t) p->ne1, (size_t) p->ne0)),
+                           (const float *) resolve(ctx, p->src, bytes), p->ne0, p->ne1);
+      }
+    case HTP_OPS_MAT_MUL_Q4_0_Q8_0:
+    case HTP_OPS_MAT_MUL_Q8_0_Q8_0:
+    case HTP_OPS_MAT_MUL_Q4_0_A32:
+    case HTP_OPS_MAT_MUL_Q8_0_A32:
+      {
+        // reference: op_executor.cc:114-149 (sizes), with ggml row-layout weights
+        const auto *p  = reinterpret_cast<const MatMulParams *>(req->payload);
+        const int   wt = (req->op == HTP_OPS_MAT_MUL_Q4_0_Q8_0 || req->op == HTP_OPS_MAT_MUL_Q4_0_A32) ? htpops::kQ4_0 :
+                                                                                                         htpops::kQ8_0;
+        const bool  f32_act = req->op == HTP_OPS_MAT_MUL_Q4_0_A32 || req->op == HTP_OPS_MAT_MUL_Q8_0_A32;
+        size_t      out_bytes, act_bytes;
+        if (p->m <= 0 || p->k <= 0 || p->n <= 0 || p->k % 32 != 0 ||
+            !mul3((size_t) p->m, (size_t) p->n, 4, &out_bytes) || !mul3((size_t) p->m, (size_t) p->k, 4, &act_bytes)) {
+          return fail(ctx, HTPOPS_ERR_REJECTED, "mat_mul: bad size (m=%d k=%d n=%d)", p->m, p->k, p->n);
+        }
+        float      *out = (float *) resolve(ctx, p->output, out_bytes);
+        const void *w   = resolve(ctx, p->weight, weight_bytes((size_t) p->n, (size_t) p->k, wt));
+        if (f32_act) {
+          return op_mat_mul_f32(ctx, out, (const float *) resolve(ctx, p->activation, act_bytes), w, p->m, p->k, p->n,
+                                wt);
+        }
+        return op_mat_mul_q8(ctx, out, resolve(ctx, p->activation, q8_0_bytes((size_t) p->m, (size_t) p->k)), w, p->m,
+                             p->k, p->n, wt);
+      }
+    case HTP_OPS_FLASH_ATTN_QO_F32_KV_F16:
+    case HTP_OPS_FLASH_ATTN_F16:
+      {
+        // reference: op_executor.cc:151-196
+        const bool  ext    = req->op == HTP_OPS_FLASH_ATTN_F16;
+        const auto *p      = reinterpret_cast<const FlashAttnParams *>(req->payload);
+        const int   causal = ext ? reinterpret_cast<const FlashAttnExParams *>(req->payload)->causal : 0;
+        if (p->qo_len <= 0 || p->kv_len <= 0 || p->n_heads <= 0 || p->n_kv_heads <= 0 || p->head_dim <= 0) {
+          return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: non-positive size");
+        }
+        size_t qo_elems, kv_elems, qo_bytes, kv_bytes, mask_bytes;
+        if (!mul3((size_t) p->qo_len, (size_t) p->n_heads, (size_t) p->head_dim, &qo_elems) ||
+            !mul3((size_t) p->kv_len, (size_t) p->n_kv_heads, (size_t) p->head_dim, &kv_elems) ||
+            !mul3(qo_elems, ext ? 2 : 4, 1, &qo_bytes) || !mul3(kv_elems, 2, 1, &kv_bytes) ||
+            !mul3((size_t) p->qo_len, ((size_t) p->kv_len + 63) / 64 * 64, 2, &mask_bytes)) {
+          return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: size overflow");
+        }
+        const void *mask = nullptr;
+        if (p->mask.fd >= 0 && lookup(ctx, p->mask.fd)) {
+          // the kernel strides the mask by align_up(kv_len, 64) (reference: flash_attn.c:152)
+          mask = resolve(ctx, p->mask, mask_bytes);
+          if (!mask) {
+            return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: mask buffer smaller than qo_len * align_up(kv_len, 64) * 2");
+          }
+        }
+        return op_flash_attn(ctx, resolve(ctx, p->o, qo_bytes), resolve(ctx, p->q, qo_bytes),
+                             resolve(ctx, p->k, kv_bytes), resolve(ctx, p->v, kv_bytes), mask, p->qo_len, p->kv_len,
+                             p->n_heads, p->n_kv_heads, p->head_dim, ext ? 0 : 1, causal);
+      }
+    case HTP_OPS_MAT_MUL_PERMUTED_W16A32:
+    case HTP_OPS_MAT_MUL_PERMUTED_W4D16A32:
+    case HTP_OPS_MAT_MUL_PERMUTED_W8D16A32:
+    case HTP_OPS_MAT_MUL_PERMUTED_W4D16A32_IQ4_NL:
+      return fail(ctx, HTPOPS_ERR_REJECTED, "op %u: tile-permuted weight formats are not built; use the row-layout ops",
+                  req->op);
+    default:
+      // the reference returns 0 without touching anything (op_executor.cc:200-203); a silent success on an
+      // unknown op hides host bugs, so this backend reports it
+      return fail(ctx, HTPOPS_ERR_REJECTED, "unknown op %u", req->op);
+  }
+}
+
+extern "C" int htpops_process_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes) {
+  if (!ctx || !msg) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  const int n_reqs = msg->n_reqs;
+  if (n_reqs < 0 || n_reqs > (1 << 20)) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "message: n_reqs=%d", n_reqs);
+  }
+  if (msg_bytes) {
+    const size_t hdr = sizeof(struct MessageHeader) + ((size_t) n_reqs + 1) * sizeof(int32_t);
+    if (hdr > msg_bytes) {
+      return fail(ctx, HTPOPS_ERR_REJECTED, "message: header of %zu bytes does not fit %zu", hdr, msg_bytes);
+    }
+    int32_t prev = (int32_t) hdr;
+    for (int i = 0; i <= n_reqs; ++i) {
+      const int32_t off = msg->req_offsets[i];
+      if (off < prev || (size_t) off > msg_bytes || (i < n_reqs && (size_t) off + sizeof(struct RequestHeader) > msg_bytes)) {
+        return fail(ctx, HTPOPS_ERR_REJECTED, "message: request offset %d (entry %d) outside the message", off, i);
+      }
+      prev = off;
+    }
+  }
+  const uint8_t v0 = msg->state.v[0];
+
+  for (int i = 0; i < n_reqs; ++i) {
+    struct RequestHeader *hdr  = message_header_get_request_ptr(msg, i);
+    const size_t          size = message_header_get_request_size(msg, i);
+    switch (hdr->type) {
+      case REQUEST_TYPE_OP_COMPUTE:
+        if (size < sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest)) {
+          hdr->state = HTPOPS_ERR_REJECTED;
+        } else {
+          hdr->state = htpops_execute_op(ctx, reinterpret_cast<const struct OpComputeRequest *>(hdr->data));
+        }
+        break;
+      case REQUEST_TYPE_RPCMEM_MAP:
+        {
+          // reference: commu.c:102-110 -- only the puts are acted on
+          const auto *map = reinterpret_cast<const struct RpcmemMapRequest *>(hdr->data);
+          int         ret = 0;
+          if (size < sizeof(struct RequestHeader) + sizeof(struct RpcmemMapRequest) || map->n_puts < 0 ||
+              size < sizeof(struct RequestHeader) + sizeof(struct RpcmemMapRequest) + (size_t) map->n_puts * 4) {
+            ret = HTPOPS_ERR_REJECTED;
+          } else {
+            for (int j = 0; j < map->n_puts; ++j) {
+              htpops_buffer_release(ctx, map->fds[j]);
+            }
+          }
+          hdr->state = ret;
+        }
+        break;
+      default:
+        break;  // NO_OP and unknown types are skipped, state untouched (commu.c:111-113)
+    }
+  }
+
+  int ret = htpops_synchronize(ctx);
+  if (ret != HTPOPS_OK) {
+    for (int i = 0; i < n_reqs; ++i) {
+      struct RequestHeader *hdr = message_header_get_request_ptr(msg, i);
+      if (hdr->type == REQUEST_TYPE_OP_COMPUTE && hdr->state == 0) {
+        hdr->state = ret;
+      }
+    }
+  }
+  // publish completion: state.d = v0 | 1 << 8 with release ordering (reference: commu.c:125-126)
+  store_state(msg, (uint64_t) v0 | ((uint64_t) 1 << 8));
+  return HTPOPS_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ channel
+
+namespace {
+
+void poll_loop(htpops_context *ctx) {
+  if (ctx->has_device) {
+    (void) hipSetDevice(ctx->device);
+  }
+  while (!ctx->poller_stop.load(std::memory_order_acquire)) {
+    const uint64_t d  = load_state(ctx->chan_msg);
+    const uint8_t  v0 = d & 0xff, v1 = (d >> 8) & 0xff;
+    if (v0 == 0 || v1 != 0) {  // reference: commu.c:70-75
+      std::this_thread::sleep_for(std::chrono::microseconds(1));
+      continue;
+    }
+    if (htpops_process_message(ctx, ctx->chan_msg, ctx->chan_bytes) != HTPOPS_OK) {
+      // malformed message: still complete the handshake so the producer does not spin forever
+      store_state(ctx->chan_msg, (uint64_t) v0 | ((uint64_t) 1 << 8));
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" int htpops_create_channel(htpops_context *ctx, void *msg, size_t max_msg_size) {
+  if (!ctx || !msg || max_msg_size < sizeof(struct MessageHeader) + sizeof(int32_t)) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "create_channel: null or too small message buffer");
+  }
+  if (ctx->chan_msg) {
+    return fail(ctx, HTPOPS_ERR_BUSY, "create_channel: a channel is already active");
+  }
+  memset(msg, 0, max_msg_size);  // reference: commu.c:160-161
+  ctx->chan_msg   = static_cast<struct MessageHeader *>(msg);
+  ctx->chan_bytes = max_msg_size;
+  ctx->poller_stop.store(false);
+  ctx->poller = std::thread(poll_loop, ctx);
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_destroy_channel(htpops_context *ctx) {
+  if (!ctx || !ctx->chan_msg) {
+    return HTPOPS_OK;
+  }
+  ctx->poller_stop.store(true, std::memory_order_release);
+  if (ctx->poller.joinable()) {
+    ctx->poller.join();
+  }
+  ctx->chan_msg   = nullptr;
+  ctx->chan_bytes = 0;
+  return HTPOPS_OK;
+}
+
+// ------------------------------------------------------------------------------------------------ direct entries
+
+extern "C" int htpops_rms_norm_f32(htpops_context *ctx, int dst_fd, int dst_offset, int src_fd, int src_offset,
+                                   int ne0, int ne1) {
+  struct {
+    struct OpComputeRequest req;
+    struct RmsNormF32Params params;
+  } HTPOPS_PACKED r;
+  r.req.op     = HTP_OPS_RMS_NORM_F32;
+  r.params.dst = { dst_fd, dst_offset };
+  r.params.src = { src_fd, src_offset };
+  r.params.ne0 = ne0;
+  r.params.ne1 = ne1;
+  int ret      = htpops_execute_op(ctx, &r.req);
+  if (ret != HTPOPS_OK) {
+    return ret;
+  }
+  return htpops_synchronize(ctx);
+}
+
+extern "C" int htpops_mat_mul_permuted_w16a32(htpops_context *ctx, int output_fd, int output_offset,
+                                              int activation_fd, int activation_offset, int weight_fd,
+                                              int weight_offset, int m, int k, int n) {
+  struct {
+    struct OpComputeRequest req;
+    struct MatMulParams     params;
+  } HTPOPS_PACKED r;
+  r.req.op            = HTP_OPS_MAT_MUL_PERMUTED_W16A32;
+  r.params.output     = { output_fd, output_offset };
+  r.params.activation = { activation_fd, activation_offset };
+  r.params.weight     = { weight_fd, weight_offset };
+  r.params.m          = m;
+  r.params.k          = k;
+  r.params.n          = n;
+  int ret             = htpops_execute_op(ctx, &r.req);
+  if (ret != HTPOPS_OK) {
+    return ret;
+  }
+  return htpops_synchronize(ctx);
+}
+
+// ------------------------------------------------------------------------------------------------ pointer entries
+
+extern "C" int htpops_rms_norm_f32_ex_ptr(htpops_context *ctx, float *dst, const float *src, const float *weight,
+                                          float eps, int ne0, int ne1) {
+  return ctx ? op_rms_norm(ctx, dst, src, weight, eps, ne0, ne1) : HTPOPS_ERR_REJECTED;
+}
+
+extern "C" int htpops_quantize_q8_0_ptr(htpops_context *ctx, void *dst, const float *src, int k, int m) {
+  return ctx ? op_quantize(ctx, dst, src, k, m) : HTPOPS_ERR_REJECTED;
+}
+
+extern "C" int htpops_rms_norm_quantize_q8_0_ptr(htpops_context *ctx, void *dst, const float *src,
+                                                 const float *weight, float eps, int ne0, int ne1) {
+  return ctx ? op_rms_norm_quantize(ctx, dst, src, weight, eps, ne0, ne1) : HTPOPS_ERR_REJECTED;
+}
+
+extern "C" int htpops_mat_mul_q8_0_act_ptr(htpops_context *ctx, float *dst, const void *act_q8_0, const void *weight,
+                                           int m, int k, int n, int weight_type) {
+  return ctx ? op_mat_mul_q8(ctx, dst, act_q8_0, weight, m, k, n, weight_type) : HTPOPS_ERR_REJECTED;
+}
+
+extern "C" int htpops_mat_mul_f32_act_ptr(htpops_context *ctx, float *dst, const float *act, const void *weight, int m,
+                                          int k, int n, int weight_type) {
+  return ctx ? op_mat_mul_f32(ctx, dst, act, weight, m, k, n, weight_type) : HTPOPS_ERR_REJECTED;
+}
+
+extern "C" int htpops_flash_attn_ptr(htpops_context *ctx, void *o, const void *q, const void *k, const void *v,
+                                     const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads,
+                                     int head_dim, int qo_is_f32, int causal) {
+  return ctx ? op_flash_attn(ctx, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, head_dim, qo_is_f32, causal) :
+               HTPOPS_ERR_REJECTED;
+}
+
+// ------------------------------------------------------------------------------------------------ measurement
+
+extern "C" int htpops_timer_start(htpops_context *ctx) {
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_timer_stop(htpops_context *ctx) {
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_timer_elapsed_ms(htpops_context *ctx, float *ms) {
+  if (!ctx || !ms) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, hipEventSynchronize(ctx->ev_stop));
+  HTPOPS_HIP(ctx, hipEventElapsedTime(ms, ctx->ev_start, ctx->ev_stop));
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_measure_mfma_peak(htpops_context *ctx, int kind, int iters, double *tera_ops) {
+  if (!ctx || !tera_ops || iters <= 0 || kind < 0 || kind > 2) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  hipDeviceProp_t prop;
+  HTPOPS_HIP(ctx, hipGetDeviceProperties(&prop, ctx->device));
+  const int n_blocks = prop.multiProcessorCount * 2;  // 4 waves per block -> 2 waves per SIMD
+  int      *sink     = nullptr;
+  HTPOPS_HIP(ctx, hipMalloc((void **) &sink, sizeof(int)));
+  hipError_t e = htpops::launch_mfma_loop(ctx->stream, kind, 16, sink, n_blocks);  // warm-up
+  float      ms = 0.f;
+  if (e == hipSuccess) e = hipEventRecord(ctx->ev_start, ctx->stream);
+  if (e == hipSuccess) e = htpops::launch_mfma_loop(ctx->stream, kind, iters, sink, n_blocks);
+  if (e == hipSuccess) e = hipEventRecord(ctx->ev_stop, ctx->stream);
+  if (e == hipSuccess) e = hipEventSynchronize(ctx->ev_stop);
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop);
+  (void) hipFree(sink);
+  if (e != hipSuccess) {
+    return hip_fail(ctx, e, "mfma loop");
+  }
+  const double ops_per_mfma = kind == 0 ? 2.0 * 32 * 32 * 32 : (kind == 1 ? 2.0 * 16 * 16 * 64 : 2.0 * 32 * 32 * 16);
+  const double total        = (double) n_blocks * 4 /*waves*/ * (double) iters * 4 /*chains*/ * ops_per_mfma;
+  *tera_ops                 = total / ((double) ms * 1e-3) / 1e12;
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_measure_copy_bandwidth(htpops_context *ctx, size_t bytes, int iters, double *gbps) {
+  if (!ctx || !gbps || iters <= 0 || bytes < 16) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  void *a = nullptr, *b = nullptr;
+  HTPOPS_HIP(ctx, hipMalloc(&a, bytes));
+  hipError_t e = hipMalloc(&b, bytes);
+  if (e != hipSuccess) {
+    (void) hipFree(a);
+    return hip_fail(ctx, e, "hipMalloc");
+  }
+  float ms = 0.f;
+  e        = hipMemsetAsync(a, 1, bytes, ctx->stream);
+  if (e == hipSuccess) e = htpops::launch_copy(ctx->stream, b, a, bytes);
+  if (e == hipSuccess) e = hipEventRecord(ctx->ev_start, ctx->stream);
+  for (int i = 0; i < iters && e == hipSuccess; ++i) {
+    e = htpops::launch_copy(ctx->stream, b, a, bytes);
+  }
+  if (e == hipSuccess) e = hipEventRecord(ctx->ev_stop, ctx->stream);
+  if (e == hipSuccess) e = hipEventSynchronize(ctx->ev_stop);
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop);
+  (void) hipFree(a);
+  (void) hipFree(b);
+  if (e != hipSuccess) {
+    return hip_fail(ctx, e, "copy loop");
+  }
+  *gbps = 2.0 * (double) (bytes / 16 * 16) * iters / ((double) ms * 1e-3) / 1e9;
+  return HTPOPS_OK;
+}

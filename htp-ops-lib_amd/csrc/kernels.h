@@ -1,0 +1,48 @@
+// Host-callable launchers of the gfx950 kernels. Every launcher validates nothing (the C-ABI layer does),
+// enqueues on `stream`, and returns the status of the launch.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace htpops {
+
+enum WeightType { kQ4_0 = 2, kQ8_0 = 8 };  // enum ggml_type values (reference: include/dsp/quants.h:33-74)
+
+// fp32 [m][k] -> block_q8_0 [m][k/32]
+hipError_t launch_quantize_q8_0(hipStream_t stream, void *dst, const float *src, int k, int m);
+
+// y = x * rsqrt(mean(x^2) + eps) * w; w may be null
+hipError_t launch_rms_norm_f32(hipStream_t stream, float *dst, const float *src, const float *weight, float eps,
+                               int ne0, int ne1);
+// same, result quantized to block_q8_0 [ne1][ne0/32]; ne0 % 32 == 0
+hipError_t launch_rms_norm_quantize_q8_0(hipStream_t stream, void *dst, const float *src, const float *weight,
+                                         float eps, int ne0, int ne1);
+
+// out fp32 [m][n] = act block_q8_0 [m][k/32] x weight [n][k/32]
+// decode path: one pass over the weight bytes per activation row
+hipError_t launch_gemv_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
+                                int n, WeightType wt);
+// prefill path: int8 MFMA over LDS-staged tiles; needs k % 32 == 0
+hipError_t launch_gemm_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
+                                int n, WeightType wt);
+// picks between the two by m
+hipError_t launch_mat_mul_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
+                                   int n, WeightType wt);
+
+// attention; see htpops_flash_attn_ptr. `workspace` holds split-KV partials (decode), size from
+// flash_attn_workspace_bytes.
+size_t     flash_attn_workspace_bytes(int qo_len, int kv_len, int n_heads, int head_dim);
+hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const void *k, const void *v,
+                             const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
+                             bool qo_is_f32, bool causal, void *workspace);
+
+// measurement helpers
+hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t bytes);
+hipError_t launch_mfma_loop(hipStream_t stream, int kind, int iters, int *sink, int n_blocks);
+
+// Tuning override hooks read once from the environment (HTPOPS_GEMV_ROWS etc.); 0 = heuristic.
+int env_int(const char *name, int fallback);
+
+}  // namespace htpops

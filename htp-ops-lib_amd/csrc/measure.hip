@@ -1,0 +1,96 @@
+// Measurement kernels: a plain copy (HBM counter calibration, attainable bandwidth) and MFMA-only loops
+// (attainable matrix-core rate). They carry no op semantics.
+#include "device_utils.h"
+#include "kernels.h"
+
+#include <stdlib.h>
+
+namespace htpops {
+
+namespace {
+
+typedef int      v4i __attribute__((ext_vector_type(4)));
+typedef int      v16i __attribute__((ext_vector_type(16)));
+typedef float    v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+
+__global__ __launch_bounds__(256) void copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n16) {
+  const size_t stride = (size_t) gridDim.x * blockDim.x;
+  for (size_t i = (size_t) blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) {
+    dst[i] = src[i];
+  }
+}
+
+// Four independent accumulator chains per wave keep the matrix pipe full.
+template <int KIND>
+__global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, int *sink) {
+  const int seed = threadIdx.x;
+  if (KIND == 0) {
+    v4i  a = { seed, seed + 1, seed + 2, seed + 3 }, b = { seed * 3, 5, 7, 9 };
+    v16i c0 = { 0 }, c1 = { 0 }, c2 = { 0 }, c3 = { 0 };
+    for (int i = 0; i < iters; ++i) {
+      c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c1, 0, 0, 0);
+      c2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c2, 0, 0, 0);
+      c3 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c3, 0, 0, 0);
+    }
+    if (c0[0] + c1[1] + c2[2] + c3[3] == 0x7fffffff) {
+      sink[0] = 1;
+    }
+  } else if (KIND == 1) {
+    v4i a = { seed, seed + 1, seed + 2, seed + 3 }, b = { seed * 3, 5, 7, 9 };
+    v4i c0 = { 0 }, c1 = { 0 }, c2 = { 0 }, c3 = { 0 };
+    for (int i = 0; i < iters; ++i) {
+      c0 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c1, 0, 0, 0);
+      c2 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c2, 0, 0, 0);
+      c3 = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c3, 0, 0, 0);
+    }
+    if (c0[0] + c1[1] + c2[2] + c3[3] == 0x7fffffff) {
+      sink[0] = 1;
+    }
+  } else {
+    v8h  a, b;
+    for (int i = 0; i < 8; ++i) {
+      a[i] = (_Float16) (float) ((seed + i) & 7);
+      b[i] = (_Float16) (float) ((seed * 3 + i) & 3);
+    }
+    v16f c0 = { 0 }, c1 = { 0 }, c2 = { 0 }, c3 = { 0 };
+    for (int i = 0; i < iters; ++i) {
+      c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c0, 0, 0, 0);
+      c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c1, 0, 0, 0);
+      c2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c2, 0, 0, 0);
+      c3 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c3, 0, 0, 0);
+    }
+    if (c0[0] + c1[1] + c2[2] + c3[3] == -1.0f) {
+      sink[0] = 1;
+    }
+  }
+}
+
+}  // namespace
+
+hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t bytes) {
+  const size_t n16 = bytes / 16;
+  hipLaunchKernelGGL(copy_kernel, dim3(256 * 8), dim3(256), 0, stream, (uint4 *) dst, (const uint4 *) src, n16);
+  return hipGetLastError();
+}
+
+hipError_t launch_mfma_loop(hipStream_t stream, int kind, int iters, int *sink, int n_blocks) {
+  dim3 grid((unsigned) n_blocks), block(256);
+  if (kind == 0) {
+    hipLaunchKernelGGL(mfma_loop_kernel<0>, grid, block, 0, stream, iters, sink);
+  } else if (kind == 1) {
+    hipLaunchKernelGGL(mfma_loop_kernel<1>, grid, block, 0, stream, iters, sink);
+  } else {
+    hipLaunchKernelGGL(mfma_loop_kernel<2>, grid, block, 0, stream, iters, sink);
+  }
+  return hipGetLastError();
+}
+
+int env_int(const char *name, int fallback) {
+  const char *v = getenv(name);
+  return (v && *v) ? atoi(v) : fallback;
+}
+
+}  // namespace htpops

@@ -1,0 +1,185 @@
+"""GPU parity: Q8_0 quantizer (bit-exact), RMSNorm (2e-3 absolute; in practice ~1e-6), quantized matmul
+(|gpu - f64| <= 1e-5 * sum|terms|, and the same against the fp32 oracle), all through the op ABI."""
+import numpy as np
+import pytest
+
+from pyhtpops import api
+from pyhtpops import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+MATMUL_RTOL = 1e-5      # relative to sum |block terms| (fp32 accumulation order differs from the oracle's)
+NORM_ATOL = 2e-3
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = api.Context(device=0)
+    yield c
+    c.close()
+
+
+# ---------------------------------------------------------------------------------------- quantizer
+
+@pytest.mark.parametrize("m,k", [(1, 4096), (8, 4096), (1, 11008), (3, 32), (5, 96), (128, 1536), (512, 4096), (7, 8960)])
+def test_quantize_q8_0_bit_exact(ctx, oracle, m, k):
+    rng = wl.rng_for(51, m * 100000 + k)
+    x = wl.make_activations(rng, m, k)
+    if m >= 3:
+        x[1] *= 1e-5          # tiny scales (fp16 subnormal d)
+        x[2] *= 2e3
+        x[0, :32] = 0         # an all-zero block
+    print("quantize case m=%d k=%d" % (m, k), flush=True)
+    got = ctx.run_quantize_q8_0(x)
+    want = oracle.quantize_q8_0(x)
+    assert np.array_equal(got, want)
+
+
+def test_quantize_q8_0_ties_and_extremes_bit_exact(ctx, oracle):
+    x = np.zeros((2, 64), np.float32)
+    x[0, 0] = 127.0
+    x[0, 1:9] = [0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 126.5, -126.5]
+    x[0, 32:64] = np.arange(32) - 16
+    x[1, :32] = np.linspace(-3e-6 * 127, 3e-6 * 127, 32)
+    x[1, 32:] = np.linspace(-6e4, 6e4, 32)
+    assert np.array_equal(ctx.run_quantize_q8_0(x), oracle.quantize_q8_0(x))
+
+
+# ------------------------------------------------------------------------------------------ rmsnorm
+
+@pytest.mark.parametrize("ne0,ne1", [(4096, 1), (1536, 1), (1536, 128), (4096, 512), (60000, 1), (33, 3), (8192, 4), (16384, 2), (24576, 2)])
+def test_rms_norm_reference_op(ctx, oracle, ne0, ne1):
+    rng = wl.rng_for(52, ne0 + ne1)
+    x = rng.uniform(-20, 20, (ne1, ne0)).astype(np.float32)   # the reference test's input range (test.c:99-102)
+    print("rms_norm case ne0=%d ne1=%d" % (ne0, ne1), flush=True)
+    got = ctx.run_rms_norm(x)
+    want = oracle.rms_norm(x, None, 1e-5)
+    assert np.abs(got - want).max() <= 1e-5   # the reference's own tolerance (test.c:116-118)
+
+
+@pytest.mark.parametrize("ne0,ne1", [(4096, 1), (1536, 128), (1536, 1), (96, 5)])
+def test_rms_norm_with_weight_and_eps(ctx, oracle, ne0, ne1):
+    rng = wl.rng_for(52, 1000 + ne0 + ne1)
+    x = wl.make_activations(rng, ne1, ne0)
+    w = (1 + 0.1 * rng.standard_normal(ne0)).astype(np.float32)
+    got = ctx.run_rms_norm(x, w, 1e-6)
+    want = oracle.rms_norm(x, w, 1e-6)
+    assert np.abs(got - want).max() <= NORM_ATOL
+    # tighter: the reference's own 1e-5 (the oracle's sequential fp32 row sum is the noisier side)
+    assert np.abs(got - want).max() <= 1e-5
+    x64 = x.astype(np.float64)
+    exact = x64 / np.sqrt((x64 ** 2).mean(axis=1, keepdims=True) + 1e-6) * w
+    assert np.abs(got - exact).max() <= 1e-6
+    got1 = ctx.run_rms_norm(x, None, 1e-6)
+    assert np.abs(got1 - oracle.rms_norm(x, None, 1e-6)).max() <= 1e-5
+
+
+@pytest.mark.parametrize("ne0,ne1", [(4096, 1), (1536, 128), (4096, 8), (16384, 2)])
+def test_fused_rms_norm_quantize_equals_the_two_ops_in_a_row(ctx, oracle, ne0, ne1):
+    rng = wl.rng_for(52, 2000 + ne0 + ne1)
+    x = wl.make_activations(rng, ne1, ne0)
+    w = (1 + 0.1 * rng.standard_normal(ne0)).astype(np.float32)
+    fused = ctx.run_rms_norm(x, w, 1e-6, quantize=True)
+    two_step = ctx.run_quantize_q8_0(ctx.run_rms_norm(x, w, 1e-6))
+    assert np.array_equal(fused, two_step)
+    # and against the oracle chain: quants within one step, scales within one fp16 ulp (the row sums differ in order)
+    want = oracle.quantize_q8_0(oracle.rms_norm(x, w, 1e-6))
+    dg, qg = wl.q8_0_split(fused, ne0)
+    dw, qw = wl.q8_0_split(want, ne0)
+    assert np.abs(qg.astype(np.int32) - qw.astype(np.int32)).max() <= 1
+    assert np.abs(dg.view(np.int16).astype(np.int32) - dw.view(np.int16).astype(np.int32)).max() <= 1
+
+
+# ------------------------------------------------------------------------------------------- matmul
+
+def check_mat_mul(ctx, oracle, rng, m, k, n, wt):
+    w = wl.make_weights(rng, n, k, wt)
+    x = wl.make_activations(rng, m, k)
+    a = oracle.quantize_q8_0(x)
+    print("mat_mul case m=%d k=%d n=%d wt=%d" % (m, k, n, wt), flush=True)
+    got = ctx.run_mat_mul(a, w, m, k, n, wt)
+    want32 = oracle.mat_mul_q8_0_act(a, w, m, k, n, wt, n_threads=8)
+    want64, mag = oracle.mat_mul_q8_0_act_f64(a, w, m, k, n, wt)
+    assert np.all(np.abs(got - want64) <= MATMUL_RTOL * mag), float((np.abs(got - want64) / mag).max())
+    assert np.all(np.abs(got - want32) <= MATMUL_RTOL * mag)
+    return got, x, w
+
+
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+@pytest.mark.parametrize("k,n", [(4096, 4096), (4096, 1024), (11008, 512), (1536, 1536), (1536, 256), (8960, 384),
+                                 (64, 32), (128, 7), (2048, 100), (1024, 33), (12288 + 64, 40), (96, 64), (32, 5), (4128, 16)])
+def test_gemv_m1(ctx, oracle, wt, k, n):
+    check_mat_mul(ctx, oracle, wl.rng_for(53, k * 7 + n + wt), 1, k, n, wt)
+
+
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+@pytest.mark.parametrize("m,k,n", [(8, 4096, 512), (2, 11008, 96), (3, 1536, 256), (8, 96, 40), (5, 64, 32), (16, 1024, 128)])
+def test_small_batch(ctx, oracle, wt, m, k, n):
+    got, x, w = check_mat_mul(ctx, oracle, wl.rng_for(54, m * 31 + k + n + wt), m, k, n, wt)
+    # the fp32-activation op quantizes on the device and must give the same bits
+    assert np.array_equal(ctx.run_mat_mul(x, w, m, k, n, wt, act_is_f32=True), got)
+
+
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+def test_mat_mul_integer_exact_special_case(ctx, wt):
+    # scales 1.0 and small integers: every partial sum is an exactly representable integer
+    rng = wl.rng_for(55, wt)
+    m, k, n = 2, 256, 96
+    w = wl.make_weights(rng, n, k, wt).reshape(n, k // 32, -1)
+    w[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    w = w.reshape(n, -1)
+    a = np.empty((m, k // 32, 34), np.uint8)
+    a[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    a[:, :, 2:] = rng.integers(-20, 21, (m, k // 32, 32), dtype=np.int8).view(np.uint8)
+    a = a.reshape(m, -1)
+    got = ctx.run_mat_mul(a, w, m, k, n, wt)
+    _, qa = wl.q8_0_split(a, k)
+    _, qw = (wl.q4_0_split if wt == wl.GGML_TYPE_Q4_0 else wl.q8_0_split)(w, k)
+    assert np.array_equal(got, (qa.astype(np.int64) @ qw.astype(np.int64).T).astype(np.float32))
+
+
+def test_block_dot_extremes_are_exact(ctx):
+    # all weights -8 and all activations -127: 32512 per block, times scales 1 -> exact
+    k, n = 128, 32
+    w = np.zeros((n, k // 32, 18), np.uint8)
+    w[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    a = np.empty((1, k // 32, 34), np.uint8)
+    a[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    a[:, :, 2:] = np.int8(-127).view(np.uint8)
+    got = ctx.run_mat_mul(a.reshape(1, -1), w.reshape(n, -1), 1, k, n, wl.GGML_TYPE_Q4_0)
+    assert np.all(got == 4 * 32512.0)
+    w[:] = 0xFF
+    w[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    got = ctx.run_mat_mul(a.reshape(1, -1), w.reshape(n, -1), 1, k, n, wl.GGML_TYPE_Q4_0)
+    assert np.all(got == 4 * (-7 * 127 * 32.0))
+
+
+def test_message_with_a_decode_chain_runs_in_order(ctx, oracle):
+    # RMSNorm -> quantize -> GEMV submitted as one mailbox message (config 0 of the benchmark, small n)
+    rng = wl.rng_for(0, 0)
+    k, n = 4096, 256
+    w = wl.make_q4_0_weights(rng, n, k)
+    x = wl.make_activations(rng, 1, k)
+    hx, hn, hq, hw, ho = ctx.upload(x), ctx.alloc(k * 4), ctx.alloc(k // 32 * 34), ctx.upload(w), ctx.alloc(n * 4)
+    ones = ctx.upload(np.ones(k, np.float32))
+    reqs = [
+        (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(api.HTP_OPS_RMS_NORM_F32_EX, api.rms_norm_ex_params((hn, 0), (hx, 0), (ones, 0), k, 1, 1e-6))),
+        (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(api.HTP_OPS_QUANTIZE_Q8_0, api.rms_norm_params((hq, 0), (hn, 0), k, 1))),
+        (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(api.HTP_OPS_MAT_MUL_Q4_0_Q8_0, api.mat_mul_params((ho, 0), (hq, 0), (hw, 0), 1, k, n))),
+        (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(api.HTP_OPS_RMS_NORM_F32, api.rms_norm_params((hn, 0), (hx, 0), 0, 1))),
+    ]
+    msg = api.build_message(reqs)
+    msg[0] = 1
+    assert ctx.process_message(msg) == 0
+    assert api.message_request_states(msg) == [0, 0, 0, -1] and msg[1] == 1
+    got = ctx.read(ho, np.float32, n)
+    normed = oracle.rms_norm(x, np.ones(k, np.float32), 1e-6)
+    gpu_normed = ctx.read(hn, np.float32, k)
+    assert np.abs(gpu_normed - normed[0]).max() <= 1e-5
+    # quantization of the GPU's own normalized row is bit-exact, and the GEMV on it matches the oracle
+    a = oracle.quantize_q8_0(gpu_normed[None, :])
+    assert np.array_equal(ctx.read(hq, np.uint8, k // 32 * 34), a[0])
+    want64, mag = oracle.mat_mul_q8_0_act_f64(a, w, 1, k, n, wl.GGML_TYPE_Q4_0)
+    assert np.all(np.abs(got - want64[0]) <= MATMUL_RTOL * mag[0])
+    for h in (hx, hn, hq, hw, ho, ones):
+        ctx.release(h)
