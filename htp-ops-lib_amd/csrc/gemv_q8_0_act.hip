@@ -480,10 +480,8 @@ hipError_t launch_gemv_row(hipStream_t stream, float *out, const uint32_t *act, 
   static const int use_shared     = env_int("HTPOPS_GEMV_SHARED", 1);
   constexpr int    PD             = Pair<WT>::kDwords;
   if (use_shared && pairs <= 192) {
-    int r = 2, threads = 256;
-    if (pairs > 64) {
-      r = 1, threads = 512;
-    }
+    // measured on MI355X: short-lived waves (one row set each) in 256-thread groups stream best
+    int r = 1, threads = 256;
     if (forced_r) {
       r = forced_r;
     }

@@ -183,3 +183,49 @@ def test_message_with_a_decode_chain_runs_in_order(ctx, oracle):
     assert np.all(np.abs(got - want64[0]) <= MATMUL_RTOL * mag[0])
     for h in (hx, hn, hq, hw, ho, ones):
         ctx.release(h)
+
+
+# --------------------------------------------------------------------------------- prefill (MFMA) path
+
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+@pytest.mark.parametrize("m,k,n", [(128, 1536, 256), (512, 4096, 128), (100, 11008, 96), (33, 2048, 70),
+                                   (64, 192, 64), (129, 320, 65), (32, 4096, 512), (17, 1536, 130), (512, 128, 64)])
+def test_gemm_mfma(ctx, oracle, wt, m, k, n):
+    check_mat_mul(ctx, oracle, wl.rng_for(56, m * 131 + k + n + wt), m, k, n, wt)
+
+
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+def test_gemm_mfma_integer_exact(ctx, wt):
+    # scales 1.0 and small integers: the block sums come straight out of the matrix cores
+    rng = wl.rng_for(57, wt)
+    m, k, n = 96, 512, 160
+    w = wl.make_weights(rng, n, k, wt).reshape(n, k // 32, -1)
+    w[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    w = w.reshape(n, -1)
+    a = np.empty((m, k // 32, 34), np.uint8)
+    a[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    a[:, :, 2:] = rng.integers(-127, 128, (m, k // 32, 32), dtype=np.int8).view(np.uint8)
+    a = a.reshape(m, -1)
+    got = ctx.run_mat_mul(a, w, m, k, n, wt)
+    _, qa = wl.q8_0_split(a, k)
+    _, qw = (wl.q4_0_split if wt == wl.GGML_TYPE_Q4_0 else wl.q8_0_split)(w, k)
+    assert np.array_equal(got, (qa.astype(np.int64) @ qw.astype(np.int64).T).astype(np.float32))
+
+
+def test_gemm_full_prefill_shape_rows_match_the_decode_kernel(ctx, oracle):
+    # M = 512, K = 4096, N = 11008 is too large for the scalar oracle in a test: check (a) a sample of rows against
+    # the oracle and (b) every row against the GEMV kernel of the same row (independent kernel, same arithmetic)
+    rng = wl.rng_for(2, 0)
+    m, k, n = 512, 4096, 11008
+    w = wl.make_q4_0_weights(rng, n, k)
+    x = wl.make_activations(rng, m, k)
+    a = oracle.quantize_q8_0(x)
+    print("full prefill shape", flush=True)
+    got = ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
+    rows = [0, 1, 31, 32, 255, 256, 511]
+    want64, mag = oracle.mat_mul_q8_0_act_f64(a[rows], w, len(rows), k, n, wl.GGML_TYPE_Q4_0)
+    assert np.all(np.abs(got[rows] - want64) <= MATMUL_RTOL * mag)
+    for r in (5, 130, 300, 500):
+        gemv = ctx.run_mat_mul(a[r:r + 1], w, 1, k, n, wl.GGML_TYPE_Q4_0)
+        scale = np.abs(gemv).max()
+        assert np.abs(gemv[0] - got[r]).max() <= 2e-5 * scale
