@@ -1,8 +1,519 @@
+// Attention for gfx950: O = softmax(Q K^T / sqrt(D) + mask) V per head, GQA by h_kv = h / (n_heads / n_kv_heads).
+//
+// Replaces simple_flash_attn (reference: src/dsp/ops/flash_attn.c:1368-1420, core :139-825): the same blockwise
+// online-softmax recurrence with exp2 and the scale 1/sqrt(D) * log2(e) (reference :210-215, :1440), laid out for
+// 64-wide wavefronts and MFMA instead of HVX/HMX tiles in VTCM. Q/O are fp32 (the reference op) or fp16; K/V fp16
+// [kv_len][n_kv_heads][D]; the optional fp16 mask [qo_len][align_up(kv_len, 64)] is ADDED to the scaled scores (the
+// scalar routine's convention, reference :1505-1512); `causal` hides key j from query i when j > i + kv_len - qo_len.
+//
+// Two kernels:
+//  * prefill (any qo_len): one workgroup = 32 query rows x up to 4 query heads of one KV head (one wave per head,
+//    so a K/V tile staged in LDS serves the whole GQA group). Scores are computed transposed, S^T = K Q^T with
+//    v_mfma_f32_32x32x16_f16, which puts one query per lane: row max / row sum are register reductions plus one
+//    exchange between the two lane halves. O^T += V^T P^T uses V transposed on its way into LDS; P goes from the
+//    score registers straight into the MFMA B operand. Under `causal`, KV blocks above the diagonal are skipped.
+//  * decode (qo_len == 1): bandwidth bound. The KV range is split across workgroups (n_kv_heads alone would leave
+//    the GPU idle); 16 lanes share a key (16 bytes of K and V each), all heads of the GQA group are scored against
+//    the same K/V registers, and a second tiny kernel merges the per-split (max, sum, O) partials.
+#include "device_utils.h"
 #include "kernels.h"
+
 namespace htpops {
-size_t flash_attn_workspace_bytes(int, int, int, int) { return 0; }
-hipError_t launch_flash_attn(hipStream_t, void *, const void *, const void *, const void *, const void *, int, int, int,
-                             int, int, bool, bool, void *) {
-  return hipErrorNotSupported;
+
+namespace {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef _Float16 v2h __attribute__((ext_vector_type(2)));
+typedef float    v16f __attribute__((ext_vector_type(16)));
+
+constexpr float kLog2e = 1.44269504f;
+
+__device__ __forceinline__ float fast_exp2(float x) {
+  return __builtin_amdgcn_exp2f(x);  // v_exp_f32; exp2(-inf) = 0
 }
+
+// ------------------------------------------------------------------------------------------------ prefill
+
+constexpr int kPfThreads = 256;
+constexpr int kBQ        = 32;  // query rows per wave tile
+constexpr int kBK        = 64;  // keys per KV block
+
+template <int D>
+struct PrefillSmem {
+  // K tile: [key][D] halfs, rows padded by 16 bytes (conflict-free 16-byte fragment reads)
+  _Float16 k[kBK][D + 8];
+  // V^T tile: [d][key] halfs, rows padded by 8 bytes; row d stores key j at column (j + 8 (d / 32)) % 64 so that the
+  // transposing stores of one wave hit 64 different banks
+  _Float16 vt[D][kBK + 4];
+};
+
+template <int D, bool QO_F32>
+__global__ __launch_bounds__(kPfThreads) void flash_attn_prefill_kernel(void *__restrict__ o_ptr,
+                                                                        const void *__restrict__ q_ptr,
+                                                                        const _Float16 *__restrict__ k_ptr,
+                                                                        const _Float16 *__restrict__ v_ptr,
+                                                                        const _Float16 *__restrict__ mask, int qo_len,
+                                                                        int kv_len, int n_heads, int n_kv_heads,
+                                                                        int causal) {
+  __shared__ PrefillSmem<D> sm;
+  constexpr int KSTEPS = D / 16;  // MFMA k-steps over the head dimension
+  constexpr int DT     = D / 32;  // 32-row tiles of O^T
+
+  const int group = n_heads / n_kv_heads;
+  const int gc    = group < 4 ? group : 4;  // heads handled by one workgroup
+  const int qsub  = 4 / gc;                 // query sub-blocks per workgroup (waves left over when group < 4)
+  const int sub_groups = (group + gc - 1) / gc;
+
+  const int tid  = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int half = lane >> 5;
+  const int col  = lane & 31;
+
+  const int h_kv     = blockIdx.y / sub_groups;
+  const int h_in_grp = (blockIdx.y % sub_groups) * gc + wave % gc;
+  const bool wave_on = h_in_grp < group && wave / gc < qsub;
+  const int  head    = h_kv * group + (h_in_grp < group ? h_in_grp : 0);
+  const int  q_base  = (blockIdx.x * qsub + (wave / gc < qsub ? wave / gc : 0)) * kBQ;
+  const int  q_row   = q_base + col;                  // this lane's query
+  const bool q_ok    = wave_on && q_row < qo_len;
+  const int  q_clamp = q_row < qo_len ? q_row : qo_len - 1;
+
+  const size_t qo_stride = (size_t) n_heads * D;
+  const size_t kv_stride = (size_t) n_kv_heads * D;
+  const size_t mask_ld   = ((size_t) kv_len + 63) / 64 * 64;
+  const float  scale     = (1.0f / sqrtf((float) D)) * kLog2e;
+
+  // Q fragments (B operand of S^T = K Q^T): lane (query, half) holds d = 16 s + 8 half .. + 7 for every k-step s
+  v8h qf[KSTEPS];
+  {
+    const size_t base = (size_t) q_clamp * qo_stride + (size_t) head * D;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      const int d0 = 16 * s + 8 * half;
+      if (QO_F32) {
+        const float4 *p  = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(q_ptr) + base + d0);
+        const float4  a  = p[0], b = p[1];
+        qf[s][0] = (_Float16) (a.x * scale), qf[s][1] = (_Float16) (a.y * scale);
+        qf[s][2] = (_Float16) (a.z * scale), qf[s][3] = (_Float16) (a.w * scale);
+        qf[s][4] = (_Float16) (b.x * scale), qf[s][5] = (_Float16) (b.y * scale);
+        qf[s][6] = (_Float16) (b.z * scale), qf[s][7] = (_Float16) (b.w * scale);
+      } else {
+        const v8h raw = *reinterpret_cast<const v8h *>(reinterpret_cast<const _Float16 *>(q_ptr) + base + d0);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          qf[s][e] = (_Float16) ((float) raw[e] * scale);
+        }
+      }
+    }
+  }
+
+  v16f  oacc[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      oacc[t][r] = 0.0f;
+    }
+  }
+  float m_run = -INFINITY;  // running max of this lane's query (same in both halves)
+  float l_run = 0.0f;       // running sum over this half's keys only; halves are added at the end
+
+  // keys visible to the LAST query row of the workgroup bound the KV loop under `causal`
+  const int q_hi     = min(qo_len, (int) (blockIdx.x + 1) * qsub * kBQ) - 1;
+  const int kv_limit = causal ? min(kv_len, q_hi + (kv_len - qo_len) + 1) : kv_len;
+  const int q_shift  = kv_len - qo_len;
+
+  for (int k0 = 0; k0 < kv_limit; k0 += kBK) {
+    __syncthreads();  // previous block's fragments are no longer needed
+    // ---- stage K [key][D] and V^T [d][key] ----
+    {
+      // K: 16-byte pieces, coalesced along d
+      constexpr int PIECES = kBK * D / 8;  // 8 halfs each
+#pragma unroll
+      for (int i = tid; i < PIECES; i += kPfThreads) {
+        const int key = i / (D / 8), part = i % (D / 8);
+        const int kg  = min(k0 + key, kv_len - 1);
+        const v8h v   = *reinterpret_cast<const v8h *>(k_ptr + (size_t) kg * kv_stride + (size_t) h_kv * D + part * 8);
+        *reinterpret_cast<v8h *>(&sm.k[key][part * 8]) = v;
+      }
+      // V^T: a task = (key pair, 8-wide d chunk): two 16-byte loads, eight 4-byte transposed stores
+      constexpr int TASKS = (kBK / 2) * (D / 8);
+#pragma unroll
+      for (int i = tid; i < TASKS; i += kPfThreads) {
+        const int c = i % (D / 8), kp = i / (D / 8);
+        const int kg0 = min(k0 + 2 * kp, kv_len - 1), kg1 = min(k0 + 2 * kp + 1, kv_len - 1);
+        const v8h a = *reinterpret_cast<const v8h *>(v_ptr + (size_t) kg0 * kv_stride + (size_t) h_kv * D + c * 8);
+        const v8h b = *reinterpret_cast<const v8h *>(v_ptr + (size_t) kg1 * kv_stride + (size_t) h_kv * D + c * 8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int d   = c * 8 + e;
+          const int pos = (2 * kp + 8 * (d / 32)) % kBK;
+          v2h       pr  = { a[e], b[e] };
+          *reinterpret_cast<v2h *>(&sm.vt[d][pos]) = pr;
+        }
+      }
+    }
+    __syncthreads();
+
+    // ---- S^T = K Q^T: two 32-key tiles ----
+    v16f st[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        st[kt][r] = 0.0f;
+      }
+#pragma unroll
+      for (int s = 0; s < KSTEPS; ++s) {
+        const v8h kf = *reinterpret_cast<const v8h *>(&sm.k[32 * kt + col][16 * s + 8 * half]);
+        st[kt]       = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], st[kt], 0, 0, 0);
+      }
+    }
+
+    // ---- mask, online softmax (lane = query; register r of tile kt is key 32 kt + 8 (r / 4) + 4 half + r % 4) ----
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = k0 + 32 * kt + 8 * (r >> 2) + 4 * half + (r & 3);
+        float     s   = st[kt][r];
+        if (mask) {
+          s += (float) mask[(size_t) q_clamp * mask_ld + (size_t) min(key, (int) mask_ld - 1)];
+        }
+        if (key >= kv_len || (causal && key > q_row + q_shift)) {
+          s = -INFINITY;
+        }
+        st[kt][r] = s;
+        mx        = fmaxf(mx, s);
+      }
+    }
+    mx                 = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+    const float m_new  = fmaxf(m_run, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // a fully masked prefix keeps exp2 arguments finite
+    const float alpha  = fast_exp2(m_run - m_safe);            // exp2(-inf) = 0 on the first visible block
+    float       psum   = 0.0f;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = fast_exp2(st[kt][r] - m_safe);
+        st[kt][r]     = p;
+        psum += p;
+      }
+    }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        oacc[t][r] *= alpha;
+      }
+    }
+
+    // ---- O^T += V^T P^T ----
+    // MFMA (kt, u) covers keys 32 kt + 16 u + {4 half + 0..3, 8 + 4 half + 0..3}: exactly registers 8 u .. 8 u + 7
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        v8h pf;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          pf[e] = (_Float16) st[kt][8 * u + e];
+        }
+#pragma unroll
+        for (int t = 0; t < DT; ++t) {
+          const int d    = 32 * t + col;
+          const int key0 = (32 * kt + 16 * u + 4 * half + 8 * t) % kBK;  // rotated column of the first 4 keys
+          const int key1 = (key0 + 8) % kBK;
+          const v4h a0   = *reinterpret_cast<const v4h *>(&sm.vt[d][key0]);
+          const v4h a1   = *reinterpret_cast<const v4h *>(&sm.vt[d][key1]);
+          v8h       vf   = { a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3] };
+          oacc[t]        = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf, oacc[t], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // ---- finish: O = O^T / l, one query per lane; register r of tile t is d = 32 t + 8 (r / 4) + 4 half + r % 4 ----
+  const float l_tot = l_run + __shfl_xor(l_run, 32, kWave);
+  const float inv   = 1.0f / l_tot;
+  if (q_ok) {
+    const size_t base = (size_t) q_row * qo_stride + (size_t) head * D;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const int d0 = 32 * t + 8 * rg + 4 * half;
+        float     v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = oacc[t][4 * rg + e] * inv;
+        }
+        if (QO_F32) {
+          *reinterpret_cast<float4 *>(reinterpret_cast<float *>(o_ptr) + base + d0) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+          v4h hv = { (_Float16) v[0], (_Float16) v[1], (_Float16) v[2], (_Float16) v[3] };
+          *reinterpret_cast<v4h *>(reinterpret_cast<_Float16 *>(o_ptr) + base + d0) = hv;
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ decode
+
+constexpr int kDecThreads  = 256;
+constexpr int kDecMaxGroup = 8;   // query heads scored per pass against one K/V stream
+constexpr int kDecSplit    = 128; // keys per workgroup
+
+// partial record per (head, split): m, l, then D floats of un-normalised O
+template <int D, int GH, bool QO_F32>
+__global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *__restrict__ part,
+                                                                        const void *__restrict__ q_ptr,
+                                                                        const _Float16 *__restrict__ k_ptr,
+                                                                        const _Float16 *__restrict__ v_ptr,
+                                                                        const _Float16 *__restrict__ mask, int kv_len,
+                                                                        int n_heads, int n_kv_heads, int head0_in_group,
+                                                                        int n_splits) {
+  constexpr int LPK = D / 8;        // lanes per key (8 halfs = 16 bytes each)
+  constexpr int KPW = kWave / LPK;  // keys per wave per pass
+  constexpr int WAVES = kDecThreads / kWave;
+  __shared__ float red_m[WAVES][GH], red_l[WAVES][GH], red_o[WAVES][GH][D];
+
+  const int group = n_heads / n_kv_heads;
+  const int h_kv  = blockIdx.y;
+  const int split = blockIdx.x;
+  const int lane  = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub   = lane % LPK;  // which 8 dims
+  const int kslot = lane / LPK;  // which key of the pass
+  const float scale = (1.0f / sqrtf((float) D)) * kLog2e;
+  const size_t kv_stride = (size_t) n_kv_heads * D;
+
+  // q for the GH heads, this lane's 8 dims, pre-scaled
+  float q[GH][8];
+#pragma unroll
+  for (int g = 0; g < GH; ++g) {
+    const int hg = min(head0_in_group + g, group - 1);
+    const size_t base = (size_t) (h_kv * group + hg) * D + sub * 8;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = QO_F32 ? reinterpret_cast<const float *>(q_ptr)[base + e] :
+                               (float) reinterpret_cast<const _Float16 *>(q_ptr)[base + e];
+      q[g][e]       = v * scale;
+    }
+  }
+
+  float m_run[GH], l_run[GH], o[GH][8];
+#pragma unroll
+  for (int g = 0; g < GH; ++g) {
+    m_run[g] = -INFINITY, l_run[g] = 0.0f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      o[g][e] = 0.0f;
+    }
+  }
+
+  const int k_begin = split * kDecSplit;
+  const int k_end   = min(kv_len, k_begin + kDecSplit);
+  for (int kb = k_begin + wave * KPW; kb < k_end; kb += WAVES * KPW) {
+    const int  key  = kb + kslot;
+    const bool live = key < k_end;
+    const int  kc   = live ? key : k_end - 1;
+    const v8h  kv8  = *reinterpret_cast<const v8h *>(k_ptr + (size_t) kc * kv_stride + (size_t) h_kv * D + sub * 8);
+    const v8h  vv8  = *reinterpret_cast<const v8h *>(v_ptr + (size_t) kc * kv_stride + (size_t) h_kv * D + sub * 8);
+    float kf[8], vf[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      kf[e] = (float) kv8[e], vf[e] = (float) vv8[e];
+    }
+    const float mk = (mask && live) ? (float) mask[key] : 0.0f;  // row 0 of the mask (qo_len == 1)
+#pragma unroll
+    for (int g = 0; g < GH; ++g) {
+      float s = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        s += q[g][e] * kf[e];
+      }
+      s = group_sum<LPK>(s) + mk;  // every lane of the key's group holds the score
+      s = live ? s : -INFINITY;
+      const float m_new  = fmaxf(m_run[g], s);
+      const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+      const float alpha  = fast_exp2(m_run[g] - m_safe);
+      const float p      = fast_exp2(s - m_safe);
+      l_run[g]           = l_run[g] * alpha + p;
+      m_run[g]           = m_new;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        o[g][e] = o[g][e] * alpha + p * vf[e];
+      }
+    }
+  }
+
+  // merge the KPW key slots of the wave (lanes with equal `sub`), then the waves, then write the partial
+#pragma unroll
+  for (int g = 0; g < GH; ++g) {
+    float m_all = m_run[g];
+#pragma unroll
+    for (int off = LPK; off < kWave; off <<= 1) {
+      m_all = fmaxf(m_all, __shfl_xor(m_all, off, kWave));
+    }
+    const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
+    const float f      = fast_exp2(m_run[g] - m_safe);
+    float       l      = l_run[g] * f;
+#pragma unroll
+    for (int off = LPK; off < kWave; off <<= 1) {
+      l += __shfl_xor(l, off, kWave);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float v = o[g][e] * f;
+#pragma unroll
+      for (int off = LPK; off < kWave; off <<= 1) {
+        v += __shfl_xor(v, off, kWave);
+      }
+      if (kslot == 0) {
+        red_o[wave][g][sub * 8 + e] = v;
+      }
+    }
+    if (lane == 0) {
+      red_m[wave][g] = m_all, red_l[wave][g] = l;
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < GH * D; i += kDecThreads) {
+    const int g = i / D, d = i % D;
+    if (head0_in_group + g >= group) {
+      continue;
+    }
+    float m_all = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      m_all = fmaxf(m_all, red_m[w][g]);
+    }
+    const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
+    float       l = 0.0f, v = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const float f = fast_exp2(red_m[w][g] - m_safe);
+      l += red_l[w][g] * f;
+      v += red_o[w][g][d] * f;
+    }
+    const int    head = h_kv * group + head0_in_group + g;
+    float       *rec  = part + ((size_t) head * n_splits + split) * (D + 2);
+    if (d == 0) {
+      rec[0] = m_all, rec[1] = l;
+    }
+    rec[2 + d] = v;
+  }
+}
+
+template <int D, bool QO_F32>
+__global__ __launch_bounds__(D) void flash_attn_decode_merge_kernel(void *__restrict__ o_ptr,
+                                                                    const float *__restrict__ part, int n_splits) {
+  const int    head = blockIdx.x, d = threadIdx.x;
+  const float *rec0 = part + (size_t) head * n_splits * (D + 2);
+  float        m_all = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) {
+    m_all = fmaxf(m_all, rec0[(size_t) s * (D + 2)]);
+  }
+  const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
+  float       l = 0.0f, v = 0.0f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float *rec = rec0 + (size_t) s * (D + 2);
+    const float  f   = fast_exp2(rec[0] - m_safe);
+    l += rec[1] * f;
+    v += rec[2 + d] * f;
+  }
+  const float out = v * (1.0f / l);
+  if (QO_F32) {
+    reinterpret_cast<float *>(o_ptr)[(size_t) head * D + d] = out;
+  } else {
+    reinterpret_cast<_Float16 *>(o_ptr)[(size_t) head * D + d] = (_Float16) out;
+  }
+}
+
+template <int D, bool QO_F32>
+hipError_t launch_prefill(hipStream_t stream, void *o, const void *q, const void *k, const void *v, const void *mask,
+                          int qo_len, int kv_len, int n_heads, int n_kv_heads, bool causal) {
+  const int group      = n_heads / n_kv_heads;
+  const int gc         = group < 4 ? group : 4;
+  const int qsub       = 4 / gc;
+  const int sub_groups = (group + gc - 1) / gc;
+  const dim3 grid((unsigned) ((qo_len + qsub * kBQ - 1) / (qsub * kBQ)), (unsigned) (n_kv_heads * sub_groups));
+  hipLaunchKernelGGL((flash_attn_prefill_kernel<D, QO_F32>), grid, dim3(kPfThreads), 0, stream, o, q,
+                     (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, qo_len, kv_len, n_heads,
+                     n_kv_heads, causal ? 1 : 0);
+  return hipGetLastError();
+}
+
+template <int D, bool QO_F32>
+hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void *k, const void *v, const void *mask,
+                         int kv_len, int n_heads, int n_kv_heads, float *workspace) {
+  const int  group    = n_heads / n_kv_heads;
+  const int  n_splits = (kv_len + kDecSplit - 1) / kDecSplit;
+  const dim3 grid((unsigned) n_splits, (unsigned) n_kv_heads);
+  for (int h0 = 0; h0 < group; h0 += kDecMaxGroup) {
+    const int gh = group - h0;
+#define HTPOPS_DECODE(GH)                                                                                          \
+  hipLaunchKernelGGL((flash_attn_decode_kernel<D, GH, QO_F32>), grid, dim3(kDecThreads), 0, stream, workspace, q,   \
+                     (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, kv_len, n_heads,          \
+                     n_kv_heads, h0, n_splits)
+    if (gh >= 8) {
+      HTPOPS_DECODE(8);
+    } else if (gh > 4) {
+      HTPOPS_DECODE(8);
+    } else if (gh > 2) {
+      HTPOPS_DECODE(4);
+    } else if (gh == 2) {
+      HTPOPS_DECODE(2);
+    } else {
+      HTPOPS_DECODE(1);
+    }
+#undef HTPOPS_DECODE
+  }
+  hipLaunchKernelGGL((flash_attn_decode_merge_kernel<D, QO_F32>), dim3((unsigned) n_heads), dim3(D), 0, stream, o,
+                     workspace, n_splits);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+size_t flash_attn_workspace_bytes(int qo_len, int kv_len, int n_heads, int head_dim) {
+  if (qo_len != 1) {
+    return 0;
+  }
+  const size_t n_splits = ((size_t) kv_len + kDecSplit - 1) / kDecSplit;
+  return (size_t) n_heads * n_splits * ((size_t) head_dim + 2) * sizeof(float);
+}
+
+hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const void *k, const void *v,
+                             const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
+                             bool qo_is_f32, bool causal, void *workspace) {
+  if (head_dim != 64 && head_dim != 128) {
+    return hipErrorNotSupported;
+  }
+  // with a single query row the causal rule (key j visible iff j <= kv_len - 1) hides nothing
+  if (qo_len == 1) {
+    float *ws = static_cast<float *>(workspace);
+    if (head_dim == 128) {
+      return qo_is_f32 ? launch_decode<128, true>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws) :
+                         launch_decode<128, false>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws);
+    }
+    return qo_is_f32 ? launch_decode<64, true>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws) :
+                       launch_decode<64, false>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws);
+  }
+  if (head_dim == 128) {
+    return qo_is_f32 ?
+             launch_prefill<128, true>(stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, causal) :
+             launch_prefill<128, false>(stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, causal);
+  }
+  return qo_is_f32 ? launch_prefill<64, true>(stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, causal) :
+                     launch_prefill<64, false>(stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, causal);
+}
+
 }  // namespace htpops

@@ -643,10 +643,11 @@ extern "C" int htpops_execute_op(htpops_context *ctx, const struct OpComputeRequ
   }
 }
 
-extern "C" int htpops_process_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes) {
-  if (!ctx || !msg) {
-    return HTPOPS_ERR_REJECTED;
-  }
+namespace {
+
+// Walks a message and enqueues every request in order (reference: src/dsp/commu.c:91-114). Returns 0 or the
+// framing error; per-request results go to RequestHeader.state.
+int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes) {
   const int n_reqs = msg->n_reqs;
   if (n_reqs < 0 || n_reqs > (1 << 20)) {
     return fail(ctx, HTPOPS_ERR_REJECTED, "message: n_reqs=%d", n_reqs);
@@ -665,8 +666,6 @@ extern "C" int htpops_process_message(htpops_context *ctx, struct MessageHeader 
       prev = off;
     }
   }
-  const uint8_t v0 = msg->state.v[0];
-
   for (int i = 0; i < n_reqs; ++i) {
     struct RequestHeader *hdr  = message_header_get_request_ptr(msg, i);
     const size_t          size = message_header_get_request_size(msg, i);
@@ -698,10 +697,26 @@ extern "C" int htpops_process_message(htpops_context *ctx, struct MessageHeader 
         break;  // NO_OP and unknown types are skipped, state untouched (commu.c:111-113)
     }
   }
+  return HTPOPS_OK;
+}
 
-  int ret = htpops_synchronize(ctx);
+}  // namespace
+
+extern "C" int htpops_enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes) {
+  if (!ctx || !msg) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  return enqueue_message(ctx, msg, msg_bytes);
+}
+
+extern "C" int htpops_finish_message(htpops_context *ctx, struct MessageHeader *msg) {
+  if (!ctx || !msg) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  const uint8_t v0  = msg->state.v[0];
+  int           ret = htpops_synchronize(ctx);
   if (ret != HTPOPS_OK) {
-    for (int i = 0; i < n_reqs; ++i) {
+    for (int i = 0; i < msg->n_reqs; ++i) {
       struct RequestHeader *hdr = message_header_get_request_ptr(msg, i);
       if (hdr->type == REQUEST_TYPE_OP_COMPUTE && hdr->state == 0) {
         hdr->state = ret;
@@ -711,6 +726,17 @@ extern "C" int htpops_process_message(htpops_context *ctx, struct MessageHeader 
   // publish completion: state.d = v0 | 1 << 8 with release ordering (reference: commu.c:125-126)
   store_state(msg, (uint64_t) v0 | ((uint64_t) 1 << 8));
   return HTPOPS_OK;
+}
+
+extern "C" int htpops_process_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes) {
+  if (!ctx || !msg) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  int ret = enqueue_message(ctx, msg, msg_bytes);
+  if (ret != HTPOPS_OK) {
+    return ret;
+  }
+  return htpops_finish_message(ctx, msg);
 }
 
 // ------------------------------------------------------------------------------------------------ channel

@@ -89,6 +89,13 @@ int htpops_execute_op(htpops_context *ctx, const struct OpComputeRequest *req);
  * required to be set. */
 int htpops_process_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes);
 
+/* The two halves of htpops_process_message, for producers that keep several messages in flight:
+ * htpops_enqueue_message walks the message and enqueues its requests (per-request codes are stored at once; the
+ * done byte is not touched); htpops_finish_message waits for the stream and publishes completion. Messages
+ * enqueued on one context run in enqueue order (the reference's single consumer thread, src/dsp/commu.c:43). */
+int htpops_enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes);
+int htpops_finish_message(htpops_context *ctx, struct MessageHeader *msg);
+
 /* Replaces htp_ops_create_channel / htp_ops_destroy_channel (reference: include/htp_ops.idl:11-12,
  * src/dsp/commu.c:151-212): starts a consumer thread that polls msg->state exactly as
  * msg_receiver_loop does (run when v[0] != 0 && v[1] == 0) and calls htpops_process_message.

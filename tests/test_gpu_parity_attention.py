@@ -1,0 +1,114 @@
+"""GPU parity of the attention op against the oracle (2e-3 absolute, the bar for fp16 attention), the fixtures
+written from the reference's scalar routine, and size-independent invariants at the benchmark's full sizes."""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+from pyhtpops import api
+from pyhtpops import workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+ATOL = 2e-3
+
+
+@pytest.fixture(scope="module")
+def ctx():
+    c = api.Context(device=0)
+    yield c
+    c.close()
+
+
+CASES = [
+    # qo, kv, heads, kv heads, D
+    (1, 300, 8, 2, 128), (1, 4096, 32, 8, 128), (1, 70, 4, 4, 64), (1, 129, 16, 1, 128), (1, 1, 4, 2, 64),
+    (5, 70, 4, 2, 64), (40, 300, 4, 1, 128), (33, 517, 4, 4, 128), (64, 64, 2, 1, 64), (128, 128, 8, 2, 128),
+    (100, 260, 6, 2, 128), (31, 95, 3, 1, 64), (2, 2, 2, 2, 64), (96, 200, 8, 1, 128),
+]
+
+
+@pytest.mark.parametrize("qo,kv,nh,nkv,d", CASES)
+def test_reference_op_fp32_qo_with_and_without_mask(ctx, oracle, qo, kv, nh, nkv, d):
+    rng = wl.rng_for(61, qo * 1000 + kv + nh)
+    q, k, v = wl.make_attention_inputs(rng, qo, kv, nh, nkv, d)
+    q32 = q.astype(np.float32)
+    print("attention case", qo, kv, nh, nkv, d, flush=True)
+    for mask in (None, wl.make_causal_mask(qo, kv)):
+        got = ctx.run_flash_attn(q32, k, v, mask, nh, nkv, d)
+        want = oracle.flash_attn(q32, k, v, mask, nh, nkv, d)
+        assert got.dtype == np.float32 and np.abs(got - want).max() <= ATOL
+
+
+@pytest.mark.parametrize("qo,kv,nh,nkv,d", CASES)
+def test_fp16_op_with_causal_flag(ctx, oracle, qo, kv, nh, nkv, d):
+    rng = wl.rng_for(62, qo * 1000 + kv + nh)
+    q, k, v = wl.make_attention_inputs(rng, qo, kv, nh, nkv, d)
+    got = ctx.run_flash_attn(q, k, v, None, nh, nkv, d, causal=True)
+    want = oracle.flash_attn(q, k, v, None, nh, nkv, d, True)
+    assert got.dtype == np.float16
+    assert np.abs(got.astype(np.float32) - want.astype(np.float32)).max() <= ATOL
+    # the causal flag and the equivalent additive mask agree
+    masked = ctx.run_flash_attn(q, k, v, wl.make_causal_mask(qo, kv), nh, nkv, d, causal=False)
+    assert np.abs(got.astype(np.float32) - masked.astype(np.float32)).max() <= 1e-3
+
+
+def test_fixtures_from_the_reference_routine(ctx, golden_dir):
+    files = sorted(glob.glob(os.path.join(golden_dir, "naive_flash_attn_*.npz")))
+    assert len(files) >= 3
+    for f in files:
+        z = np.load(f)
+        qo, kv, nh, nkv, d, masked = [int(t) for t in z["dims"]]
+        got = ctx.run_flash_attn(z["q"], z["k"], z["v"], z["mask"] if masked else None, nh, nkv, d)
+        assert np.abs(got - z["out"]).max() <= ATOL, os.path.basename(f)
+
+
+def test_additive_mask_with_finite_biases(ctx, oracle):
+    # the op follows the scalar routine's additive convention (reference flash_attn.c:1505-1512)
+    rng = wl.rng_for(63, 0)
+    qo, kv, nh, nkv, d = 37, 130, 4, 2, 128
+    q, k, v = wl.make_attention_inputs(rng, qo, kv, nh, nkv, d)
+    mask = np.full((qo, 192), -np.inf, np.float16)
+    mask[:, :kv] = (rng.standard_normal((qo, kv)) * 2).astype(np.float16)
+    q32 = q.astype(np.float32)
+    got = ctx.run_flash_attn(q32, k, v, mask, nh, nkv, d)
+    assert np.abs(got - oracle.flash_attn(q32, k, v, mask, nh, nkv, d)).max() <= ATOL
+
+
+def test_full_size_invariants(ctx):
+    # benchmark shapes: 32 query heads, 8 KV heads, D = 128; decode kv = 4096, prefill q = kv = 2048 (causal)
+    rng = wl.rng_for(3, 0)
+    nh, nkv, d = 32, 8, 128
+    q, k, v = wl.make_attention_inputs(rng, 2048, 2048, nh, nkv, d)
+    print("full-size prefill", flush=True)
+    out = ctx.run_flash_attn(q, k, v, None, nh, nkv, d, causal=True).astype(np.float32)
+    # (a) rows of softmax sum to one: V = ones gives O = ones
+    ones = ctx.run_flash_attn(q, k, np.ones_like(v), None, nh, nkv, d, causal=True).astype(np.float32)
+    assert np.abs(ones - 1.0).max() <= 2e-3
+    # (b) query 0 sees key 0 only
+    assert np.abs(out[0] - np.repeat(v[0].astype(np.float32), nh // nkv, axis=0)).max() <= 2e-3
+    # (c) decode over the same keys equals the last row of the causal prefill
+    print("full-size decode", flush=True)
+    last = ctx.run_flash_attn(q[-1:], k, v, None, nh, nkv, d, causal=True).astype(np.float32)
+    assert np.abs(last[0] - out[-1]).max() <= 2e-3
+    # (d) decode at kv = 4096: convex combination of values stays inside their range, permuting keys changes nothing
+    q1, k4, v4 = wl.make_attention_inputs(rng, 1, 4096, nh, nkv, d)
+    o1 = ctx.run_flash_attn(q1, k4, v4, None, nh, nkv, d, causal=True).astype(np.float32)
+    perm = rng.permutation(4096)
+    o2 = ctx.run_flash_attn(q1, k4[perm], v4[perm], None, nh, nkv, d, causal=True).astype(np.float32)
+    assert np.abs(o1 - o2).max() <= 2e-3
+    vmax = np.repeat(np.abs(v4.astype(np.float32)).max(axis=0), nh // nkv, axis=0)
+    assert np.all(np.abs(o1[0]) <= vmax + 1e-3)
+
+
+def test_rejections(ctx):
+    q, k = ctx.alloc(8 * 128 * 4), ctx.alloc(64 * 3 * 128 * 2)
+    R = api.HTPOPS_ERR_REJECTED
+    p = api.flash_attn_params((q, 0), (q, 0), (k, 0), (k, 0), (-1, 0), 1, 64, 8, 3, 128)
+    assert ctx.execute(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16, p) == R     # n_heads % n_kv_heads
+    p = api.flash_attn_params((q, 0), (q, 0), (k, 0), (k, 0), (-1, 0), 1, 64, 4, 2, 96)
+    assert ctx.execute(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16, p) == R     # head_dim not built
+    p = api.flash_attn_params((q, 0), (q, 0), (k, 0), (k, 0), (-1, 0), 1, 4096, 8, 2, 128)
+    assert ctx.execute(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16, p) == R     # K/V buffer too small
+    ctx.release(q), ctx.release(k)
