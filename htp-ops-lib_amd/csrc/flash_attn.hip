@@ -271,7 +271,24 @@ constexpr int kDecThreads  = 256;
 constexpr int kDecMaxGroup = 8;   // query heads scored per pass against one K/V stream
 constexpr int kDecSplit    = 128; // keys per workgroup
 
-// partial record per (head, split): m, l, then D floats of un-normalised O
+// sum over the 16 (or 8) consecutive lanes of a key group with DPP row operations; every lane gets the sum
+template <int LPK>
+__device__ __forceinline__ float key_group_sum(float v) {
+#define HTPOPS_DPP_ADD(ctrl) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, 0xf, 0xf, false))
+  HTPOPS_DPP_ADD(0xB1);   // quad_perm [1,0,3,2]
+  HTPOPS_DPP_ADD(0x4E);   // quad_perm [2,3,0,1]
+  HTPOPS_DPP_ADD(0x141);  // row_half_mirror: 8 lanes
+  if (LPK == 16) {
+    HTPOPS_DPP_ADD(0x140);  // row_mirror: 16 lanes
+  }
+#undef HTPOPS_DPP_ADD
+  return v;
+}
+
+// partial record per (head, split): m, l, then D floats of un-normalised O.
+// A workgroup owns kDecSplit consecutive keys of one KV head. LPK = D / 8 lanes share a key (16 bytes of K and of
+// V each); every K and V load of the wave is issued before the first use, the scores of all GH heads are formed
+// against the same registers, and the per-slot (max, sum, O) partials are merged through LDS.
 template <int D, int GH, bool QO_F32>
 __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *__restrict__ part,
                                                                         const void *__restrict__ q_ptr,
@@ -280,10 +297,12 @@ __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *_
                                                                         const _Float16 *__restrict__ mask, int kv_len,
                                                                         int n_heads, int n_kv_heads, int head0_in_group,
                                                                         int n_splits) {
-  constexpr int LPK = D / 8;        // lanes per key (8 halfs = 16 bytes each)
-  constexpr int KPW = kWave / LPK;  // keys per wave per pass
-  constexpr int WAVES = kDecThreads / kWave;
-  __shared__ float red_m[WAVES][GH], red_l[WAVES][GH], red_o[WAVES][GH][D];
+  constexpr int LPK    = D / 8;        // lanes per key (8 halfs = 16 bytes each)
+  constexpr int KPW    = kWave / LPK;  // keys per wave per pass
+  constexpr int WAVES  = kDecThreads / kWave;
+  constexpr int SLOTS  = WAVES * KPW;  // independent partial streams in the workgroup
+  constexpr int PASSES = kDecSplit / SLOTS;
+  __shared__ float red_m[SLOTS][GH], red_l[SLOTS][GH], red_o[SLOTS][GH][D];
 
   const int group = n_heads / n_kv_heads;
   const int h_kv  = blockIdx.y;
@@ -291,14 +310,28 @@ __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *_
   const int lane  = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int sub   = lane % LPK;  // which 8 dims
   const int kslot = lane / LPK;  // which key of the pass
+  const int slot  = wave * KPW + kslot;
   const float scale = (1.0f / sqrtf((float) D)) * kLog2e;
   const size_t kv_stride = (size_t) n_kv_heads * D;
+
+  const int k_begin = split * kDecSplit;
+  const int k_end   = min(kv_len, k_begin + kDecSplit);
+
+  // all K and V of this lane, requested up front (keys of a pass are consecutive across slots)
+  v8h kreg[PASSES], vreg[PASSES];
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    const int    key = min(k_begin + p * SLOTS + slot, k_end - 1);
+    const size_t off = (size_t) key * kv_stride + (size_t) h_kv * D + sub * 8;
+    kreg[p]          = *reinterpret_cast<const v8h *>(k_ptr + off);
+    vreg[p]          = *reinterpret_cast<const v8h *>(v_ptr + off);
+  }
 
   // q for the GH heads, this lane's 8 dims, pre-scaled
   float q[GH][8];
 #pragma unroll
   for (int g = 0; g < GH; ++g) {
-    const int hg = min(head0_in_group + g, group - 1);
+    const int    hg   = min(head0_in_group + g, group - 1);
     const size_t base = (size_t) (h_kv * group + hg) * D + sub * 8;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
@@ -308,80 +341,54 @@ __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *_
     }
   }
 
-  float m_run[GH], l_run[GH], o[GH][8];
+  float sc[PASSES][GH];
+  float m_loc[GH];
 #pragma unroll
   for (int g = 0; g < GH; ++g) {
-    m_run[g] = -INFINITY, l_run[g] = 0.0f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      o[g][e] = 0.0f;
-    }
+    m_loc[g] = -INFINITY;
   }
-
-  const int k_begin = split * kDecSplit;
-  const int k_end   = min(kv_len, k_begin + kDecSplit);
-  for (int kb = k_begin + wave * KPW; kb < k_end; kb += WAVES * KPW) {
-    const int  key  = kb + kslot;
-    const bool live = key < k_end;
-    const int  kc   = live ? key : k_end - 1;
-    const v8h  kv8  = *reinterpret_cast<const v8h *>(k_ptr + (size_t) kc * kv_stride + (size_t) h_kv * D + sub * 8);
-    const v8h  vv8  = *reinterpret_cast<const v8h *>(v_ptr + (size_t) kc * kv_stride + (size_t) h_kv * D + sub * 8);
-    float kf[8], vf[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      kf[e] = (float) kv8[e], vf[e] = (float) vv8[e];
-    }
-    const float mk = (mask && live) ? (float) mask[key] : 0.0f;  // row 0 of the mask (qo_len == 1)
+  for (int p = 0; p < PASSES; ++p) {
+    const int  key  = k_begin + p * SLOTS + slot;
+    const bool live = key < k_end;
+    const float mk  = (mask && live) ? (float) mask[key] : 0.0f;  // row 0 of the mask (qo_len == 1)
 #pragma unroll
     for (int g = 0; g < GH; ++g) {
       float s = 0.0f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        s += q[g][e] * kf[e];
+        s += q[g][e] * (float) kreg[p][e];
       }
-      s = group_sum<LPK>(s) + mk;  // every lane of the key's group holds the score
-      s = live ? s : -INFINITY;
-      const float m_new  = fmaxf(m_run[g], s);
-      const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
-      const float alpha  = fast_exp2(m_run[g] - m_safe);
-      const float p      = fast_exp2(s - m_safe);
-      l_run[g]           = l_run[g] * alpha + p;
-      m_run[g]           = m_new;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        o[g][e] = o[g][e] * alpha + p * vf[e];
-      }
+      s        = key_group_sum<LPK>(s) + mk;
+      s        = live ? s : -INFINITY;
+      sc[p][g] = s;
+      m_loc[g] = fmaxf(m_loc[g], s);
     }
   }
-
-  // merge the KPW key slots of the wave (lanes with equal `sub`), then the waves, then write the partial
+  float o[GH][8], l_loc[GH];
 #pragma unroll
   for (int g = 0; g < GH; ++g) {
-    float m_all = m_run[g];
+    const float m_safe = (m_loc[g] == -INFINITY) ? 0.0f : m_loc[g];
+    l_loc[g]           = 0.0f;
 #pragma unroll
-    for (int off = LPK; off < kWave; off <<= 1) {
-      m_all = fmaxf(m_all, __shfl_xor(m_all, off, kWave));
+    for (int e = 0; e < 8; ++e) {
+      o[g][e] = 0.0f;
     }
-    const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
-    const float f      = fast_exp2(m_run[g] - m_safe);
-    float       l      = l_run[g] * f;
 #pragma unroll
-    for (int off = LPK; off < kWave; off <<= 1) {
-      l += __shfl_xor(l, off, kWave);
+    for (int p = 0; p < PASSES; ++p) {
+      const float pr = fast_exp2(sc[p][g] - m_safe);
+      l_loc[g] += pr;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        o[g][e] += pr * (float) vreg[p][e];
+      }
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      float v = o[g][e] * f;
-#pragma unroll
-      for (int off = LPK; off < kWave; off <<= 1) {
-        v += __shfl_xor(v, off, kWave);
-      }
-      if (kslot == 0) {
-        red_o[wave][g][sub * 8 + e] = v;
-      }
+      red_o[slot][g][sub * 8 + e] = o[g][e];
     }
-    if (lane == 0) {
-      red_m[wave][g] = m_all, red_l[wave][g] = l;
+    if (sub == 0) {
+      red_m[slot][g] = m_loc[g], red_l[slot][g] = l_loc[g];
     }
   }
   __syncthreads();
@@ -392,19 +399,19 @@ __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *_
     }
     float m_all = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
+    for (int w = 0; w < SLOTS; ++w) {
       m_all = fmaxf(m_all, red_m[w][g]);
     }
     const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
     float       l = 0.0f, v = 0.0f;
 #pragma unroll
-    for (int w = 0; w < WAVES; ++w) {
+    for (int w = 0; w < SLOTS; ++w) {
       const float f = fast_exp2(red_m[w][g] - m_safe);
       l += red_l[w][g] * f;
       v += red_o[w][g][d] * f;
     }
-    const int    head = h_kv * group + head0_in_group + g;
-    float       *rec  = part + ((size_t) head * n_splits + split) * (D + 2);
+    const int head = h_kv * group + head0_in_group + g;
+    float    *rec  = part + ((size_t) head * n_splits + split) * (D + 2);
     if (d == 0) {
       rec[0] = m_all, rec[1] = l;
     }
@@ -415,19 +422,65 @@ __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *_
 template <int D, bool QO_F32>
 __global__ __launch_bounds__(D) void flash_attn_decode_merge_kernel(void *__restrict__ o_ptr,
                                                                     const float *__restrict__ part, int n_splits) {
+  // phase 1: the (max, sum) heads of all splits are fetched in parallel and turned into rescale factors in LDS;
+  // phase 2: every thread sums its column with independent loads.
+  extern __shared__ float merge_f[];  // [n_splits] factors, then [1] total
+  __shared__ float        merge_red[2][D / kWave > 0 ? D / kWave : 1];
   const int    head = blockIdx.x, d = threadIdx.x;
   const float *rec0 = part + (size_t) head * n_splits * (D + 2);
-  float        m_all = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) {
-    m_all = fmaxf(m_all, rec0[(size_t) s * (D + 2)]);
+  float        m_loc = -INFINITY;
+  for (int s = d; s < n_splits; s += D) {
+    m_loc = fmaxf(m_loc, rec0[(size_t) s * (D + 2)]);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    m_loc = fmaxf(m_loc, __shfl_xor(m_loc, off));
+  }
+  if ((d & 63) == 0) {
+    merge_red[0][d >> 6] = m_loc;
+  }
+  __syncthreads();
+  float m_all = merge_red[0][0];
+#pragma unroll
+  for (int w = 1; w < D / kWave; ++w) {
+    m_all = fmaxf(m_all, merge_red[0][w]);
   }
   const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
-  float       l = 0.0f, v = 0.0f;
-  for (int s = 0; s < n_splits; ++s) {
+  float       l_loc  = 0.0f;
+  for (int s = d; s < n_splits; s += D) {
     const float *rec = rec0 + (size_t) s * (D + 2);
     const float  f   = fast_exp2(rec[0] - m_safe);
-    l += rec[1] * f;
-    v += rec[2 + d] * f;
+    merge_f[s]       = f;
+    l_loc += rec[1] * f;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    l_loc += __shfl_xor(l_loc, off);
+  }
+  if ((d & 63) == 0) {
+    merge_red[1][d >> 6] = l_loc;
+  }
+  __syncthreads();
+  float l = 0.0f;
+#pragma unroll
+  for (int w = 0; w < D / kWave; ++w) {
+    l += merge_red[1][w];
+  }
+  float v = 0.0f;
+  int   s = 0;
+  for (; s + 8 <= n_splits; s += 8) {
+    float x[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      x[u] = rec0[(size_t) (s + u) * (D + 2) + 2 + d];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      v += x[u] * merge_f[s + u];
+    }
+  }
+  for (; s < n_splits; ++s) {
+    v += rec0[(size_t) s * (D + 2) + 2 + d] * merge_f[s];
   }
   const float out = v * (1.0f / l);
   if (QO_F32) {
@@ -476,8 +529,8 @@ hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void 
     }
 #undef HTPOPS_DECODE
   }
-  hipLaunchKernelGGL((flash_attn_decode_merge_kernel<D, QO_F32>), dim3((unsigned) n_heads), dim3(D), 0, stream, o,
-                     workspace, n_splits);
+  hipLaunchKernelGGL((flash_attn_decode_merge_kernel<D, QO_F32>), dim3((unsigned) n_heads), dim3(D),
+                     (size_t) n_splits * sizeof(float), stream, o, workspace, n_splits);
   return hipGetLastError();
 }
 

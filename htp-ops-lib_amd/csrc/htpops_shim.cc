@@ -288,8 +288,11 @@ int op_mat_mul_q8(htpops_context *ctx, float *dst, const void *act, const void *
   if (int r = need_device(ctx)) {
     return r;
   }
+  if (int r = ensure_workspace(ctx, htpops::mat_mul_workspace_bytes(m, k))) {
+    return r;
+  }
   HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, act, weight, m, k, n,
-                                                  (htpops::WeightType) weight_type));
+                                                  (htpops::WeightType) weight_type, ctx->workspace));
   return HTPOPS_OK;
 }
 
@@ -304,12 +307,15 @@ int op_mat_mul_f32(htpops_context *ctx, float *dst, const float *act, const void
   if (int r = need_device(ctx)) {
     return r;
   }
-  if (int r = ensure_workspace(ctx, q8_0_bytes((size_t) m, (size_t) k))) {
+  // workspace: [quantized activations][what the matmul kernels need]
+  const size_t q_bytes = (q8_0_bytes((size_t) m, (size_t) k) + 255) & ~(size_t) 255;
+  if (int r = ensure_workspace(ctx, q_bytes + htpops::mat_mul_workspace_bytes(m, k))) {
     return r;
   }
-  HTPOPS_HIP(ctx, htpops::launch_quantize_q8_0(ctx->stream, ctx->workspace, act, k, m));
-  HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, ctx->workspace, weight, m, k, n,
-                                                  (htpops::WeightType) weight_type));
+  uint8_t *ws = static_cast<uint8_t *>(ctx->workspace);
+  HTPOPS_HIP(ctx, htpops::launch_quantize_q8_0(ctx->stream, ws, act, k, m));
+  HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, ws, weight, m, k, n,
+                                                  (htpops::WeightType) weight_type, ws + q_bytes));
   return HTPOPS_OK;
 }
 

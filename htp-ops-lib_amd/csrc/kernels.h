@@ -24,12 +24,15 @@ hipError_t launch_rms_norm_quantize_q8_0(hipStream_t stream, void *dst, const fl
 // decode path: one pass over the weight bytes per activation row
 hipError_t launch_gemv_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
                                 int n, WeightType wt);
-// prefill path: int8 MFMA over LDS-staged tiles; needs k % 32 == 0
+// prefill path: MFMA over LDS-staged tiles; needs k % 64 == 0 (else hipErrorNotSupported). `workspace` (size from
+// gemm_workspace_bytes, may be null) holds the converted activations of the large-m kernel.
+size_t     gemm_workspace_bytes(int m, int k);
 hipError_t launch_gemm_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
-                                int n, WeightType wt);
+                                int n, WeightType wt, void *workspace);
 // picks between the two by m
+size_t     mat_mul_workspace_bytes(int m, int k);
 hipError_t launch_mat_mul_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
-                                   int n, WeightType wt);
+                                   int n, WeightType wt, void *workspace);
 
 // attention; see htpops_flash_attn_ptr. `workspace` holds split-KV partials (decode), size from
 // flash_attn_workspace_bytes.
