@@ -29,7 +29,8 @@ struct Buffer {
   bool   live  = false;
 };
 
-constexpr int kMaxHandles = 1 << 20;
+constexpr int kMaxHandles  = 1 << 20;
+constexpr int kTicketSlots = 1 << 16;
 
 }  // namespace
 
@@ -44,6 +45,8 @@ struct htpops_context {
   // scratch owned by the context: quantized activations of the fp32-activation matmul, attention partials
   void  *workspace       = nullptr;
   size_t workspace_bytes = 0;
+  // zeroed ticket counters of the K-sliced matmul (each launch leaves them zeroed)
+  unsigned *tickets = nullptr;
 
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
 
@@ -288,11 +291,12 @@ int op_mat_mul_q8(htpops_context *ctx, float *dst, const void *act, const void *
   if (int r = need_device(ctx)) {
     return r;
   }
-  if (int r = ensure_workspace(ctx, htpops::mat_mul_workspace_bytes(m, k))) {
+  if (int r = ensure_workspace(ctx, htpops::mat_mul_workspace_bytes(m, k, n))) {
     return r;
   }
   HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, act, weight, m, k, n,
-                                                  (htpops::WeightType) weight_type, ctx->workspace));
+                                                  (htpops::WeightType) weight_type, ctx->workspace, ctx->tickets,
+                                                  kTicketSlots));
   return HTPOPS_OK;
 }
 
@@ -309,13 +313,14 @@ int op_mat_mul_f32(htpops_context *ctx, float *dst, const float *act, const void
   }
   // workspace: [quantized activations][what the matmul kernels need]
   const size_t q_bytes = (q8_0_bytes((size_t) m, (size_t) k) + 255) & ~(size_t) 255;
-  if (int r = ensure_workspace(ctx, q_bytes + htpops::mat_mul_workspace_bytes(m, k))) {
+  if (int r = ensure_workspace(ctx, q_bytes + htpops::mat_mul_workspace_bytes(m, k, n))) {
     return r;
   }
   uint8_t *ws = static_cast<uint8_t *>(ctx->workspace);
   HTPOPS_HIP(ctx, htpops::launch_quantize_q8_0(ctx->stream, ws, act, k, m));
   HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, ws, weight, m, k, n,
-                                                  (htpops::WeightType) weight_type, ws + q_bytes));
+                                                  (htpops::WeightType) weight_type, ws + q_bytes, ctx->tickets,
+                                                  kTicketSlots));
   return HTPOPS_OK;
 }
 
@@ -372,7 +377,9 @@ extern "C" int htpops_init_backend(htpops_context **out_ctx, int device) {
       return HTPOPS_ERR_NO_DEVICE;
     }
     if (hipSetDevice(device) != hipSuccess || hipStreamCreate(&ctx->stream) != hipSuccess ||
-        hipEventCreate(&ctx->ev_start) != hipSuccess || hipEventCreate(&ctx->ev_stop) != hipSuccess) {
+        hipEventCreate(&ctx->ev_start) != hipSuccess || hipEventCreate(&ctx->ev_stop) != hipSuccess ||
+        hipMalloc(reinterpret_cast<void **>(&ctx->tickets), kTicketSlots * sizeof(unsigned)) != hipSuccess ||
+        hipMemset(ctx->tickets, 0, kTicketSlots * sizeof(unsigned)) != hipSuccess) {
       delete ctx;
       return HTPOPS_ERR_HIP;
     }
@@ -403,6 +410,9 @@ extern "C" int htpops_close(htpops_context *ctx) {
     }
   }
   if (ctx->has_device) {
+    if (ctx->tickets) {
+      (void) hipFree(ctx->tickets);
+    }
     if (ctx->workspace) {
       (void) hipFree(ctx->workspace);
     }

@@ -24,15 +24,22 @@ hipError_t launch_rms_norm_quantize_q8_0(hipStream_t stream, void *dst, const fl
 // decode path: one pass over the weight bytes per activation row
 hipError_t launch_gemv_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
                                 int n, WeightType wt);
+// small-batch path (m <= 32, k % 64 == 0, else hipErrorNotSupported): one pass over the weight bytes for all rows,
+// block dots on v_mfma_i32_32x32x32_i8
+// `workspace` (matmul_skinny_workspace_bytes) holds per-slice partial tiles, `tickets` is an array of
+// `ticket_slots` zeroed counters that the kernel leaves zeroed; without them K is not sliced (slower).
+size_t     matmul_skinny_workspace_bytes(int m, int k, int n);
+hipError_t launch_matmul_skinny(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
+                                int n, WeightType wt, void *workspace, unsigned *tickets, int ticket_slots);
 // prefill path: MFMA over LDS-staged tiles; needs k % 64 == 0 (else hipErrorNotSupported). `workspace` (size from
 // gemm_workspace_bytes, may be null) holds the converted activations of the large-m kernel.
 size_t     gemm_workspace_bytes(int m, int k);
 hipError_t launch_gemm_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
                                 int n, WeightType wt, void *workspace);
 // picks between the two by m
-size_t     mat_mul_workspace_bytes(int m, int k);
+size_t     mat_mul_workspace_bytes(int m, int k, int n);
 hipError_t launch_mat_mul_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
-                                   int n, WeightType wt, void *workspace);
+                                   int n, WeightType wt, void *workspace, unsigned *tickets, int ticket_slots);
 
 // attention; see htpops_flash_attn_ptr. `workspace` holds split-KV partials (decode), size from
 // flash_attn_workspace_bytes.

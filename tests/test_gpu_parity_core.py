@@ -113,7 +113,9 @@ def test_gemv_m1(ctx, oracle, wt, k, n):
 
 
 @pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
-@pytest.mark.parametrize("m,k,n", [(8, 4096, 512), (2, 11008, 96), (3, 1536, 256), (8, 96, 40), (5, 64, 32), (16, 1024, 128)])
+@pytest.mark.parametrize("m,k,n", [(8, 4096, 512), (2, 11008, 96), (3, 1536, 256), (8, 96, 40), (5, 64, 32), (16, 1024, 128),
+                                   (8, 11008, 1024), (8, 4096, 100), (13, 2048, 70), (32, 4096, 64), (31, 11008, 40),
+                                   (40, 1024, 96), (63, 640, 33), (9, 64, 32), (4, 8960, 1536)])
 def test_small_batch(ctx, oracle, wt, m, k, n):
     got, x, w = check_mat_mul(ctx, oracle, wl.rng_for(54, m * 31 + k + n + wt), m, k, n, wt)
     # the fp32-activation op quantizes on the device and must give the same bits
@@ -183,6 +185,42 @@ def test_message_with_a_decode_chain_runs_in_order(ctx, oracle):
     assert np.all(np.abs(got - want64[0]) <= MATMUL_RTOL * mag[0])
     for h in (hx, hn, hq, hw, ho, ones):
         ctx.release(h)
+
+
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+@pytest.mark.parametrize("m", [2, 8, 12, 27])
+def test_small_batch_integer_exact(ctx, wt, m):
+    # scales 1.0, full-range int8 activations: the output is the exact integer matrix product
+    rng = wl.rng_for(58, wt + m)
+    k, n = 640, 77
+    w = wl.make_weights(rng, n, k, wt).reshape(n, k // 32, -1)
+    w[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    w = w.reshape(n, -1)
+    a = np.empty((m, k // 32, 34), np.uint8)
+    a[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    a[:, :, 2:] = rng.integers(-127, 128, (m, k // 32, 32), dtype=np.int8).view(np.uint8)
+    a = a.reshape(m, -1)
+    got = ctx.run_mat_mul(a, w, m, k, n, wt)
+    _, qa = wl.q8_0_split(a, k)
+    _, qw = (wl.q4_0_split if wt == wl.GGML_TYPE_Q4_0 else wl.q8_0_split)(w, k)
+    assert np.array_equal(got, (qa.astype(np.int64) @ qw.astype(np.int64).T).astype(np.float32))
+
+
+def test_small_batch_repeated_launches_are_bit_identical(ctx):
+    # K is cut into slices that are summed in a fixed order by the last workgroup of a row tile: the result must not
+    # depend on which workgroup that is, and the ticket counters must come back to zero after every launch
+    rng = wl.rng_for(59, 0)
+    m, k, n = 8, 11008, 2048
+    w = wl.make_q4_0_weights(rng, n, k)
+    a = wl.quantize_q8_0_numpy(wl.make_activations(rng, m, k)) if hasattr(wl, "quantize_q8_0_numpy") else \
+        ctx.run_quantize_q8_0(wl.make_activations(rng, m, k))
+    first = ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
+    for _ in range(5):
+        assert np.array_equal(ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0), first)
+    # every row agrees with the one-row kernel
+    for r in (0, 3, 7):
+        one = ctx.run_mat_mul(a[r:r + 1], w, 1, k, n, wl.GGML_TYPE_Q4_0)
+        assert np.abs(one[0] - first[r]).max() <= 2e-5 * np.abs(one).max()
 
 
 # --------------------------------------------------------------------------------- prefill (MFMA) path
