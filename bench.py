@@ -3,16 +3,19 @@
 
 A step is one Llama-7B decoder layer's seven Q4_0 x Q8_0 matrix-vector products at m = 1 (q/k/v/o 4096x4096,
 gate/up 11008x4096, down 4096x11008), submitted as ONE mailbox message (seven OP_COMPUTE requests) and executed
-back-to-back on the context's stream. Weights of LAYERS distinct layers are resident in HBM and steps rotate
+back-to-back on the context's stream; requests that read the same activation buffer (q/k/v, gate/up) share a launch. Weights of LAYERS distinct layers are resident in HBM and steps rotate
 through them (LAYERS x 113.8 MB > the 256 MB memory-side cache), so every step streams its weights from HBM.
 `value` is algorithmic bytes per step / time per step (weights once, Q8_0 activations once, fp32 outputs once).
 
 The same run also measures, and reports inside the JSON line:
-  roofline      the headline shape alone (down-proj GEMV, n = 4096, k = 11008): bytes per launch / average launch
-                duration from HIP events on the launching stream, against 8 TB/s
+  roofline      the launch that takes the largest share of the step (gate + up, 2 x 11008 x 4096 in one launch):
+                algorithmic bytes per launch / average launch duration from HIP events on the launching stream,
+                against 8 TB/s
   prefill_gemm  m = 512 Q4_0 GEMM, both shapes of config 2, in int8 Tera-ops/s (2 m n k per launch)
   small_batch   the same layer at m = 8
   q8_0_block    the Qwen2-1.5B-like Q8_0 block of config 4 at m = 1
+  attention     config 3: decode (1 x 4096) and causal prefill (2048 x 2048), 32 query / 8 KV heads of 128, fp16
+  launches      the four kernel launches of the step one by one (q+k+v, o, gate+up, down) on cold weights
   cpu_baseline  the scalar C oracle (a port of the same arithmetic) on the host cores, same layer, m = 1
   peaks         MFMA-only loops and a plain copy kernel measured on this device
 Every GPU result used for timing is first checked against the oracle on a sample of rows.
@@ -39,6 +42,18 @@ Q4, Q8 = 2, 8
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
+
+
+def measured_traffic(launch):
+    """HBM-side bytes per launch of the named launch, from hardware counters collected in separate profiler passes
+    over this script (FETCH_SIZE and WRITE_SIZE, each scaled by the same counter's reading for the plain copy
+    kernel of known size); the figures live beside the package because counters cannot be read from inside a run."""
+    path = os.path.join(ROOT, "htp-ops-lib_amd", "pyhtpops", "measured_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f)["launches"][launch]["traffic_bytes"]
+    except (OSError, KeyError, ValueError):
+        return None
 
 
 def main():
@@ -68,14 +83,18 @@ def main():
     for _, n, k in shapes:
         if (n, k) not in uniq:
             uniq[(n, k)] = wl.make_q4_0_weights(rng, n, k)
-    acts, act_q, h_act = {}, {}, {}
+    # The data flow of a decoder layer decides which requests may share a launch: q/k/v read the normed hidden
+    # state, o reads the attention output, gate/up read the second normed hidden state, down reads the gated product.
+    # Four distinct activation buffers reproduce that (requests on different buffers are never batched together).
+    ACT_OF = {"q": 0, "k": 0, "v": 0, "o": 1, "gate": 2, "up": 2, "down": 3}
+    ACT_K = {0: 4096, 1: 4096, 2: 4096, 3: 11008}
+    act_q, h_act = {}, {}
     for m in (1, 8):
-        for k in (4096, 11008):
+        for g, k in ACT_K.items():
             x = wl.make_activations(rng, m, k)
-            acts[(m, k)] = x
-            act_q[(m, k)] = ctx.run_quantize_q8_0(x)                       # quantized on the GPU ...
-            assert np.array_equal(act_q[(m, k)], orc.quantize_q8_0(x)), "Q8_0 quantizer is not bit-exact"  # ... bit-exact
-            h_act[(m, k)] = ctx.upload(act_q[(m, k)])
+            act_q[(m, g)] = ctx.run_quantize_q8_0(x)                       # quantized on the GPU ...
+            assert np.array_equal(act_q[(m, g)], orc.quantize_q8_0(x)), "Q8_0 quantizer is not bit-exact"  # ... bit-exact
+            h_act[(m, g)] = ctx.upload(act_q[(m, g)])
     layers = []
     for _ in range(LAYERS):
         layers.append([ctx.upload(uniq[(n, k)]) for _, n, k in shapes])
@@ -85,9 +104,9 @@ def main():
 
     def layer_message(layer, m):
         reqs = []
-        for i, (_, n, k) in enumerate(shapes):
+        for i, (name, n, k) in enumerate(shapes):
             body = api.op_compute_request(api.HTP_OPS_MAT_MUL_Q4_0_Q8_0,
-                                          api.mat_mul_params((h_out[m][i], 0), (h_act[(m, k)], 0), (layers[layer][i], 0), m, k, n))
+                                          api.mat_mul_params((h_out[m][i], 0), (h_act[(m, ACT_OF[name])], 0), (layers[layer][i], 0), m, k, n))
             reqs.append((api.REQUEST_TYPE_OP_COMPUTE, body))
         return api.build_message(reqs)
 
@@ -102,10 +121,10 @@ def main():
         assert ctx.process_message(msg) == 0
         check_states(msg)
         worst = 0.0
-        for i, (_, n, k) in enumerate(shapes):
+        for i, (name, n, k) in enumerate(shapes):
             got = ctx.read(h_out[m][i], np.float32, m * n).reshape(m, n)
             rows = np.unique(np.linspace(0, n - 1, 96).astype(int))
-            want, mag = orc.mat_mul_q8_0_act_f64(act_q[(m, k)], uniq[(n, k)][rows], m, k, len(rows), Q4)
+            want, mag = orc.mat_mul_q8_0_act_f64(act_q[(m, ACT_OF[name])], uniq[(n, k)][rows], m, k, len(rows), Q4)
             err = np.abs(got[:, rows] - want) / mag
             worst = max(worst, float(err.max()))
             assert np.all(err <= 1e-5), "matmul %d outside 1e-5 relative: %g" % (i, err.max())
@@ -138,7 +157,7 @@ def main():
     value = layer_bytes[1] / (ms_step * 1e-3) / 1e9
     log("layer m=1: %.2f us/step (events) %.2f us/step (wall)  %.0f GB/s" % (ms_step * 1e3, wall_step * 1e3, value))
 
-    # ------------------------------------------------------------------ headline shape alone (roofline)
+    # ------------------------------------------------------------------ the step's four launches, one by one
     def time_single(n, k, m, wt, handles, h_a, h_o, reps, op):
         reqs = [(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, api.mat_mul_params((h_o, 0), (h_a, 0), (h, 0), m, k, n)))
                 for h in handles]
@@ -152,16 +171,39 @@ def main():
         check_states(msg)
         return ms * 1e3 / (reps * len(handles))  # us per launch
 
-    down = [layers[l][6] for l in range(LAYERS)]
-    extra_down = [ctx.upload(uniq[(4096, 11008)]) for _ in range(8)]  # 16 x 25.4 MB = 406 MB of distinct buffers
-    us_down = time_single(4096, 11008, 1, Q4, down + extra_down, h_act[(1, 11008)], h_out[1][6], 30, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)
-    us_down_hot = time_single(4096, 11008, 1, Q4, down[:1] * 16, h_act[(1, 11008)], h_out[1][6], 30, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)
-    bytes_down = wl.matmul_algorithmic_bytes(1, 11008, 4096, Q4)
-    gbps_down = bytes_down / us_down / 1e3
-    log("down-proj GEMV 4096x11008: %.2f us cold (%.0f GB/s, %.1f%% of 8 TB/s); %.2f us cache-resident" % (
-        us_down, gbps_down, gbps_down / 80, us_down_hot))
-    for h in extra_down:
-        ctx.release(h)
+    def time_launch(names, reps=40):
+        """One message = this launch (the requests `names` of a layer, which share an activation buffer) for every
+        resident layer in turn: LAYERS back-to-back launches on cold weights; HIP events on the launching stream."""
+        reqs = []
+        for l in range(LAYERS):
+            for i, (name, n, k) in enumerate(shapes):
+                if name in names:
+                    reqs.append((api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
+                        api.HTP_OPS_MAT_MUL_Q4_0_Q8_0,
+                        api.mat_mul_params((h_out[1][i], 0), (h_act[(1, ACT_OF[name])], 0), (layers[l][i], 0), 1, k, n))))
+        msg = api.build_message(reqs)
+        for _ in range(3):
+            ctx.enqueue_message(msg)
+        ctx.synchronize()
+        ctx.timer_start()
+        for _ in range(reps):
+            ctx.enqueue_message(msg)
+        ms = ctx.timer_stop_ms()
+        ctx.finish_message(msg)
+        check_states(msg)
+        us = ms * 1e3 / (reps * LAYERS)
+        nbytes = sum(wl.matmul_algorithmic_bytes(1, k, n, Q4) for name, n, k in shapes if name in names)
+        return {"launch": "+".join(names), "us_per_launch": round(us, 3), "bytes_per_launch": nbytes,
+                "GBps": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+
+    launches = [time_launch(("q", "k", "v")), time_launch(("o",)), time_launch(("gate", "up")), time_launch(("down",))]
+    for r in launches:
+        log("launch %-8s %.2f us  %.0f GB/s (%.1f%% of 8 TB/s)" % (r["launch"], r["us_per_launch"], r["GBps"],
+                                                                  r["frac_of_hbm_peak"] * 100))
+    dominant = max(launches, key=lambda r: r["us_per_launch"])  # gate+up: the largest share of the step
+    # the same weights again and again: served by the 256 MB memory-side cache, not by HBM
+    us_hot = time_single(11008, 4096, 1, Q4, [layers[0][4]] * 16, h_act[(1, 2)], h_out[1][4], 30, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)
+    log("gate GEMV 11008x4096 on cache-resident weights: %.2f us" % us_hot)
 
     # ------------------------------------------------------------------ m = 8
     ms_step8, _ = time_layers(8, max(20, args.steps // 4), 5)
@@ -190,25 +232,79 @@ def main():
         ctx.release(ha), ctx.release(ho)
 
     # ------------------------------------------------------------------ Q8_0 block (config 4), m = 1
+    # same protocol as the headline step: one message per layer, 8 layers of distinct weights (8 x 49.7 MB) rotated
     rng4 = wl.rng_for(4, 0)
-    q8_bytes, q8_us = 0, 0.0
-    for name, n, k in wl.QWEN2_1P5B_LAYER:
-        if name in ("k", "o", "up"):
-            continue  # same shapes as q, v, gate: measured once, counted twice below
-        w8 = wl.make_q8_0_weights(rng4, n, k)
-        copies = [ctx.upload(w8) for _ in range(max(2, int(300e6 // w8.nbytes)))]
-        aq = ctx.run_quantize_q8_0(wl.make_activations(rng4, 1, k))
-        ha, ho = ctx.upload(aq), ctx.alloc(n * 4)
-        us = time_single(n, k, 1, Q8, copies, ha, ho, 5, api.HTP_OPS_MAT_MUL_Q8_0_Q8_0)
-        got = ctx.read(ho, np.float32, n)
-        want, mag = orc.mat_mul_q8_0_act_f64(aq, w8[:64], 1, k, 64, Q8)
-        assert np.all(np.abs(got[:64] - want[0]) <= 1e-5 * mag[0])
-        mult = 2 if name in ("q", "v", "gate") else 1
-        q8_bytes += mult * wl.matmul_algorithmic_bytes(1, k, n, Q8)
-        q8_us += mult * us
-        for h in copies + [ha, ho]:
+    shapes8 = wl.QWEN2_1P5B_LAYER
+    uniq8 = {}
+    for _, n, k in shapes8:
+        if (n, k) not in uniq8:
+            uniq8[(n, k)] = wl.make_q8_0_weights(rng4, n, k)
+    act8 = {g: ctx.run_quantize_q8_0(wl.make_activations(rng4, 1, k)) for g, k in {0: 1536, 1: 1536, 2: 1536, 3: 8960}.items()}
+    h_act8 = {g: ctx.upload(a) for g, a in act8.items()}
+    layers8 = [[ctx.upload(uniq8[(n, k)]) for _, n, k in shapes8] for _ in range(LAYERS)]
+    h_out8 = [ctx.alloc(n * 4) for _, n, _ in shapes8]
+    msgs8 = [api.build_message([(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
+        api.HTP_OPS_MAT_MUL_Q8_0_Q8_0,
+        api.mat_mul_params((h_out8[i], 0), (h_act8[ACT_OF[name]], 0), (layers8[l][i], 0), 1, k, n)))
+        for i, (name, n, k) in enumerate(shapes8)]) for l in range(LAYERS)]
+    assert ctx.process_message(msgs8[0]) == 0
+    check_states(msgs8[0])
+    for i, (name, n, k) in enumerate(shapes8):
+        got = ctx.read(h_out8[i], np.float32, n)
+        rows = np.unique(np.linspace(0, n - 1, 64).astype(int))
+        want, mag = orc.mat_mul_q8_0_act_f64(act8[ACT_OF[name]], uniq8[(n, k)][rows], 1, k, len(rows), Q8)
+        assert np.all(np.abs(got[rows] - want[0]) <= 1e-5 * mag[0]), "Q8_0 matmul %s outside 1e-5 relative" % name
+    for s_ in range(20):
+        ctx.enqueue_message(msgs8[s_ % LAYERS])
+    ctx.synchronize()
+    ctx.timer_start()
+    for s_ in range(200):
+        ctx.enqueue_message(msgs8[s_ % LAYERS])
+    q8_us = ctx.timer_stop_ms() * 1e3 / 200
+    for msg in msgs8:
+        ctx.finish_message(msg)
+        check_states(msg)
+    q8_bytes = sum(wl.matmul_algorithmic_bytes(1, k, n, Q8) for _, n, k in shapes8)
+    log("Q8_0 block m=1: %.1f us/step (7 GEMVs in 4 launches), %.0f GB/s" % (q8_us, q8_bytes / q8_us / 1e3))
+    for h in [h for l in layers8 for h in l] + h_out8 + list(h_act8.values()):
+        ctx.release(h)
+
+    # ------------------------------------------------------------------ attention (config 3): 32 query / 8 KV heads, D = 128
+    rng3 = wl.rng_for(3, 0)
+    nh, nkv, hd = 32, 8, 128
+    attention = []
+    for qo, kv, copies, reps in ((1, 4096, 24, 10), (2048, 2048, 1, 10)):
+        q, kk, vv = wl.make_attention_inputs(rng3, qo, kv, nh, nkv, hd)
+        hq, ho = ctx.upload(q), ctx.alloc(q.nbytes)
+        hks, hvs = [ctx.upload(kk) for _ in range(copies)], [ctx.upload(vv) for _ in range(copies)]  # 24 x 16.8 MB: cold
+        reqs = [(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
+            api.HTP_OPS_FLASH_ATTN_F16, api.flash_attn_params((ho, 0), (hq, 0), (hk, 0), (hv, 0), (-1, 0), qo, kv, nh, nkv, hd, causal=True)))
+                for hk, hv in zip(hks, hvs)]
+        msg = api.build_message(reqs * reps)
+        ctx.process_message(msg)
+        ctx.timer_start()
+        ctx.process_message(msg)
+        us = ctx.timer_stop_ms() * 1e3 / (copies * reps)
+        check_states(msg)
+        got = ctx.read(ho, np.float16, qo * nh * hd).reshape(qo, nh, hd).astype(np.float64)
+        worst = 0.0
+        for r in sorted({0, qo // 3, qo - 1}):
+            for h in (0, 13, 31):
+                vis = r + (kv - qo) + 1  # causal: keys 0 .. r + kv - qo
+                kh = kk[:vis, h // (nh // nkv)].astype(np.float64)
+                sc = kh @ q[r, h].astype(np.float64) / np.sqrt(hd)
+                pr = np.exp(sc - sc.max())
+                want = (pr / pr.sum()) @ vv[:vis, h // (nh // nkv)].astype(np.float64)
+                worst = max(worst, float(np.abs(got[r, h] - want).max()))
+        assert worst <= 2e-3, "attention outside 2e-3 absolute: %g" % worst
+        kv_bytes = 2 * kv * nkv * hd * 2
+        flops = 4.0 * nh * qo * kv * hd * (0.5 if qo > 1 else 1.0)  # causal: half of the score matrix
+        attention.append({"qo_len": qo, "kv_len": kv, "us": round(us, 2), "kv_GBps": round(kv_bytes / us / 1e3, 1),
+                          "tera_flops_causal": round(flops / us / 1e6, 2), "max_abs_err_vs_f64": worst})
+        log("attention qo=%d kv=%d: %.2f us  KV %.0f GB/s  %.1f TFLOP/s  (max |err| %.1e)" % (
+            qo, kv, us, kv_bytes / us / 1e3, flops / us / 1e6, worst))
+        for h in [hq, ho] + hks + hvs:
             ctx.release(h)
-    log("Q8_0 block m=1: %.1f us for 7 GEMVs, %.0f GB/s" % (q8_us, q8_bytes / q8_us / 1e3))
 
     # ------------------------------------------------------------------ device ceilings
     peaks = {
@@ -231,13 +327,13 @@ def main():
         t0 = time.perf_counter()
         reps = 0
         while time.perf_counter() - t0 < 10.0:
-            for _, n, k in shapes:
-                native.mat_mul_q8_0_act(act_q[(1, k)], uniq[(n, k)], 1, k, n, Q4, n_threads=cores)
+            for name, n, k in shapes:
+                native.mat_mul_q8_0_act(act_q[(1, ACT_OF[name])], uniq[(n, k)], 1, k, n, Q4, n_threads=cores)
             reps += 1
         t_mt = (time.perf_counter() - t0) / reps
         t0 = time.perf_counter()
-        for _, n, k in shapes:
-            native.mat_mul_q8_0_act(act_q[(1, k)], uniq[(n, k)], 1, k, n, Q4, n_threads=1)
+        for name, n, k in shapes:
+            native.mat_mul_q8_0_act(act_q[(1, ACT_OF[name])], uniq[(n, k)], 1, k, n, Q4, n_threads=1)
         t_1 = time.perf_counter() - t0
         cpu = {"value": round(layer_bytes[1] / t_mt / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
                "sample": "the same 7-GEMV layer at m=1 with the scalar C oracle (gcc -O3 -march=native, pthreads over output "
@@ -264,15 +360,17 @@ def main():
                                "%d layers of distinct weights rotated (cold HBM reads)" % LAYERS,
                    "algorithmic_bytes_per_step": layer_bytes[1], "pct_of_hbm_peak": round(value / HBM_PEAK_GBPS * 100, 2),
                    "wall_ms_per_step": round(wall_step, 6)},
-        "roofline": {"bound": "hbm", "achieved": round(gbps_down, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps_down / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "gemv_shared_act_kernel<Q4_0> n=4096 k=11008 m=1", "bytes_per_launch": bytes_down,
-                     "us_per_launch": round(us_down, 3), "us_per_launch_cache_resident": round(us_down_hot, 3)},
+        "roofline": {"bound": "hbm", "achieved": dominant["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": dominant["frac_of_hbm_peak"], "traffic": measured_traffic(dominant["launch"]),
+                     "kernel": "gemv_shared_act_kernel<Q4_0, 64 lanes per row>, grouped launch %s (k=4096, m=1)" % dominant["launch"],
+                     "bytes_per_launch": dominant["bytes_per_launch"], "us_per_launch": dominant["us_per_launch"]},
+        "launches": launches,
         "cpu_baseline": cpu,
         "prefill_gemm": prefill,
         "small_batch": {"m": 8, "us_per_step": round(ms_step8 * 1e3, 2),
                         "GBps": round(layer_bytes[8] / ms_step8 / 1e6, 1)},
-        "q8_0_block": {"m": 1, "us_7_gemvs": round(q8_us, 2), "GBps": round(q8_bytes / q8_us / 1e3, 1)},
+        "attention": attention,
+        "q8_0_block": {"m": 1, "us_per_step": round(q8_us, 2), "GBps": round(q8_bytes / q8_us / 1e3, 1)},
         "peaks": peaks,
     }
     ctx.close()

@@ -296,14 +296,29 @@ __device__ __forceinline__ float group_sum_dpp(float v) {
 // workgroup instead of being fetched by every wave: the texture path then carries (almost) only weight bytes.
 // Weight loads are issued first, the cooperative activation copy second, so the weights are in flight while the
 // workgroup synchronises. Partial sums are reduced with DPP row operations instead of LDS permutes.
+//
+// One launch can serve several weight matrices that share the activation row (the q/k/v or gate/up projections of a
+// decoder layer): blockIdx.y picks the member, whose weight pointer, output pointer and row count come from the
+// argument table.
+struct GemvGroupArgs {
+  const uint32_t *w[kGemvGroupMax];
+  float          *out[kGemvGroupMax];
+  int             n[kGemvGroupMax];
+};
+
 template <int WT, int G, int ITERS, int R, int THREADS>
-__global__ __launch_bounds__(THREADS) void gemv_shared_act_kernel(float *__restrict__ out,
-                                                                  const uint32_t *__restrict__ act,
-                                                                  const uint32_t *__restrict__ w, int n, int pairs) {
+__global__ __launch_bounds__(THREADS) void gemv_shared_act_kernel(GemvGroupArgs grp, const uint32_t *__restrict__ act,
+                                                                  int pairs) {
   extern __shared__ __attribute__((aligned(16))) uint32_t act_lds[];
   constexpr int PD    = Pair<WT>::kDwords;
   constexpr int SLOTS = kWave / G;
   constexpr int WAVES = THREADS / kWave;
+  const int                       n   = grp.n[blockIdx.y];
+  float *__restrict__             out = grp.out[blockIdx.y];
+  const uint32_t *__restrict__    w   = grp.w[blockIdx.y];
+  if ((int) (blockIdx.x * (WAVES * SLOTS * R)) >= n) {
+    return;  // whole workgroup: this member has fewer rows than the widest one
+  }
   const int     lane  = threadIdx.x & (kWave - 1);
   const int     wave  = threadIdx.x / kWave;
   const int     g     = lane % G;
@@ -387,21 +402,25 @@ __global__ __launch_bounds__(THREADS) void gemv_shared_act_kernel(float *__restr
 }
 
 template <int WT, int G, int ITERS, int R, int THREADS>
-hipError_t launch_shared_act_instance(hipStream_t stream, float *out, const uint32_t *act, const uint32_t *w, int n,
+hipError_t launch_shared_act_instance(hipStream_t stream, const GemvGroupArgs &grp, int count, const uint32_t *act,
                                       int pairs) {
   constexpr int rows_per_group = (THREADS / kWave) * (kWave / G) * R;
-  const dim3    grid((unsigned) ((n + rows_per_group - 1) / rows_per_group));
+  int           n_max          = 0;
+  for (int i = 0; i < count; ++i) {
+    n_max = grp.n[i] > n_max ? grp.n[i] : n_max;
+  }
+  const dim3 grid((unsigned) ((n_max + rows_per_group - 1) / rows_per_group), (unsigned) count);
   hipLaunchKernelGGL((gemv_shared_act_kernel<WT, G, ITERS, R, THREADS>), grid, dim3(THREADS),
-                     (size_t) pairs * kActPairDwords * 4, stream, out, act, w, n, pairs);
+                     (size_t) pairs * kActPairDwords * 4, stream, grp, act, pairs);
   return hipGetLastError();
 }
 
 template <int WT, int G, int ITERS>
-hipError_t launch_shared_act(hipStream_t stream, float *out, const uint32_t *act, const uint32_t *w, int n, int pairs,
+hipError_t launch_shared_act(hipStream_t stream, const GemvGroupArgs &grp, int count, const uint32_t *act, int pairs,
                              int r, int threads) {
 #define HTPOPS_CASE(R, T)                                                                         \
   if (r == R && threads == T) {                                                                   \
-    return launch_shared_act_instance<WT, G, ITERS, R, T>(stream, out, act, w, n, pairs);        \
+    return launch_shared_act_instance<WT, G, ITERS, R, T>(stream, grp, count, act, pairs);       \
   }
   HTPOPS_CASE(1, 256)
   HTPOPS_CASE(2, 256)
@@ -473,34 +492,54 @@ hipError_t launch_pairs(hipStream_t stream, float *out, const uint32_t *act, con
   return hipGetLastError();
 }
 
+constexpr int kSharedActMaxPairs = 192;  // longest activation row the shared-activation kernel stages (k = 12288)
+
+bool shared_act_enabled() {
+  static const int use_shared = env_int("HTPOPS_GEMV_SHARED", 1);
+  return use_shared != 0;
+}
+
+// the default kernel for `count` weight matrices that share one activation row of `pairs` <= kSharedActMaxPairs
 template <int WT>
-hipError_t launch_gemv_row(hipStream_t stream, float *out, const uint32_t *act, const uint32_t *w, int n, int pairs) {
+hipError_t launch_gemv_shared(hipStream_t stream, const GemvGroupArgs &grp, int count, const uint32_t *act, int pairs) {
   static const int forced_r       = env_int("HTPOPS_GEMV_ROWS", 0);
   static const int forced_threads = env_int("HTPOPS_GEMV_THREADS", 0);
-  static const int use_shared     = env_int("HTPOPS_GEMV_SHARED", 1);
-  constexpr int    PD             = Pair<WT>::kDwords;
-  if (use_shared && pairs <= 192) {
-    // measured on MI355X: short-lived waves (one row set each) in 256-thread groups stream best
-    int r = 1, threads = 256;
-    if (forced_r) {
-      r = forced_r;
-    }
-    if (forced_threads) {
-      threads = forced_threads;
-    }
-    if (pairs <= 16) {
-      return launch_shared_act<WT, 16, 1>(stream, out, act, w, n, pairs, r, threads);
-    }
-    if (pairs <= 32) {
-      return launch_shared_act<WT, 32, 1>(stream, out, act, w, n, pairs, r, threads);
-    }
-    if (pairs <= 64) {
-      return launch_shared_act<WT, 64, 1>(stream, out, act, w, n, pairs, r, threads);
-    }
-    if (pairs <= 128) {
-      return launch_shared_act<WT, 64, 2>(stream, out, act, w, n, pairs, r, threads);
-    }
-    return launch_shared_act<WT, 64, 3>(stream, out, act, w, n, pairs, r, threads);
+  // measured on MI355X: short-lived waves (one row set each) in 256-thread groups stream best; only very wide
+  // launches of short rows (gate + up of a 7B layer: 22016 rows of 64 pairs) gain from two rows per lane group
+  int total_rows = 0;
+  for (int i = 0; i < count; ++i) {
+    total_rows += grp.n[i];
+  }
+  int r = (pairs <= 64 && total_rows >= 16384) ? 2 : 1, threads = 256;
+  if (forced_r) {
+    r = forced_r;
+  }
+  if (forced_threads) {
+    threads = forced_threads;
+  }
+  if (pairs <= 16) {
+    return launch_shared_act<WT, 16, 1>(stream, grp, count, act, pairs, r, threads);
+  }
+  if (pairs <= 32) {
+    return launch_shared_act<WT, 32, 1>(stream, grp, count, act, pairs, r, threads);
+  }
+  if (pairs <= 64) {
+    return launch_shared_act<WT, 64, 1>(stream, grp, count, act, pairs, r, threads);
+  }
+  if (pairs <= 128) {
+    return launch_shared_act<WT, 64, 2>(stream, grp, count, act, pairs, r, threads);
+  }
+  return launch_shared_act<WT, 64, 3>(stream, grp, count, act, pairs, r, threads);
+}
+
+template <int WT>
+hipError_t launch_gemv_row(hipStream_t stream, float *out, const uint32_t *act, const uint32_t *w, int n, int pairs) {
+  static const int forced_r = env_int("HTPOPS_GEMV_ROWS", 0);
+  constexpr int    PD       = Pair<WT>::kDwords;
+  if (shared_act_enabled() && pairs <= kSharedActMaxPairs) {
+    GemvGroupArgs grp = {};
+    grp.w[0] = w, grp.out[0] = out, grp.n[0] = n;
+    return launch_gemv_shared<WT>(stream, grp, 1, act, pairs);
   }
   // rows in flight per lane group: fewer for long rows (register budget), more for short ones
   auto pick_r = [&](int regs_per_row, int slots) {
@@ -562,6 +601,24 @@ hipError_t launch_gemv_q8_0_act(hipStream_t stream, float *out, const void *act,
     }
   }
   return hipSuccess;
+}
+
+hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *act,
+                                      const void *const *weights, const int *ns, int k, WeightType wt) {
+  const int nblk = k / kQK;
+  if (count < 1 || count > kGemvGroupMax || nblk % 2 != 0 || nblk / 2 > kSharedActMaxPairs || !shared_act_enabled() ||
+      (reinterpret_cast<uintptr_t>(act) & 3) != 0) {
+    return hipErrorNotSupported;
+  }
+  GemvGroupArgs grp = {};
+  for (int i = 0; i < count; ++i) {
+    if ((reinterpret_cast<uintptr_t>(weights[i]) & 3) != 0) {
+      return hipErrorNotSupported;
+    }
+    grp.w[i] = static_cast<const uint32_t *>(weights[i]), grp.out[i] = outs[i], grp.n[i] = ns[i];
+  }
+  return wt == kQ4_0 ? launch_gemv_shared<kQ4_0>(stream, grp, count, static_cast<const uint32_t *>(act), nblk / 2) :
+                       launch_gemv_shared<kQ8_0>(stream, grp, count, static_cast<const uint32_t *>(act), nblk / 2);
 }
 
 }  // namespace htpops

@@ -661,6 +661,88 @@ extern "C" int htpops_execute_op(htpops_context *ctx, const struct OpComputeRequ
 
 namespace {
 
+// Consecutive one-row matmul requests of a message that read the SAME activation row (q/k/v or gate/up of a decoder
+// layer) are collected and run as one kernel launch: the result of every request is what its own launch would have
+// produced (same kernel, same arithmetic), the requests just stop paying a launch and a ramp-up each. A request
+// joins the open batch only if its output cannot feed or clobber anything the batch reads or writes.
+struct GemvBatch {
+  int                   wt = 0, k = 0, count = 0;
+  const void           *act = nullptr;
+  struct RequestHeader *hdr[htpops::kGemvGroupMax];
+  float                *out[htpops::kGemvGroupMax];
+  const void           *w[htpops::kGemvGroupMax];
+  int                   n[htpops::kGemvGroupMax];
+};
+
+bool ranges_overlap(const void *a, size_t a_bytes, const void *b, size_t b_bytes) {
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+  return a0 < b0 + b_bytes && b0 < a0 + a_bytes;
+}
+
+void flush_batch(htpops_context *ctx, GemvBatch &b) {
+  if (b.count == 0) {
+    return;
+  }
+  int ret = HTPOPS_OK;
+  if (b.count > 1) {
+    const hipError_t e = htpops::launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k,
+                                                            (htpops::WeightType) b.wt);
+    if (e == hipErrorNotSupported) {
+      (void) hipGetLastError();
+      for (int i = 0; i < b.count; ++i) {
+        b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act, b.w[i], 1, b.k, b.n[i], b.wt);
+      }
+    } else if (e != hipSuccess) {
+      ret = fail(ctx, HTPOPS_ERR_HIP, "grouped mat_mul launch: %s", hipGetErrorString(e));
+    }
+  } else {
+    ret = op_mat_mul_q8(ctx, b.out[0], b.act, b.w[0], 1, b.k, b.n[0], b.wt);
+  }
+  if (ret != HTPOPS_OK) {
+    for (int i = 0; i < b.count; ++i) {
+      b.hdr[i]->state = ret;
+    }
+  }
+  b.count = 0;
+}
+
+// true: the request is now part of the batch and its state is set; false: run it the ordinary way (after a flush)
+bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct RequestHeader *hdr, GemvBatch &b) {
+  static const int enabled = htpops::env_int("HTPOPS_BATCH_GEMV", 1);
+  if (!enabled || !ctx->has_device ||
+      (req->op != HTP_OPS_MAT_MUL_Q4_0_Q8_0 && req->op != HTP_OPS_MAT_MUL_Q8_0_Q8_0)) {
+    return false;
+  }
+  const auto *p = reinterpret_cast<const MatMulParams *>(req->payload);
+  if (p->m != 1 || p->k <= 0 || p->n <= 0 || p->k % 64 != 0) {
+    return false;
+  }
+  const int    wt        = req->op == HTP_OPS_MAT_MUL_Q4_0_Q8_0 ? htpops::kQ4_0 : htpops::kQ8_0;
+  const size_t out_bytes = (size_t) p->n * 4, act_bytes = q8_0_bytes(1, (size_t) p->k);
+  const size_t w_bytes   = weight_bytes((size_t) p->n, (size_t) p->k, wt);
+  float       *out       = (float *) resolve(ctx, p->output, out_bytes);
+  const void  *w         = resolve(ctx, p->weight, w_bytes);
+  const void  *act       = resolve(ctx, p->activation, act_bytes);
+  if (!out || !w || !act || !aligned(out, 4) || !aligned(w, 4) || !aligned(act, 4) ||
+      ranges_overlap(out, out_bytes, act, act_bytes) || ranges_overlap(out, out_bytes, w, w_bytes)) {
+    return false;  // the ordinary path reports what is wrong, or handles the aliasing in order
+  }
+  bool join = b.count > 0 && b.count < htpops::kGemvGroupMax && b.wt == wt && b.k == p->k && b.act == act;
+  for (int i = 0; join && i < b.count; ++i) {
+    const size_t wi = weight_bytes((size_t) b.n[i], (size_t) b.k, b.wt);
+    join = !ranges_overlap(out, out_bytes, b.out[i], (size_t) b.n[i] * 4) && !ranges_overlap(out, out_bytes, b.w[i], wi) &&
+           !ranges_overlap(b.out[i], (size_t) b.n[i] * 4, w, w_bytes);
+  }
+  if (!join) {
+    flush_batch(ctx, b);
+    b.wt = wt, b.k = p->k, b.act = act;
+  }
+  b.hdr[b.count] = hdr, b.out[b.count] = out, b.w[b.count] = w, b.n[b.count] = p->n;
+  ++b.count;
+  hdr->state = HTPOPS_OK;
+  return true;
+}
+
 // Walks a message and enqueues every request in order (reference: src/dsp/commu.c:91-114). Returns 0 or the
 // framing error; per-request results go to RequestHeader.state.
 int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes) {
@@ -682,19 +764,28 @@ int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_b
       prev = off;
     }
   }
+  GemvBatch batch;
   for (int i = 0; i < n_reqs; ++i) {
     struct RequestHeader *hdr  = message_header_get_request_ptr(msg, i);
     const size_t          size = message_header_get_request_size(msg, i);
     switch (hdr->type) {
       case REQUEST_TYPE_OP_COMPUTE:
         if (size < sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest)) {
+          flush_batch(ctx, batch);
           hdr->state = HTPOPS_ERR_REJECTED;
         } else {
-          hdr->state = htpops_execute_op(ctx, reinterpret_cast<const struct OpComputeRequest *>(hdr->data));
+          const auto *req = reinterpret_cast<const struct OpComputeRequest *>(hdr->data);
+          const bool  matmul_payload =
+            size >= sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest) + sizeof(MatMulParams);
+          if (!(matmul_payload && try_batch(ctx, req, hdr, batch))) {
+            flush_batch(ctx, batch);
+            hdr->state = htpops_execute_op(ctx, req);
+          }
         }
         break;
       case REQUEST_TYPE_RPCMEM_MAP:
         {
+          flush_batch(ctx, batch);
           // reference: commu.c:102-110 -- only the puts are acted on
           const auto *map = reinterpret_cast<const struct RpcmemMapRequest *>(hdr->data);
           int         ret = 0;
@@ -713,6 +804,7 @@ int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_b
         break;  // NO_OP and unknown types are skipped, state untouched (commu.c:111-113)
     }
   }
+  flush_batch(ctx, batch);
   return HTPOPS_OK;
 }
 

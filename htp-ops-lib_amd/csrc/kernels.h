@@ -24,6 +24,11 @@ hipError_t launch_rms_norm_quantize_q8_0(hipStream_t stream, void *dst, const fl
 // decode path: one pass over the weight bytes per activation row
 hipError_t launch_gemv_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
                                 int n, WeightType wt);
+// several weight matrices against ONE shared activation row (m = 1) in a single launch; hipErrorNotSupported when
+// the shapes do not fit the fast kernel (the caller then launches them one by one)
+constexpr int kGemvGroupMax = 8;
+hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *act,
+                                      const void *const *weights, const int *ns, int k, WeightType wt);
 // small-batch path (m <= 32, k % 64 == 0, else hipErrorNotSupported): one pass over the weight bytes for all rows,
 // block dots on v_mfma_i32_32x32x32_i8
 // `workspace` (matmul_skinny_workspace_bytes) holds per-slice partial tiles, `tickets` is an array of

@@ -206,6 +206,42 @@ def test_small_batch_integer_exact(ctx, wt, m):
     assert np.array_equal(got, (qa.astype(np.int64) @ qw.astype(np.int64).T).astype(np.float32))
 
 
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+def test_message_batches_same_activation_gemvs(ctx, oracle, wt):
+    # One message: ten one-row matmuls on activation A with different n (they run as grouped launches of up to
+    # eight), one on activation B, then one more on A whose output buffer is B's output (must stay ordered).
+    rng = wl.rng_for(60, wt)
+    k = 1536
+    op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
+    ns = [256, 1536, 33, 1, 640, 64, 100, 8, 2048, 17]
+    ws = [wl.make_weights(rng, n, k, wt) for n in ns]
+    a = oracle.quantize_q8_0(wl.make_activations(rng, 1, k))
+    b = oracle.quantize_q8_0(wl.make_activations(rng, 1, k))
+    ha, hb = ctx.upload(a), ctx.upload(b)
+    hws = [ctx.upload(w) for w in ws]
+    houts = [ctx.alloc(n * 4) for n in ns]
+    handles = [ha, hb] + hws + houts
+    try:
+        reqs = [(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, api.mat_mul_params((ho, 0), (ha, 0), (hw, 0), 1, k, n)))
+                for ho, hw, n in zip(houts, hws, ns)]
+        # activation B into output 0, then activation A into output 0 again: the last writer must win
+        reqs.append((api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, api.mat_mul_params((houts[0], 0), (hb, 0), (hws[0], 0), 1, k, ns[0]))))
+        reqs.append((api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, api.mat_mul_params((houts[1], 0), (ha, 0), (hws[1], 0), 1, k, ns[1]))))
+        msg = api.build_message(reqs)
+        assert ctx.process_message(msg) == 0
+        assert all(s == 0 for s in api.message_request_states(msg))
+        got = [ctx.read(ho, np.float32, n) for ho, n in zip(houts, ns)]
+        for i, (w, n) in enumerate(zip(ws, ns)):
+            act = b if i == 0 else a
+            single = ctx.run_mat_mul(act, w, 1, k, n, wt)[0]
+            assert np.array_equal(got[i], single), "request %d differs from its own launch" % i
+            want64, mag = oracle.mat_mul_q8_0_act_f64(act, w, 1, k, n, wt)
+            assert np.all(np.abs(got[i] - want64[0]) <= MATMUL_RTOL * mag[0])
+    finally:
+        for h in handles:
+            ctx.release(h)
+
+
 def test_small_batch_repeated_launches_are_bit_identical(ctx):
     # K is cut into slices that are summed in a fixed order by the last workgroup of a row tile: the result must not
     # depend on which workgroup that is, and the ticket counters must come back to zero after every launch
