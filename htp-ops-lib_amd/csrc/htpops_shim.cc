@@ -48,6 +48,16 @@ struct htpops_context {
   // zeroed ticket counters of the K-sliced matmul (each launch leaves them zeroed)
   unsigned *tickets = nullptr;
 
+  // weights of ops 1-4 converted to MFMA fragment order, keyed by the source range; dropped when the source
+  // buffer is written through the registry or released
+  struct FragEntry {
+    const void *src;
+    size_t      src_bytes;
+    int         kind, k, n;
+    void       *frag;
+  };
+  std::vector<FragEntry> frag_cache;
+
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
 
   // mailbox channel
@@ -191,6 +201,31 @@ int ensure_workspace(htpops_context *ctx, size_t bytes) {
   return HTPOPS_OK;
 }
 
+void drop_fragments(htpops_context *ctx, const void *ptr, size_t bytes) {
+  const uintptr_t lo = reinterpret_cast<uintptr_t>(ptr), hi = lo + bytes;
+  bool            synced = false;
+  for (size_t i = 0; i < ctx->frag_cache.size();) {
+    const auto     &e  = ctx->frag_cache[i];
+    const uintptr_t e0 = reinterpret_cast<uintptr_t>(e.src);
+    if (e0 < hi && lo < e0 + e.src_bytes) {
+      if (!synced && ctx->has_device) {
+        (void) hipStreamSynchronize(ctx->stream);  // a queued kernel may still read the fragments
+        synced = true;
+      }
+      (void) hipFree(e.frag);
+      ctx->frag_cache[i] = ctx->frag_cache.back();
+      ctx->frag_cache.pop_back();
+    } else {
+      ++i;
+    }
+  }
+}
+
+size_t permuted_weight_bytes(size_t n, size_t k, int kind) {
+  // reference: op_executor.cc:100-102, :124-126
+  return kind == 1 ? k * n * 2 : k * n / 256 * (kind == 3 ? 272 : 144);
+}
+
 size_t q8_0_bytes(size_t rows, size_t k) {
   return rows * (k / 32) * 34;
 }
@@ -324,6 +359,47 @@ int op_mat_mul_f32(htpops_context *ctx, float *dst, const float *act, const void
   return HTPOPS_OK;
 }
 
+// hmx_mat_mul_permuted_w16a32 / hmx_mat_mul_permuted_qk_0_d16a32 (reference: src/dsp/ops/mat_mul.c:758-855, :875-1153)
+int op_mat_mul_permuted(htpops_context *ctx, float *dst, const float *act, const void *weight, int m, int k, int n,
+                        int kind) {
+  // reference: mat_mul.c:760-769, :878-892
+  if (!dst || !act || !weight || m <= 0 || k <= 0 || n <= 0) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "mat_mul_permuted: null buffer or non-positive size (m=%d k=%d n=%d)", m, k, n);
+  }
+  if (k % 32 != 0 || n % 32 != 0) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "mat_mul_permuted: k=%d and n=%d must be multiples of 32", k, n);
+  }
+  if (!aligned(dst, 128) || !aligned(act, 128) || !aligned(weight, 128)) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "mat_mul_permuted: buffers must be 128-byte aligned");
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  const void *frag = nullptr;
+  for (const auto &e : ctx->frag_cache) {
+    if (e.src == weight && e.kind == kind && e.k == k && e.n == n) {
+      frag = e.frag;
+      break;
+    }
+  }
+  if (!frag) {
+    void *fresh = nullptr;
+    HTPOPS_HIP(ctx, hipMalloc(&fresh, htpops::permuted_weight_fragment_bytes(k, n)));
+    const hipError_t e = htpops::launch_permuted_weight_to_fragments(ctx->stream, fresh, weight, k, n, kind);
+    if (e != hipSuccess) {
+      (void) hipFree(fresh);
+      return fail(ctx, HTPOPS_ERR_HIP, "weight conversion: %s", hipGetErrorString(e));
+    }
+    ctx->frag_cache.push_back({ weight, permuted_weight_bytes((size_t) n, (size_t) k, kind), kind, k, n, fresh });
+    frag = fresh;
+  }
+  if (int r = ensure_workspace(ctx, htpops::permuted_act_fragment_bytes(m, k))) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, htpops::launch_mat_mul_fragments(ctx->stream, dst, act, frag, m, k, n, ctx->workspace));
+  return HTPOPS_OK;
+}
+
 int op_flash_attn(htpops_context *ctx, void *o, const void *q, const void *k, const void *v, const void *mask,
                   int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim, int qo_is_f32, int causal) {
   if (!o || !q || !k || !v || qo_len <= 0 || kv_len <= 0 || n_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0) {
@@ -413,6 +489,10 @@ extern "C" int htpops_close(htpops_context *ctx) {
     if (ctx->tickets) {
       (void) hipFree(ctx->tickets);
     }
+    for (const auto &e : ctx->frag_cache) {
+      (void) hipFree(e.frag);
+    }
+    ctx->frag_cache.clear();
     if (ctx->workspace) {
       (void) hipFree(ctx->workspace);
     }
@@ -485,6 +565,7 @@ extern "C" int htpops_buffer_release(htpops_context *ctx, int handle) {
     return HTPOPS_OK;  // unknown handles are ignored (reference: mmap_mgr.cc:29-37)
   }
   int ret = HTPOPS_OK;
+  drop_fragments(ctx, b->ptr, b->size);
   if (b->owned) {
     if (ctx->has_device) {
       hipError_t e = hipFree(b->ptr);  // waits for work that may still use the block
@@ -520,6 +601,7 @@ extern "C" int htpops_buffer_write(htpops_context *ctx, int handle, size_t offse
     memcpy(dst, src, bytes);
     return HTPOPS_OK;
   }
+  drop_fragments(ctx, dst, bytes);  // converted copies of weights that lived here are stale now
   HTPOPS_HIP(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
   HTPOPS_HIP(ctx, hipStreamSynchronize(ctx->stream));
   return HTPOPS_OK;
@@ -650,8 +732,20 @@ extern "C" int htpops_execute_op(htpops_context *ctx, const struct OpComputeRequ
     case HTP_OPS_MAT_MUL_PERMUTED_W4D16A32:
     case HTP_OPS_MAT_MUL_PERMUTED_W8D16A32:
     case HTP_OPS_MAT_MUL_PERMUTED_W4D16A32_IQ4_NL:
-      return fail(ctx, HTPOPS_ERR_REJECTED, "op %u: tile-permuted weight formats are not built; use the row-layout ops",
-                  req->op);
+      {
+        // reference: op_executor.cc:96-149; the op id doubles as the weight kind
+        const auto *p    = reinterpret_cast<const MatMulParams *>(req->payload);
+        const int   kind = (int) req->op;
+        size_t      out_bytes, act_bytes;
+        if (p->m <= 0 || p->k <= 0 || p->n <= 0 || p->k % 32 != 0 || p->n % 32 != 0 ||
+            !mul3((size_t) p->m, (size_t) p->n, 4, &out_bytes) || !mul3((size_t) p->m, (size_t) p->k, 4, &act_bytes)) {
+          return fail(ctx, HTPOPS_ERR_REJECTED, "mat_mul_permuted: bad size (m=%d k=%d n=%d)", p->m, p->k, p->n);
+        }
+        return op_mat_mul_permuted(ctx, (float *) resolve(ctx, p->output, out_bytes),
+                                   (const float *) resolve(ctx, p->activation, act_bytes),
+                                   resolve(ctx, p->weight, permuted_weight_bytes((size_t) p->n, (size_t) p->k, kind)),
+                                   p->m, p->k, p->n, kind);
+      }
     default:
       // the reference returns 0 without touching anything (op_executor.cc:200-203); a silent success on an
       // unknown op hides host bugs, so this backend reports it

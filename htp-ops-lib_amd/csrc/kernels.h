@@ -46,6 +46,16 @@ size_t     mat_mul_workspace_bytes(int m, int k, int n);
 hipError_t launch_mat_mul_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
                                    int n, WeightType wt, void *workspace, unsigned *tickets, int ticket_slots);
 
+// The reference's native weight formats (ops 1-4): a weight buffer (weight_kind 1 fp16 tiles, 2 Q4_0, 3 Q8_0,
+// 4 IQ4_NL super-blocks) is converted once into MFMA fragment order (permuted_weight_fragment_bytes), then
+// out fp32 [m][n] = fp16(act fp16 x W fp16); `act_fragments` is scratch of permuted_act_fragment_bytes.
+size_t     permuted_weight_fragment_bytes(int k, int n);
+size_t     permuted_act_fragment_bytes(int m, int k);
+hipError_t launch_permuted_weight_to_fragments(hipStream_t stream, void *dst, const void *src, int k, int n,
+                                               int weight_kind);
+hipError_t launch_mat_mul_fragments(hipStream_t stream, float *out, const float *act, const void *weight_fragments,
+                                    int m, int k, int n, void *act_fragments);
+
 // attention; see htpops_flash_attn_ptr. `workspace` holds split-KV partials (decode), size from
 // flash_attn_workspace_bytes.
 size_t     flash_attn_workspace_bytes(int qo_len, int kv_len, int n_heads, int head_dim);

@@ -326,6 +326,18 @@ class Context:
         finally:
             self.release(ha), self.release(hw), self.release(ho)
 
+    def run_mat_mul_permuted(self, act, weight_raw, m, k, n, op, repeats=1):
+        """The reference's ops 1-4: fp32 activations, weights in the reference's tile order (raw bytes)."""
+        act = np.ascontiguousarray(act, dtype=np.float32)
+        ha, hw, ho = self.upload(act), self.upload(np.ascontiguousarray(weight_raw).view(np.uint8)), self.alloc(m * n * 4)
+        try:
+            for _ in range(repeats):
+                self._check(self.execute(op, mat_mul_params((ho, 0), (ha, 0), (hw, 0), m, k, n)))
+            self.synchronize()
+            return self.read(ho, np.float32, m * n).reshape(m, n)
+        finally:
+            self.release(ha), self.release(hw), self.release(ho)
+
     def run_flash_attn(self, q, k, v, mask, n_heads, n_kv_heads, head_dim, causal=False):
         """q fp32 -> the reference op (id 5); q fp16 -> the extended op with the causal flag."""
         qo_len, kv_len = q.shape[0], k.shape[0]

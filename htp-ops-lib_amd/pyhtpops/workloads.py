@@ -119,3 +119,54 @@ QWEN2_1P5B_LAYER = [
 def matmul_algorithmic_bytes(m, k, n, weight_type):
     """Compulsory traffic: every weight byte once, Q8_0 activations once, fp32 outputs once."""
     return n * row_bytes(k, weight_type) + m * row_bytes(k, GGML_TYPE_Q8_0) + m * n * 4
+
+
+# ---------------------------------------------------------------------------- the reference's native weight formats
+IQ4_NL_VALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.int32)
+
+
+def w16_tile_layout(w_kn):
+    """fp16 weights W[k][n] -> the 32x32 tile order of the reference's fp16 matmul (reference: src/host/test.c:300-312):
+    tile (n/32)*(K/32) + k/32, element (k%32 & ~1)*32 + (n%32)*2 + (k&1)."""
+    k, n = w_kn.shape
+    kk, nn = np.meshgrid(np.arange(k), np.arange(n), indexing="ij")
+    idx = ((nn // 32) * (k // 32) + kk // 32) * 1024 + ((kk % 32) & ~1) * 32 + (nn % 32) * 2 + (kk & 1)
+    out = np.empty(k * n, np.float16)
+    out[idx.reshape(-1)] = w_kn.astype(np.float16).reshape(-1)
+    return out
+
+
+def make_permuted_weights(rng, n, k, kind):
+    """Random weights in the super-block formats of ops 2-4 (kind = op id: 2 Q4_0, 3 Q8_0, 4 IQ4_NL): per 32x32 tile
+    four super-blocks of 8 fp16 scales + 128 nibble bytes (144 B) or 256 int8 (272 B). Returns the raw bytes."""
+    n_sb = (n // 32) * (k // 32) * 4
+    scale = 0.01 if kind == 3 else 0.02
+    d = (np.abs(rng.standard_normal((n_sb, 8))) * scale).astype(np.float16)
+    if kind == 3:
+        q = rng.integers(-127, 128, (n_sb, 256), dtype=np.int8).view(np.uint8)
+    else:
+        q = rng.integers(0, 256, (n_sb, 128), dtype=np.uint8)
+    return np.concatenate([d.view(np.uint8).reshape(n_sb, 16), q], axis=1).reshape(-1)
+
+
+def permuted_to_kn(raw, n, k, kind):
+    """Independent numpy reading of the super-block formats: raw bytes -> float32 W[k][n] with values
+    fp16(q * scale). Built from the tile geometry alone (a scale covers 2 K rows x 16 columns; a 64-element vector
+    is one row pair, columns interleaved with K parity), used to cross-check the C oracle."""
+    size = 272 if kind == 3 else 144
+    sb = np.asarray(raw, np.uint8).reshape(-1, size)
+    n_sb = sb.shape[0]
+    scales = sb[:, :16].copy().view(np.float16).astype(np.float32)           # [n_sb][8]
+    if kind == 3:
+        q = sb[:, 16:].copy().view(np.int8).astype(np.int32).reshape(n_sb, 4, 64)   # vector v = bytes 64v..64v+63
+    else:
+        b = sb[:, 16:].astype(np.int32).reshape(n_sb, 64, 2)                 # [e][byte parity]
+        lo, hi = b & 15, b >> 4
+        nib = np.stack([lo[:, :, 0], lo[:, :, 1], hi[:, :, 0], hi[:, :, 1]], axis=1)  # vectors 0..3
+        q = IQ4_NL_VALUES[nib] if kind == 4 else nib - 8
+    sc = np.repeat(scales.reshape(n_sb, 4, 2), 32, axis=2)                   # [n_sb][v][64]
+    vals = (q.astype(np.float32) * sc).astype(np.float16).astype(np.float32)  # one rounding to fp16
+    # super-block s of tile t holds row pairs 4s..4s+3; element e = column e//2, K parity e%2
+    tiles = vals.reshape(n // 32, k // 32, 4, 4, 32, 2)                       # [n0][k0][s][v][col][par]
+    w = tiles.transpose(1, 2, 3, 5, 0, 4).reshape(k, n)                       # k = k0*32 + (4s+v)*2 + par
+    return w

@@ -536,3 +536,106 @@ int oracle_mat_mul_w16a32(float *out, const float *act, const uint16_t *w_tiles,
   }
   return 0;
 }
+
+/* ----------------------------------------------- tile-permuted super-blocks
+ * my_block_q4_0 (144 B = 8 fp16 scales + 128 quant bytes) and my_block_q8_0 (272 B = 8 scales + 256 int8)
+ * hold 256 weights of one 32x32 HMX tile: 8 K rows x 32 N columns. The dequantizer writes four 64-element
+ * vectors per super-block (reference: src/dsp/ops/mat_mul.c:383-405 and :483-505); vector v is tile row pair
+ * 4 * (super-block % 4) + v, element e of a vector is column e / 2, K parity e % 2 (the fp16 tile order of
+ * src/host/test.c:307-312), and elements 0..31 / 32..63 of vector v use scales 2v / 2v + 1 (the scale index
+ * table at :319-325: a scale covers 2 K rows x 16 columns).
+ *   Q4_0 / IQ4_NL: vectors 0, 1 come from the low nibbles of the even / odd quant bytes, vectors 2, 3 from
+ *   the high nibbles of the even / odd bytes (vlut16 sends even bytes to the low and odd bytes to the high
+ *   vector of its result pair, :383-384 with :402-405) -- this even/odd assignment is read off the HVX
+ *   instruction's documented behaviour and has no test in the reference: PARITY UNPINNED for it.
+ *   Q8_0: vunpack keeps byte order, vector v = quants[64 v .. 64 v + 63] (:483-489).
+ * Every value is fp16(q) * fp16(scale), rounded once to fp16 (qf16 multiply then convert, :402-405). */
+
+static uint16_t dequant_fp16_product(int q, uint16_t scale_bits) {
+  /* |q| <= 127 times an 11-bit significand is exact in fp32; one rounding to fp16 */
+  return oracle_fp32_to_fp16((float) q * oracle_fp16_to_fp32(scale_bits));
+}
+
+void oracle_dequantize_permuted_q4_0(const void *super_blocks, int n_super_blocks, int iq4_nl, uint16_t *out) {
+  const uint8_t *src = (const uint8_t *) super_blocks;
+  for (int i = 0; i < n_super_blocks; ++i, src += 144, out += 256) {
+    uint16_t scales[8];
+    memcpy(scales, src, 16);
+    const uint8_t *qs = src + 16;
+    for (int v = 0; v < 4; ++v) {
+      for (int e = 0; e < 64; ++e) {
+        const uint8_t byte = qs[2 * e + (v & 1)];
+        const int     nib  = (v & 2) ? (byte >> 4) : (byte & 0x0f);
+        const int     q    = iq4_nl ? kIq4nl[nib] : nib - 8;
+        out[v * 64 + e]    = dequant_fp16_product(q, scales[2 * v + (e >> 5)]);
+      }
+    }
+  }
+}
+
+void oracle_dequantize_permuted_q8_0(const void *super_blocks, int n_super_blocks, uint16_t *out) {
+  const uint8_t *src = (const uint8_t *) super_blocks;
+  for (int i = 0; i < n_super_blocks; ++i, src += 272, out += 256) {
+    uint16_t scales[8];
+    memcpy(scales, src, 16);
+    const int8_t *qs = (const int8_t *) (src + 16);
+    for (int v = 0; v < 4; ++v) {
+      for (int e = 0; e < 64; ++e) {
+        out[v * 64 + e] = dequant_fp16_product(qs[v * 64 + e], scales[2 * v + (e >> 5)]);
+      }
+    }
+  }
+}
+
+/* The reference's matmul ops 1-4 (src/dsp/ops/mat_mul.c:758-855, :875-1153): activations fp32 -> fp16, weights
+ * fp16 tiles (op 1) or tiles dequantized as above (ops 2-4), products accumulated by the matrix unit, result
+ * rounded to fp16 and widened to fp32 (:909, hmx_consume_accumulator_fp16). The accumulation precision of the
+ * HMX is not documented; here products of the fp16 operands are summed in double (exact to well below one
+ * fp16 ulp) and rounded once. weight_kind: 1 fp16 tiles, 2 Q4_0, 3 Q8_0, 4 IQ4_NL super-blocks (the op ids).
+ * out_f64, if not NULL, receives the unrounded sums. */
+int oracle_mat_mul_permuted(float *out, double *out_f64, const float *act, const void *weight, int m, int k, int n,
+                            int weight_kind) {
+  if (!out || !act || !weight || m <= 0 || k <= 0 || n <= 0 || k % 32 != 0 || n % 32 != 0 || weight_kind < 1 ||
+      weight_kind > 4) {
+    return -1;
+  }
+  const size_t    n_tiles = (size_t) (k / 32) * (size_t) (n / 32);
+  uint16_t       *tiles   = NULL;
+  const uint16_t *w16     = (const uint16_t *) weight;
+  if (weight_kind != 1) {
+    tiles = (uint16_t *) malloc(n_tiles * 1024 * sizeof(uint16_t));
+    if (!tiles) {
+      return -1;
+    }
+    if (weight_kind == 3) {
+      oracle_dequantize_permuted_q8_0(weight, (int) (n_tiles * 4), tiles);
+    } else {
+      oracle_dequantize_permuted_q4_0(weight, (int) (n_tiles * 4), weight_kind == 4, tiles);
+    }
+    w16 = tiles;
+  }
+  float *a16 = (float *) malloc((size_t) k * sizeof(float));
+  float *col = (float *) malloc((size_t) k * sizeof(float));
+  if (!a16 || !col) {
+    free(tiles), free(a16), free(col);
+    return -1;
+  }
+  for (int j = 0; j < n; ++j) {
+    for (int l = 0; l < k; ++l) {
+      col[l] = oracle_fp16_to_fp32(w16[oracle_w16_tile_index(l, j, k)]);
+    }
+    for (int i = 0; i < m; ++i) {
+      double acc = 0.0;
+      for (int l = 0; l < k; ++l) {
+        const float a = oracle_fp16_to_fp32(oracle_fp32_to_fp16(act[(size_t) i * k + l]));
+        acc += (double) a * (double) col[l];
+      }
+      if (out_f64) {
+        out_f64[(size_t) i * n + j] = acc;
+      }
+      out[(size_t) i * n + j] = oracle_fp16_to_fp32(oracle_fp32_to_fp16((float) acc));
+    }
+  }
+  free(tiles), free(a16), free(col);
+  return 0;
+}

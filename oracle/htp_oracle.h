@@ -10,6 +10,10 @@
  *   oracle_dequantize_*          include/dsp/quants.h:11-31, src/dsp/ops/mat_mul.c:25-32, :260-306
  *   oracle_flash_attn            src/dsp/ops/flash_attn.c:1426-1579 (naive_flash_attn)
  *   oracle_mat_mul_w16a32        src/host/test.c:307-327 (tile layout and fp32 triple loop)
+ *   oracle_dequantize_permuted_*,
+ *   oracle_mat_mul_permuted      src/dsp/ops/mat_mul.c:308-508 (super-block dequantizers), :758-855, :875-1153.
+ *                                The even/odd byte order of the Q4_0 super-block is PARITY UNPINNED (no test
+ *                                or fixture in the reference covers it); the rest is pinned by the tile layout.
  *   oracle_quantize_row_q8_0,
  *   oracle_vec_dot_*,
  *   oracle_mat_mul_q*            ggml's Q8_0 quantizer and q4_0 x q8_0 / q8_0 x q8_0 dot product. The reference
@@ -94,6 +98,17 @@ int oracle_mat_mul_w16a32(float *out, const float *act, const uint16_t *w_tiles,
 
 /* Index of weight element (kk, nn) inside the fp16 tile layout above. */
 size_t oracle_w16_tile_index(int kk, int nn, int k);
+
+/* Tile-permuted super-blocks of the reference's ops 2-4 (include/dsp/quants.h:16-31): n_super_blocks x 144 B
+ * (Q4_0, IQ4_NL) or 272 B (Q8_0) -> 256 fp16 bit patterns each, in fp16 tile order (four super-blocks = one
+ * 32x32 tile). Follows src/dsp/ops/mat_mul.c:308-508; see the .c file for what is pinned and what is not. */
+void oracle_dequantize_permuted_q4_0(const void *super_blocks, int n_super_blocks, int iq4_nl, uint16_t *out);
+void oracle_dequantize_permuted_q8_0(const void *super_blocks, int n_super_blocks, uint16_t *out);
+
+/* Ops 1-4 with the reference's operand precisions: fp16 activations x fp16 (dequantized) weights, result rounded
+ * to fp16 and widened. weight_kind = op id (1 fp16 tiles, 2 Q4_0, 3 Q8_0, 4 IQ4_NL). out_f64 may be NULL. */
+int oracle_mat_mul_permuted(float *out, double *out_f64, const float *act, const void *weight, int m, int k, int n,
+                            int weight_kind);
 
 #ifdef __cplusplus
 }

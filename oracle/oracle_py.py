@@ -70,6 +70,12 @@ class Oracle:
             getattr(lib, name).argtypes = [_c_void_p] * 5 + [_c_int] * 6
         lib.oracle_mat_mul_w16a32.restype = _c_int
         lib.oracle_mat_mul_w16a32.argtypes = [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int]
+        lib.oracle_dequantize_permuted_q4_0.restype = None
+        lib.oracle_dequantize_permuted_q4_0.argtypes = [_c_void_p, _c_int, _c_int, _c_void_p]
+        lib.oracle_dequantize_permuted_q8_0.restype = None
+        lib.oracle_dequantize_permuted_q8_0.argtypes = [_c_void_p, _c_int, _c_void_p]
+        lib.oracle_mat_mul_permuted.restype = _c_int
+        lib.oracle_mat_mul_permuted.argtypes = [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int]
         lib.oracle_w16_tile_index.restype = ctypes.c_size_t
         lib.oracle_w16_tile_index.argtypes = [_c_int, _c_int, _c_int]
 
@@ -188,6 +194,29 @@ class Oracle:
         if ret != 0:
             raise ValueError("oracle_mat_mul_w16a32 rejected its arguments")
         return out
+
+    def dequantize_permuted(self, super_blocks, kind):
+        """kind: 2 Q4_0, 3 Q8_0, 4 IQ4_NL (the op ids) -> fp16 [n_super_blocks][256] in tile order."""
+        sb = np.ascontiguousarray(super_blocks, dtype=np.uint8).reshape(-1)
+        size = 272 if kind == 3 else 144
+        n = sb.size // size
+        out = np.empty((n, 256), dtype=np.float16)
+        if kind == 3:
+            self.lib.oracle_dequantize_permuted_q8_0(_ptr(sb), n, _ptr(out))
+        else:
+            self.lib.oracle_dequantize_permuted_q4_0(_ptr(sb), n, 1 if kind == 4 else 0, _ptr(out))
+        return out
+
+    def mat_mul_permuted(self, act, weight, m, k, n, kind, want_f64=False):
+        """Ops 1-4: returns fp32 [m][n] (fp16-rounded values), optionally also the unrounded double sums."""
+        act = np.ascontiguousarray(act, dtype=np.float32)
+        weight = np.ascontiguousarray(weight)
+        out = np.empty((m, n), dtype=np.float32)
+        f64 = np.empty((m, n), dtype=np.float64)
+        ret = self.lib.oracle_mat_mul_permuted(_ptr(out), _ptr(f64), _ptr(act), _ptr(weight), m, k, n, kind)
+        if ret != 0:
+            raise ValueError("oracle_mat_mul_permuted rejected its arguments")
+        return (out, f64) if want_f64 else out
 
     def w16_tile_index(self, kk, nn, k):
         return int(self.lib.oracle_w16_tile_index(kk, nn, k))

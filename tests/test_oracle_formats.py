@@ -264,3 +264,63 @@ def test_mat_mul_against_float64_and_row_independence(oracle, weight_type):
     assert np.array_equal(oracle.mat_mul_q8_0_act(a[3:4], w, 1, k, n, weight_type)[0], out[3])
     assert np.array_equal(oracle.mat_mul_q8_0_act(a, w, m, k, n, weight_type, n_threads=4), out)
     assert np.array_equal(oracle.mat_mul_f32_act(x, w, m, k, n, weight_type), out)
+
+
+# --------------------------------------------------------------------------- reference-native formats (ops 1-4)
+
+def test_permuted_q4_0_known_answers(oracle):
+    # hand-computed from the dequantizer's vector order (reference: src/dsp/ops/mat_mul.c:383-405): quant bytes
+    # 0..127, scales 1..8
+    sb = np.zeros(144, np.uint8)
+    sb[:16] = np.arange(1, 9, dtype=np.float16).view(np.uint8)
+    sb[16:] = np.arange(128, dtype=np.uint8)
+    d = oracle.dequantize_permuted(sb, 2)[0].astype(np.float32)
+    assert d[0] == (0 - 8) * 1          # vector 0, e 0: low nibble of byte 0, scale 0
+    assert d[1] == (2 - 8) * 1          # e 1: low nibble of byte 2
+    assert d[32] == ((64 & 15) - 8) * 2  # e 32: byte 64, scale 1
+    assert d[64] == (1 - 8) * 3         # vector 1: low nibble of byte 1, scale 2
+    assert d[128] == (0 - 8) * 5        # vector 2: high nibble of byte 0, scale 4
+    assert d[192 + 33] == ((67 >> 4) - 8) * 8  # vector 3, e 33: high nibble of byte 67, scale 7
+    nl = oracle.dequantize_permuted(sb, 4)[0].astype(np.float32)
+    assert nl[0] == -127 * 1 and nl[1] == -83 * 1 and nl[128] == -127 * 5
+
+
+def test_permuted_q8_0_known_answers(oracle):
+    sb = np.zeros(272, np.uint8)
+    sb[:16] = np.array([1, 2, 3, 4, 5, 6, 7, 8], np.float16).view(np.uint8) 
+    sb[16:] = (np.arange(256) - 128).astype(np.int8).view(np.uint8)
+    d = oracle.dequantize_permuted(sb, 3)[0].astype(np.float32)
+    assert d[0] == -128 * 1 and d[31] == -97 * 1 and d[32] == -96 * 2 and d[64] == -64 * 3 and d[255] == 127 * 8
+
+
+@pytest.mark.parametrize("kind", [2, 3, 4])
+def test_permuted_dequantizer_matches_numpy_reading(oracle, kind):
+    rng = wl.rng_for(70, kind)
+    n, k = 64, 96
+    raw = wl.make_permuted_weights(rng, n, k, kind)
+    tiles = oracle.dequantize_permuted(raw, kind).reshape(-1)       # fp16 tile order
+    w = wl.permuted_to_kn(raw, n, k, kind)                          # [k][n] from the tile geometry
+    for kk, nn in [(0, 0), (1, 0), (0, 1), (31, 31), (33, 2), (95, 63), (64, 40), (7, 17), (8, 16)]:
+        assert tiles[oracle.w16_tile_index(kk, nn, k)] == np.float16(w[kk, nn])
+    assert np.array_equal(wl.w16_tile_layout(w).view(np.uint16), tiles.view(np.uint16))
+
+
+@pytest.mark.parametrize("kind", [1, 2, 3, 4])
+def test_mat_mul_permuted_against_numpy(oracle, kind):
+    rng = wl.rng_for(71, kind)
+    m, k, n = 3, 96, 64
+    x = wl.make_activations(rng, m, k)
+    if kind == 1:
+        w = (rng.standard_normal((k, n)) * 0.05).astype(np.float16).astype(np.float32)
+        raw = wl.w16_tile_layout(w)
+    else:
+        raw = wl.make_permuted_weights(rng, n, k, kind)
+        w = wl.permuted_to_kn(raw, n, k, kind)
+    got, f64 = oracle.mat_mul_permuted(x, raw, m, k, n, kind, want_f64=True)
+    want = x.astype(np.float16).astype(np.float64) @ w.astype(np.float64)
+    assert np.allclose(f64, want, rtol=1e-12, atol=1e-12)
+    assert np.array_equal(got, want.astype(np.float32).astype(np.float16).astype(np.float32))
+    # the fp32 triple loop of the reference's own test differs only by the fp16 rounding of activations and result
+    if kind == 1:
+        loose = oracle.mat_mul_w16a32(x, raw, m, k, n)
+        assert np.allclose(got, loose, rtol=4e-3, atol=4e-3)
