@@ -1,0 +1,351 @@
+// Prefill-sized quantized matmul on gfx950: out fp32 [m][n] = act block_q8_0 [m][k/32] x W (Q4_0 or Q8_0 rows).
+//
+// Replaces the many-row case of hmx_mat_mul_permuted_qk_0_d16a32 (reference: src/dsp/ops/mat_mul.c:875-1153); the
+// arithmetic is ggml's integer block dot (exact int32 block sums, one fp32 scale per block pair of scales).
+//
+// Per 32 x 32 x 32 block ("unit") the work is
+//     S = act_int8 x w_int8          one v_mfma_i32_32x32x32_i8 (exact block sums for 32 rows x 32 columns)
+//     C = d_act (x) d_w              one v_mfma_f32_32x32x8f16 with the two fp16 scales in K slot 0: the exact fp32
+//                                    product of the scales of every (row, column) pair
+//     acc = fma((float) S, C, acc)   the only vector-ALU work: one convert and one fma per block sum
+// The vector ALU is the floor of this arithmetic (M N K / 32 converts + fmas); everything else is arranged so that it
+// never waits: both operands are kept in "fragment order" -- for every 32-row tile and every block the 64 lanes'
+// 16-byte MFMA operands form one contiguous KiB -- so the inner loop is loads straight into MFMA registers, no LDS,
+// no barrier, no conversion.
+//   weights   converted once per weight buffer (nibbles -> int8 with the "- 8" applied, scales -> one dword per row
+//             and block) and cached by the caller; Q4_0 grows from 0.5625 to 1.125 bytes per weight in that cache
+//   act       converted per call from block_q8_0 rows (a pure re-ordering)
+// A wave owns 64 x 64 outputs (2 x 2 units per block) and a share of K; the KSPLIT waves of one tile are summed
+// through LDS in a fixed order.
+#include "device_utils.h"
+#include "kernels.h"
+
+namespace htpops {
+
+namespace {
+
+typedef int      v4i __attribute__((ext_vector_type(4)));
+typedef int      v16i __attribute__((ext_vector_type(16)));
+typedef float    v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+// ---- operand conversion -------------------------------------------------------------------------------------------
+// fragment (tile, block): lane (c = lane % 32, h = lane / 32) holds elements 16 h .. 16 h + 15 of block `block` of row
+// 32 tile + c; the scale array holds one dword (fp16 scale, 0) per row and block: [tile][block][32].
+
+template <int WT>
+__global__ __launch_bounds__(256) void weights_to_i8_fragments_kernel(uint4 *__restrict__ frag, uint32_t *__restrict__ scales,
+                                                                      const uint16_t *__restrict__ w, int n, int nblk,
+                                                                      int n_tiles) {
+  constexpr int WH = WT == kQ4_0 ? 9 : 17;  // halfwords per block
+  const size_t  t  = (size_t) blockIdx.x * 256 + threadIdx.x;
+  const int     lane = (int) (t & 63);
+  const size_t  f    = t >> 6;
+  const int     kb = (int) (f % (size_t) nblk), tile = (int) (f / (size_t) nblk);
+  if (tile >= n_tiles) {
+    return;
+  }
+  const int c = lane & 31, h = lane >> 5;
+  const int row = tile * 32 + c;
+  uint32_t  o[4] = { 0, 0, 0, 0 };
+  uint32_t  sc   = 0;
+  if (row < n) {
+    const uint16_t *blk = w + ((size_t) row * nblk + kb) * WH;
+    sc = blk[0];
+    if (WT == kQ4_0) {
+      // byte j: low nibble = element j, high nibble = element j + 16 (reference: mat_mul.c:266-271)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t q  = (uint32_t) blk[1 + 2 * i] | ((uint32_t) blk[2 + 2 * i] << 16);  // bytes 4i .. 4i + 3
+        const uint32_t nb = (q >> (4 * h)) & 0x0F0F0F0Fu;
+        // per byte: nibble - 8, as int8 (no borrow between bytes: add 0x80 - 8 then flip the top bit)
+        o[i] = (nb + 0x78787878u) ^ 0x80808080u;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        o[i] = (uint32_t) blk[1 + 8 * h + 2 * i] | ((uint32_t) blk[2 + 8 * h + 2 * i] << 16);
+      }
+    }
+  }
+  frag[t] = make_uint4(o[0], o[1], o[2], o[3]);
+  if (h == 0) {
+    scales[((size_t) tile * nblk + kb) * 32 + c] = sc;
+  }
+}
+
+__global__ __launch_bounds__(256) void act_to_i8_fragments_kernel(uint4 *__restrict__ frag, uint32_t *__restrict__ scales,
+                                                                  const uint16_t *__restrict__ act, int m, int nblk,
+                                                                  int m_tiles) {
+  const size_t t    = (size_t) blockIdx.x * 256 + threadIdx.x;
+  const int    lane = (int) (t & 63);
+  const size_t f    = t >> 6;
+  const int    kb = (int) (f % (size_t) nblk), tile = (int) (f / (size_t) nblk);
+  if (tile >= m_tiles) {
+    return;
+  }
+  const int c = lane & 31, h = lane >> 5;
+  const int row = tile * 32 + c;
+  uint32_t  o[4] = { 0, 0, 0, 0 };
+  uint32_t  sc   = 0;
+  if (row < m) {
+    const uint16_t *blk = act + ((size_t) row * nblk + kb) * 17;
+    sc = blk[0];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      o[i] = (uint32_t) blk[1 + 8 * h + 2 * i] | ((uint32_t) blk[2 + 8 * h + 2 * i] << 16);
+    }
+  }
+  frag[t] = make_uint4(o[0], o[1], o[2], o[3]);
+  if (h == 0) {
+    scales[((size_t) tile * nblk + kb) * 32 + c] = sc;
+  }
+}
+
+// ---- the matmul ---------------------------------------------------------------------------------------------------
+
+constexpr int kGiThreads = 256;
+constexpr int kGiWaves   = 4;
+constexpr int kGiDepth   = 2;  // fragment sets in flight per wave
+
+struct FragSet {
+  uint4    a[2], b[2];
+  uint32_t da[2], dw[2];
+};
+
+// KSPLIT waves share one 64 x 64 tile (each takes every KSPLIT-th block); a workgroup holds 4 / KSPLIT tiles that are
+// neighbours along n (they read the same activation fragments).
+template <int KSPLIT>
+__global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__restrict__ out,
+                                                                       const uint4 *__restrict__ a_frag,
+                                                                       const uint32_t *__restrict__ a_scale,
+                                                                       const uint4 *__restrict__ b_frag,
+                                                                       const uint32_t *__restrict__ b_scale, int m, int n,
+                                                                       int nblk, int m_tiles, int n_tiles) {
+  constexpr int TILES = kGiWaves / KSPLIT;
+  __shared__ float red[TILES][KSPLIT - 1][4][16][64];  // partial accumulators of the waves with ks > 0
+
+  // the wave index (and everything derived from it) is made scalar so that fragment addresses are scalar base +
+  // per-lane offset and cost no vector instructions in the loop
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int ks = wave % KSPLIT, tw = wave / KSPLIT;
+  const int c = lane & 31, h = lane >> 5;
+  // 64 x 64 tile of this wave, in units of 32: m tiles mt0, mt0 + 1; n tiles nt0, nt0 + 1
+  // Workgroup ids go round-robin over the 8 XCDs (each with its own L2). All row blocks of one column group are
+  // given consecutive slots of ONE XCD, so the weight fragments they share are fetched into that L2 once.
+  const int gy = (m_tiles + 1) / 2, gx = (n_tiles + 2 * TILES - 1) / (2 * TILES);
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int by = slot % gy, bx = (slot / gy) * 8 + xcd;
+  if (bx >= gx) {
+    return;  // whole workgroup (the grid is padded to a multiple of 8 column groups)
+  }
+  const int mt0 = by * 2, nt0 = (bx * TILES + tw) * 2;
+  const bool tile_ok = nt0 < n_tiles;  // mt0 < m_tiles by construction
+
+  const uint4    *ap[2], *bp[2];
+  const uint32_t *asp[2], *bsp[2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const size_t mt = (size_t) min(mt0 + i, m_tiles - 1), nt = (size_t) min(nt0 + i, n_tiles - 1);
+    ap[i]  = a_frag + mt * nblk * 64;
+    bp[i]  = b_frag + nt * nblk * 64;
+    asp[i] = a_scale + mt * nblk * 32;
+    bsp[i] = b_scale + nt * nblk * 32;
+  }
+  auto load = [&](FragSet &s, int kb_raw) {
+    const size_t kb = (size_t) min(kb_raw, nblk - 1);  // branch-free: blocks past the end repeat the last one ...
+    const uint32_t live = kb_raw < nblk ? 0xffffffffu : 0u;  // ... with activation scales of zero: they add nothing
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      s.a[i]  = (ap[i] + kb * 64)[lane];
+      s.b[i]  = (bp[i] + kb * 64)[lane];
+      s.da[i] = (asp[i] + kb * 32)[c] & live;
+      s.dw[i] = (bsp[i] + kb * 32)[c];
+    }
+  };
+
+  v16f acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc[i][j][r] = 0.0f;
+      }
+    }
+  }
+
+  FragSet ring[kGiDepth];
+#pragma unroll
+  for (int d = 0; d < kGiDepth; ++d) {
+    load(ring[d], ks + d * KSPLIT);
+  }
+  const v16f zf = { 0 };
+  const v16i zi = { 0 };
+  // scale operands of a unit: (scale, 0, 0, 0) in the lanes of K slots 0..3, zeros in the other lane half
+  auto scale_operand = [&](uint32_t packed) {
+    const uint2 u = make_uint2(h == 0 ? packed : 0u, 0u);
+    return __builtin_bit_cast(v4h, u);
+  };
+  auto mfma_sum = [&](const FragSet &s, int i, int j) {
+    const v4i af = { (int) s.a[i].x, (int) s.a[i].y, (int) s.a[i].z, (int) s.a[i].w };
+    const v4i bf = { (int) s.b[j].x, (int) s.b[j].y, (int) s.b[j].z, (int) s.b[j].w };
+    return __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, zi, 0, 0, 0);
+  };
+  auto mfma_scale = [&](const FragSet &s, int i, int j) {
+    return __builtin_amdgcn_mfma_f32_32x32x8f16(scale_operand(s.da[i]), scale_operand(s.dw[j]), zf, 0, 0, 0);
+  };
+
+  // Software pipeline over units (block, i, j): the two matrix instructions of the NEXT unit are issued between the
+  // 16 converts and the 16 fmas of the CURRENT one, so neither pipe waits for the other.
+  v16i sum_next = mfma_sum(ring[0], 0, 0);
+  v16f scl_next = mfma_scale(ring[0], 0, 0);
+  const int steps = (nblk - ks + KSPLIT - 1) / KSPLIT;  // blocks of this wave
+  for (int s0 = 0; s0 < steps; s0 += kGiDepth) {
+#pragma unroll
+    for (int d = 0; d < kGiDepth; ++d) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int      i = u >> 1, j = u & 1;
+        const v16i     sum_cur = sum_next;
+        const v16f     scl_cur = scl_next;
+        const FragSet &nx = u < 3 ? ring[d] : ring[(d + 1) % kGiDepth];
+        const int      ni = u < 3 ? (u + 1) >> 1 : 0, nj = u < 3 ? (u + 1) & 1 : 0;
+        // The empty volatile asm statements keep their program order and each pins the value it names: the next
+        // unit's block sums exist (in registers of their own) before this unit's converts and fmas are done.
+        sum_next = mfma_sum(nx, ni, nj);
+        asm volatile("" : "+v"(sum_next));
+        v16f f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          f[r] = (float) sum_cur[r];
+        }
+        asm volatile("" : "+v"(f));
+        scl_next = mfma_scale(nx, ni, nj);
+        asm volatile("" : "+v"(scl_next));
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          acc[i][j][r] = __builtin_fmaf(f[r], scl_cur[r], acc[i][j][r]);
+        }
+        asm volatile("" : "+v"(acc[i][j]));
+      }
+      // every matrix instruction that reads ring[d] has been issued: fetch the set DEPTH steps ahead
+      load(ring[d], ks + (s0 + d + kGiDepth) * KSPLIT);
+    }
+  }
+
+  // ---- the waves of a tile: ks > 0 park their sums in LDS, ks == 0 adds them in order and stores ----
+  if (ks > 0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          red[tw][ks - 1][i * 2 + j][r][lane] = acc[i][j][r];
+        }
+      }
+    }
+  }
+  __syncthreads();
+  if (ks == 0 && tile_ok) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if (mt0 + i < m_tiles && nt0 + j < n_tiles) {
+          const int col = (nt0 + j) * 32 + c;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            float v = acc[i][j][r];
+#pragma unroll
+            for (int s = 0; s < KSPLIT - 1; ++s) {
+              v += red[tw][s][i * 2 + j][r][lane];
+            }
+            // D[row][col]: col = lane % 32, row = 8 (r / 4) + 4 (lane / 32) + r % 4
+            const int row = (mt0 + i) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+            if (row < m && col < n) {
+              out[(size_t) row * n + col] = v;
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+size_t round256(size_t x) {
+  return (x + 255) & ~(size_t) 255;
+}
+
+}  // namespace
+
+// layout of a converted weight buffer: [fragments: n_tiles * nblk KiB][scales: n_tiles * nblk * 32 dwords]
+size_t gemm_i8_weight_fragment_bytes(int k, int n) {
+  const size_t n_tiles = ((size_t) n + 31) / 32, nblk = (size_t) k / 32;
+  return round256(n_tiles * nblk * 1024) + n_tiles * nblk * 128;
+}
+
+size_t gemm_i8_act_fragment_bytes(int m, int k) {
+  const size_t m_tiles = ((size_t) m + 31) / 32, nblk = (size_t) k / 32;
+  return round256(m_tiles * nblk * 1024) + m_tiles * nblk * 128;
+}
+
+hipError_t launch_weights_to_i8_fragments(hipStream_t stream, void *dst, const void *weight, int k, int n,
+                                          WeightType wt) {
+  if (k % 32 != 0 || (reinterpret_cast<uintptr_t>(weight) & 1) != 0) {
+    return hipErrorInvalidValue;
+  }
+  const int    nblk = k / 32, n_tiles = (n + 31) / 32;
+  const size_t pieces = (size_t) n_tiles * nblk * 64;
+  uint4       *frag   = static_cast<uint4 *>(dst);
+  uint32_t    *scales = reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(dst) + round256((size_t) n_tiles * nblk * 1024));
+  const dim3   grid((unsigned) ((pieces + 255) / 256));
+  if (wt == kQ4_0) {
+    hipLaunchKernelGGL(weights_to_i8_fragments_kernel<kQ4_0>, grid, dim3(256), 0, stream, frag, scales,
+                       static_cast<const uint16_t *>(weight), n, nblk, n_tiles);
+  } else {
+    hipLaunchKernelGGL(weights_to_i8_fragments_kernel<kQ8_0>, grid, dim3(256), 0, stream, frag, scales,
+                       static_cast<const uint16_t *>(weight), n, nblk, n_tiles);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_fragments,
+                                    int m, int k, int n, void *act_fragments) {
+  if (k % 32 != 0 || m <= 0 || n <= 0) {
+    return hipErrorInvalidValue;
+  }
+  const int    nblk = k / 32, n_tiles = (n + 31) / 32, m_tiles = (m + 31) / 32;
+  uint4       *af  = static_cast<uint4 *>(act_fragments);
+  uint32_t    *as  = reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(act_fragments) + round256((size_t) m_tiles * nblk * 1024));
+  const uint4 *bf  = static_cast<const uint4 *>(weight_fragments);
+  const uint32_t *bs = reinterpret_cast<const uint32_t *>(static_cast<const uint8_t *>(weight_fragments) +
+                                                          round256((size_t) n_tiles * nblk * 1024));
+  const size_t a_pieces = (size_t) m_tiles * nblk * 64;
+  hipLaunchKernelGGL(act_to_i8_fragments_kernel, dim3((unsigned) ((a_pieces + 255) / 256)), dim3(256), 0, stream, af, as,
+                     static_cast<const uint16_t *>(act_q8_0), m, nblk, m_tiles);
+  if (hipError_t e = hipGetLastError(); e != hipSuccess) {
+    return e;
+  }
+  // enough waves for two per SIMD: split K four ways when the tile count alone gives fewer than ~1500 waves
+  const int    wave_tiles = ((m_tiles + 1) / 2) * ((n_tiles + 1) / 2);
+  static const int forced = env_int("HTPOPS_GEMM_KSPLIT", 0);
+  const int    ksplit = forced ? forced : (wave_tiles * 2 < 1536 ? 4 : 2);
+  const unsigned gy = (unsigned) ((m_tiles + 1) / 2);
+  auto grid = [&](int tiles_per_wg) {
+    const unsigned gx = (unsigned) ((n_tiles + 2 * tiles_per_wg - 1) / (2 * tiles_per_wg));
+    return dim3((gx + 7) / 8 * 8 * gy);
+  };
+  if (ksplit == 4) {
+    hipLaunchKernelGGL(gemm_i8_fragments_kernel<4>, grid(1), dim3(kGiThreads), 0, stream, out, af, as, bf, bs, m, n, nblk,
+                       m_tiles, n_tiles);
+  } else {
+    hipLaunchKernelGGL(gemm_i8_fragments_kernel<2>, grid(2), dim3(kGiThreads), 0, stream, out, af, as, bf, bs, m, n, nblk,
+                       m_tiles, n_tiles);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace htpops

@@ -221,6 +221,13 @@ void drop_fragments(htpops_context *ctx, const void *ptr, size_t bytes) {
   }
 }
 
+// an op is about to write [ptr, ptr + bytes): converted weights made from that range are stale
+void note_device_write(htpops_context *ctx, const void *ptr, size_t bytes) {
+  if (!ctx->frag_cache.empty() && ptr) {
+    drop_fragments(ctx, ptr, bytes);
+  }
+}
+
 size_t permuted_weight_bytes(size_t n, size_t k, int kind) {
   // reference: op_executor.cc:100-102, :124-126
   return kind == 1 ? k * n * 2 : k * n / 256 * (kind == 3 ? 272 : 144);
@@ -254,6 +261,7 @@ int op_rms_norm(htpops_context *ctx, float *dst, const float *src, const float *
   if (int r = need_device(ctx)) {
     return r;
   }
+  note_device_write(ctx, dst, (size_t) ne0 * ne1 * 4);
   HTPOPS_HIP(ctx, htpops::launch_rms_norm_f32(ctx->stream, dst, src, weight, eps, ne0, ne1));
   return HTPOPS_OK;
 }
@@ -268,6 +276,7 @@ int op_quantize(htpops_context *ctx, void *dst, const float *src, int k, int m) 
   if (int r = need_device(ctx)) {
     return r;
   }
+  note_device_write(ctx, dst, q8_0_bytes((size_t) m, (size_t) k));
   HTPOPS_HIP(ctx, htpops::launch_quantize_q8_0(ctx->stream, dst, src, k, m));
   return HTPOPS_OK;
 }
@@ -284,6 +293,7 @@ int op_rms_norm_quantize(htpops_context *ctx, void *dst, const float *src, const
     return r;
   }
   if (ne0 <= 16384) {
+    note_device_write(ctx, dst, q8_0_bytes((size_t) ne1, (size_t) ne0));
     HTPOPS_HIP(ctx, htpops::launch_rms_norm_quantize_q8_0(ctx->stream, dst, src, weight, eps, ne0, ne1));
     return HTPOPS_OK;
   }
@@ -295,6 +305,7 @@ int op_rms_norm_quantize(htpops_context *ctx, void *dst, const float *src, const
   if (int r = ensure_workspace(ctx, bytes)) {
     return r;
   }
+  note_device_write(ctx, dst, q8_0_bytes((size_t) ne1, (size_t) ne0));
   HTPOPS_HIP(ctx, htpops::launch_rms_norm_f32(ctx->stream, (float *) ctx->workspace, src, weight, eps, ne0, ne1));
   HTPOPS_HIP(ctx, htpops::launch_quantize_q8_0(ctx->stream, dst, (const float *) ctx->workspace, ne0, ne1));
   return HTPOPS_OK;
@@ -318,6 +329,84 @@ int check_mat_mul(htpops_context *ctx, const void *dst, const void *act, const v
   return HTPOPS_OK;
 }
 
+// true when [ptr, ptr + bytes) lies inside a buffer this context allocated: its contents change only through
+// htpops_buffer_write or as the output of an op, both of which drop converted copies
+bool in_owned_buffer(htpops_context *ctx, const void *ptr, size_t bytes) {
+  const uintptr_t lo = reinterpret_cast<uintptr_t>(ptr);
+  for (const Buffer &b : ctx->buffers) {
+    const uintptr_t b0 = reinterpret_cast<uintptr_t>(b.ptr);
+    if (b.ptr && b.owned && lo >= b0 && lo + bytes <= b0 + b.size) {
+      return true;
+    }
+  }
+  return false;
+}
+
+constexpr int kFragKindRowLayout = 100;  // + ggml type, to keep apart from the tile-permuted kinds 1..4
+
+// How one quantized matmul will run and how much of the context's workspace it needs.
+struct MatMulPlan {
+  bool        fragments = false;  // many rows: int8 MFMA over operands in fragment order
+  const void *cached    = nullptr;
+  bool        cacheable = false;
+  size_t      act_bytes = 0, weight_bytes = 0;  // fragment sizes
+  size_t      ws_bytes  = 0;
+};
+
+MatMulPlan plan_mat_mul(htpops_context *ctx, const void *weight, int m, int k, int n, int wt) {
+  static const int frag_min_m = htpops::env_int("HTPOPS_GEMM_FRAG_MIN_M", 33);
+  MatMulPlan       p;
+  if (m >= frag_min_m && k % 32 == 0) {
+    p.fragments    = true;
+    p.act_bytes    = (htpops::gemm_i8_act_fragment_bytes(m, k) + 255) & ~(size_t) 255;
+    p.weight_bytes = htpops::gemm_i8_weight_fragment_bytes(k, n);
+    for (const auto &e : ctx->frag_cache) {
+      if (e.src == weight && e.kind == kFragKindRowLayout + wt && e.k == k && e.n == n) {
+        p.cached = e.frag;
+        break;
+      }
+    }
+    if (!p.cached) {
+      p.cacheable = in_owned_buffer(ctx, weight, weight_bytes((size_t) n, (size_t) k, wt));
+    }
+    p.ws_bytes = p.act_bytes + ((p.cached || p.cacheable) ? 0 : p.weight_bytes);
+  } else {
+    p.ws_bytes = htpops::mat_mul_workspace_bytes(m, k, n);
+  }
+  return p;
+}
+
+// `ws` is this matmul's share of the workspace (plan.ws_bytes, already ensured by the caller)
+int run_mat_mul(htpops_context *ctx, MatMulPlan &plan, float *dst, const void *act, const void *weight, int m, int k,
+                int n, int wt, uint8_t *ws) {
+  note_device_write(ctx, dst, (size_t) m * n * 4);
+  if (!plan.fragments) {
+    HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, act, weight, m, k, n, (htpops::WeightType) wt, ws,
+                                                    ctx->tickets, kTicketSlots));
+    return HTPOPS_OK;
+  }
+  const void *frags = plan.cached;
+  if (!frags) {
+    void *fresh = ws + plan.act_bytes;
+    if (plan.cacheable) {
+      HTPOPS_HIP(ctx, hipMalloc(&fresh, plan.weight_bytes));
+    }
+    const hipError_t e = htpops::launch_weights_to_i8_fragments(ctx->stream, fresh, weight, k, n, (htpops::WeightType) wt);
+    if (e != hipSuccess) {
+      if (plan.cacheable) {
+        (void) hipFree(fresh);
+      }
+      return fail(ctx, HTPOPS_ERR_HIP, "weight conversion: %s", hipGetErrorString(e));
+    }
+    if (plan.cacheable) {
+      ctx->frag_cache.push_back({ weight, weight_bytes((size_t) n, (size_t) k, wt), kFragKindRowLayout + wt, k, n, fresh });
+    }
+    frags = fresh;
+  }
+  HTPOPS_HIP(ctx, htpops::launch_gemm_i8_fragments(ctx->stream, dst, act, frags, m, k, n, ws));
+  return HTPOPS_OK;
+}
+
 int op_mat_mul_q8(htpops_context *ctx, float *dst, const void *act, const void *weight, int m, int k, int n,
                   int weight_type) {
   if (int r = check_mat_mul(ctx, dst, act, weight, m, k, n, weight_type)) {
@@ -326,13 +415,11 @@ int op_mat_mul_q8(htpops_context *ctx, float *dst, const void *act, const void *
   if (int r = need_device(ctx)) {
     return r;
   }
-  if (int r = ensure_workspace(ctx, htpops::mat_mul_workspace_bytes(m, k, n))) {
+  MatMulPlan plan = plan_mat_mul(ctx, weight, m, k, n, weight_type);
+  if (int r = ensure_workspace(ctx, plan.ws_bytes)) {
     return r;
   }
-  HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, act, weight, m, k, n,
-                                                  (htpops::WeightType) weight_type, ctx->workspace, ctx->tickets,
-                                                  kTicketSlots));
-  return HTPOPS_OK;
+  return run_mat_mul(ctx, plan, dst, act, weight, m, k, n, weight_type, static_cast<uint8_t *>(ctx->workspace));
 }
 
 int op_mat_mul_f32(htpops_context *ctx, float *dst, const float *act, const void *weight, int m, int k, int n,
@@ -346,17 +433,15 @@ int op_mat_mul_f32(htpops_context *ctx, float *dst, const float *act, const void
   if (int r = need_device(ctx)) {
     return r;
   }
-  // workspace: [quantized activations][what the matmul kernels need]
+  // workspace: [quantized activations][what the matmul itself needs]
   const size_t q_bytes = (q8_0_bytes((size_t) m, (size_t) k) + 255) & ~(size_t) 255;
-  if (int r = ensure_workspace(ctx, q_bytes + htpops::mat_mul_workspace_bytes(m, k, n))) {
+  MatMulPlan   plan    = plan_mat_mul(ctx, weight, m, k, n, weight_type);
+  if (int r = ensure_workspace(ctx, q_bytes + plan.ws_bytes)) {
     return r;
   }
   uint8_t *ws = static_cast<uint8_t *>(ctx->workspace);
   HTPOPS_HIP(ctx, htpops::launch_quantize_q8_0(ctx->stream, ws, act, k, m));
-  HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, ws, weight, m, k, n,
-                                                  (htpops::WeightType) weight_type, ws + q_bytes, ctx->tickets,
-                                                  kTicketSlots));
-  return HTPOPS_OK;
+  return run_mat_mul(ctx, plan, dst, ws, weight, m, k, n, weight_type, ws + q_bytes);
 }
 
 // hmx_mat_mul_permuted_w16a32 / hmx_mat_mul_permuted_qk_0_d16a32 (reference: src/dsp/ops/mat_mul.c:758-855, :875-1153)
@@ -375,6 +460,7 @@ int op_mat_mul_permuted(htpops_context *ctx, float *dst, const float *act, const
   if (int r = need_device(ctx)) {
     return r;
   }
+  note_device_write(ctx, dst, (size_t) m * n * 4);
   const void *frag = nullptr;
   for (const auto &e : ctx->frag_cache) {
     if (e.src == weight && e.kind == kind && e.k == k && e.n == n) {
@@ -422,6 +508,7 @@ int op_flash_attn(htpops_context *ctx, void *o, const void *q, const void *k, co
   if (int r = ensure_workspace(ctx, htpops::flash_attn_workspace_bytes(qo_len, kv_len, n_heads, head_dim))) {
     return r;
   }
+  note_device_write(ctx, o, (size_t) qo_len * n_heads * head_dim * (qo_is_f32 ? 4 : 2));
   HTPOPS_HIP(ctx, htpops::launch_flash_attn(ctx->stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads,
                                             head_dim, qo_is_f32 != 0, causal != 0, ctx->workspace));
   return HTPOPS_OK;
@@ -779,6 +866,9 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
   }
   int ret = HTPOPS_OK;
   if (b.count > 1) {
+    for (int i = 0; i < b.count; ++i) {
+      note_device_write(ctx, b.out[i], (size_t) b.n[i] * 4);
+    }
     const hipError_t e = htpops::launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k,
                                                             (htpops::WeightType) b.wt);
     if (e == hipErrorNotSupported) {

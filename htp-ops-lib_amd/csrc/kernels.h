@@ -36,12 +36,16 @@ hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *cons
 size_t     matmul_skinny_workspace_bytes(int m, int k, int n);
 hipError_t launch_matmul_skinny(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
                                 int n, WeightType wt, void *workspace, unsigned *tickets, int ticket_slots);
-// prefill path: MFMA over LDS-staged tiles; needs k % 64 == 0 (else hipErrorNotSupported). `workspace` (size from
-// gemm_workspace_bytes, may be null) holds the converted activations of the large-m kernel.
-size_t     gemm_workspace_bytes(int m, int k);
-hipError_t launch_gemm_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
-                                int n, WeightType wt, void *workspace);
-// picks between the two by m
+// many-row path: int8 MFMA over operands in fragment order. The weights are converted once
+// (launch_weights_to_i8_fragments into gemm_i8_weight_fragment_bytes) and can be cached by the caller; the
+// activations are converted per call into `act_fragments` (gemm_i8_act_fragment_bytes).
+size_t     gemm_i8_weight_fragment_bytes(int k, int n);
+size_t     gemm_i8_act_fragment_bytes(int m, int k);
+hipError_t launch_weights_to_i8_fragments(hipStream_t stream, void *dst, const void *weight, int k, int n,
+                                          WeightType wt);
+hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_fragments,
+                                    int m, int k, int n, void *act_fragments);
+// picks between the one-row and the small-batch kernel by m (any m; many rows are better served by the fragment path)
 size_t     mat_mul_workspace_bytes(int m, int k, int n);
 hipError_t launch_mat_mul_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
                                    int n, WeightType wt, void *workspace, unsigned *tickets, int ticket_slots);

@@ -1,23 +1,22 @@
-// Chooses between the decode (GEMV), small-batch (skinny MFMA) and prefill (MFMA GEMM) kernels of the quantized matmul.
+// Chooses between the one-row (GEMV) and small-batch (skinny MFMA) kernels of the quantized matmul. Many rows
+// (prefill) go through launch_gemm_i8_fragments, which needs converted weights and is therefore routed by the
+// caller that owns the conversion cache.
 #include "kernels.h"
 
 namespace htpops {
 
 size_t mat_mul_workspace_bytes(int m, int k, int n) {
-  const size_t a = gemm_workspace_bytes(m, k), b = matmul_skinny_workspace_bytes(m, k, n);
-  return a > b ? a : b;
+  return matmul_skinny_workspace_bytes(m, k, n);
 }
 
 hipError_t launch_mat_mul_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
                                    int n, WeightType wt, void *workspace, unsigned *tickets, int ticket_slots) {
-  // One activation row: pure weight streaming. More rows: the MFMA kernel reads the weights once for all rows.
-  static const int gemm_min_m   = env_int("HTPOPS_GEMM_MIN_M", 2);
-  static const int skinny_max_m = env_int("HTPOPS_SKINNY_MAX_M", 63);
-  if (m < gemm_min_m) {
+  // One activation row: pure weight streaming, one lane group per weight row.
+  if (m == 1) {
     return launch_gemv_q8_0_act(stream, out, act, weight, m, k, n, wt);
   }
   // A handful of rows: still weight streaming, with the block dots on the matrix core; 32 rows per pass.
-  if (m <= skinny_max_m && k % 64 == 0) {
+  if (k % 64 == 0) {
     const size_t act_row = (size_t) (k / 32) * 34;
     for (int m0 = 0; m0 < m; m0 += 32) {
       const int  rows = m - m0 < 32 ? m - m0 : 32;
@@ -30,11 +29,8 @@ hipError_t launch_mat_mul_q8_0_act(hipStream_t stream, float *out, const void *a
     }
     return hipSuccess;
   }
-  hipError_t e = launch_gemm_q8_0_act(stream, out, act, weight, m, k, n, wt, workspace);
-  if (e == hipErrorNotSupported) {
-    return launch_gemv_q8_0_act(stream, out, act, weight, m, k, n, wt);
-  }
-  return e;
+  // rows that are not dword multiples (k = 32 * odd): the generic kernel, row by row
+  return launch_gemv_q8_0_act(stream, out, act, weight, m, k, n, wt);
 }
 
 }  // namespace htpops
