@@ -286,6 +286,33 @@ def test_gemm_mfma_integer_exact(ctx, wt):
     assert np.array_equal(got, (qa.astype(np.int64) @ qw.astype(np.int64).T).astype(np.float32))
 
 
+def test_gemm_weight_conversion_cache_follows_the_weights(ctx, oracle):
+    # Many-row matmuls run on weights converted to MFMA operand order. For buffers the context allocated the converted
+    # copy is cached and must be dropped when the buffer is rewritten; for caller-owned (registered) memory nothing is
+    # cached, so the caller may change it freely between calls.
+    rng = wl.rng_for(61, 0)
+    m, k, n = 96, 512, 160
+    a = oracle.quantize_q8_0(wl.make_activations(rng, m, k))
+    w1, w2 = wl.make_q4_0_weights(rng, n, k), wl.make_q4_0_weights(rng, n, k)
+    ha, hw, ho = ctx.upload(a), ctx.upload(w1), ctx.alloc(m * n * 4)
+    alias = ctx.register(ctx.device_ptr(hw), w1.nbytes)  # the same memory seen as caller-owned
+    try:
+        def run(h):
+            assert ctx.execute(api.HTP_OPS_MAT_MUL_Q4_0_Q8_0, api.mat_mul_params((ho, 0), (ha, 0), (h, 0), m, k, n)) == 0
+            ctx.synchronize()
+            return ctx.read(ho, np.float32, m * n).reshape(m, n)
+        want1, mag1 = oracle.mat_mul_q8_0_act_f64(a, w1, m, k, n, wl.GGML_TYPE_Q4_0)
+        want2, mag2 = oracle.mat_mul_q8_0_act_f64(a, w2, m, k, n, wl.GGML_TYPE_Q4_0)
+        for _ in range(2):
+            assert np.all(np.abs(run(hw) - want1) <= MATMUL_RTOL * mag1)
+        ctx.write(hw, w2)
+        assert np.all(np.abs(run(hw) - want2) <= MATMUL_RTOL * mag2)
+        assert np.all(np.abs(run(alias) - want2) <= MATMUL_RTOL * mag2)
+    finally:
+        for h in (alias, ha, hw, ho):
+            ctx.release(h)
+
+
 def test_gemm_full_prefill_shape_rows_match_the_decode_kernel(ctx, oracle):
     # M = 512, K = 4096, N = 11008 is too large for the scalar oracle in a test: check (a) a sample of rows against
     # the oracle and (b) every row against the GEMV kernel of the same row (independent kernel, same arithmetic)
