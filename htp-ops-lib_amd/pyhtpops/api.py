@@ -211,10 +211,7 @@ class Context:
 
     def register(self, device_ptr, nbytes):
         """Registers caller-owned device memory (not freed on release); returns a handle."""
-        h = self.lib.htpops_buffer_register(self.ctx, ctypes.c_void_p(device_ptr), nbytes)
-        if h <= 0:
-            raise HtpOpsError(h, self.last_error())
-        return h
+        return self._check(self.lib.htpops_buffer_register(self._ctx, ctypes.c_void_p(device_ptr), int(nbytes)))
 
     def release(self, handle):
         return self.lib.htpops_buffer_release(self._ctx, int(handle))
