@@ -345,8 +345,11 @@ bool in_owned_buffer(htpops_context *ctx, const void *ptr, size_t bytes) {
 constexpr int kFragKindRowLayout = 100;  // + ggml type, to keep apart from the tile-permuted kinds 1..4
 
 // How one quantized matmul will run and how much of the context's workspace it needs.
+constexpr int kFragKindFp6Panel  = 200;  // + ggml type: FP6 operand panels of the many-row Q4_0 matmul
+
 struct MatMulPlan {
-  bool        fragments = false;  // many rows: int8 MFMA over operands in fragment order
+  bool        fragments = false;  // many rows: matrix-core kernels over converted operands
+  bool        fp6       = false;  // Q4_0 weights: FP6 panels; otherwise int8 fragments
   const void *cached    = nullptr;
   bool        cacheable = false;
   size_t      act_bytes = 0, weight_bytes = 0;  // fragment sizes
@@ -357,11 +360,17 @@ MatMulPlan plan_mat_mul(htpops_context *ctx, const void *weight, int m, int k, i
   static const int frag_min_m = htpops::env_int("HTPOPS_GEMM_FRAG_MIN_M", 33);
   MatMulPlan       p;
   if (m >= frag_min_m && k % 32 == 0) {
+    // Q4_0 weights have two many-row kernels. The FP6 one issues half the vector instructions per block but pays an
+    // exchange through memory for every output tile that several workgroups share; measured, it wins once the
+    // tiles fill the device at least once (HTPOPS_GEMM_FP6: 0 never, 1 always, unset by shape).
+    const int use_fp6 = htpops::env_int("HTPOPS_GEMM_FP6", -1);  // read per call: tests switch kernels
     p.fragments    = true;
-    p.act_bytes    = (htpops::gemm_i8_act_fragment_bytes(m, k) + 255) & ~(size_t) 255;
-    p.weight_bytes = htpops::gemm_i8_weight_fragment_bytes(k, n);
+    p.fp6          = wt == htpops::kQ4_0 && (use_fp6 < 0 ? htpops::gemm_fp6_fills_device(m, n) : use_fp6 != 0);
+    p.act_bytes    = ((p.fp6 ? htpops::gemm_fp6_act_panel_bytes(m, k) : htpops::gemm_i8_act_fragment_bytes(m, k)) + 255) & ~(size_t) 255;
+    p.weight_bytes = p.fp6 ? htpops::gemm_fp6_weight_panel_bytes(k, n) : htpops::gemm_i8_weight_fragment_bytes(k, n);
+    const int kind = (p.fp6 ? kFragKindFp6Panel : kFragKindRowLayout) + wt;
     for (const auto &e : ctx->frag_cache) {
-      if (e.src == weight && e.kind == kFragKindRowLayout + wt && e.k == k && e.n == n) {
+      if (e.src == weight && e.kind == kind && e.k == k && e.n == n) {
         p.cached = e.frag;
         break;
       }
@@ -369,7 +378,8 @@ MatMulPlan plan_mat_mul(htpops_context *ctx, const void *weight, int m, int k, i
     if (!p.cached) {
       p.cacheable = in_owned_buffer(ctx, weight, weight_bytes((size_t) n, (size_t) k, wt));
     }
-    p.ws_bytes = p.act_bytes + ((p.cached || p.cacheable) ? 0 : p.weight_bytes);
+    p.weight_bytes = (p.weight_bytes + 255) & ~(size_t) 255;
+    p.ws_bytes = p.act_bytes + ((p.cached || p.cacheable) ? 0 : p.weight_bytes) + (p.fp6 ? htpops::gemm_fp6_workspace_bytes() : 0);
   } else {
     p.ws_bytes = htpops::mat_mul_workspace_bytes(m, k, n);
   }
@@ -391,7 +401,8 @@ int run_mat_mul(htpops_context *ctx, MatMulPlan &plan, float *dst, const void *a
     if (plan.cacheable) {
       HTPOPS_HIP(ctx, hipMalloc(&fresh, plan.weight_bytes));
     }
-    const hipError_t e = htpops::launch_weights_to_i8_fragments(ctx->stream, fresh, weight, k, n, (htpops::WeightType) wt);
+    const hipError_t e = plan.fp6 ? htpops::launch_q4_0_to_fp6_panel(ctx->stream, fresh, weight, k, n)
+                                  : htpops::launch_weights_to_i8_fragments(ctx->stream, fresh, weight, k, n, (htpops::WeightType) wt);
     if (e != hipSuccess) {
       if (plan.cacheable) {
         (void) hipFree(fresh);
@@ -399,9 +410,15 @@ int run_mat_mul(htpops_context *ctx, MatMulPlan &plan, float *dst, const void *a
       return fail(ctx, HTPOPS_ERR_HIP, "weight conversion: %s", hipGetErrorString(e));
     }
     if (plan.cacheable) {
-      ctx->frag_cache.push_back({ weight, weight_bytes((size_t) n, (size_t) k, wt), kFragKindRowLayout + wt, k, n, fresh });
+      ctx->frag_cache.push_back({ weight, weight_bytes((size_t) n, (size_t) k, wt),
+                                  (plan.fp6 ? kFragKindFp6Panel : kFragKindRowLayout) + wt, k, n, fresh });
     }
     frags = fresh;
+  }
+  if (plan.fp6) {
+    uint8_t *partials = ws + plan.act_bytes + ((plan.cached || plan.cacheable) ? 0 : plan.weight_bytes);
+    HTPOPS_HIP(ctx, htpops::launch_gemm_fp6_panels(ctx->stream, dst, act, frags, m, k, n, ws, partials, ctx->tickets, kTicketSlots));
+    return HTPOPS_OK;
   }
   HTPOPS_HIP(ctx, htpops::launch_gemm_i8_fragments(ctx->stream, dst, act, frags, m, k, n, ws));
   return HTPOPS_OK;

@@ -286,6 +286,60 @@ def test_gemm_mfma_integer_exact(ctx, wt):
     assert np.array_equal(got, (qa.astype(np.int64) @ qw.astype(np.int64).T).astype(np.float32))
 
 
+@pytest.fixture
+def fp6_kernel(monkeypatch):
+    """Forces the FP6 many-row kernel (by default it only takes shapes that fill the device with whole tiles)."""
+    monkeypatch.setenv("HTPOPS_GEMM_FP6", "1")
+
+
+# ragged rows / columns / odd K-block counts; one tile shared by many workgroups (k = 4128, 11008); several tiles per
+# workgroup is covered by test_gemm_fp6_whole_tiles_on_every_workgroup
+@pytest.mark.parametrize("m,k,n", [(64, 64, 128), (128, 128, 128), (100, 96, 200), (33, 4096, 4000), (512, 32, 1024),
+                                   (300, 4128, 1000), (129, 320, 257), (512, 4096, 128), (100, 11008, 96)])
+def test_gemm_fp6(ctx, oracle, fp6_kernel, m, k, n):
+    check_mat_mul(ctx, oracle, wl.rng_for(62, m * 131 + k + n), m, k, n, wl.GGML_TYPE_Q4_0)
+
+
+def test_gemm_fp6_integer_exact_and_repeatable(ctx, fp6_kernel):
+    # scales 1.0: the block sums come straight out of the FP6 matrix instruction (int8 = 16 hi + lo, every part
+    # exact), including the extremes -127 x -8; tiles shared between workgroups are added in a fixed order, so
+    # repeated launches are bit-identical and the ticket counters come back to zero
+    rng = wl.rng_for(63, 0)
+    m, k, n = 160, 2048, 300
+    w = wl.make_weights(rng, n, k, wl.GGML_TYPE_Q4_0).reshape(n, k // 32, -1)
+    w[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    w[0, :, 2:] = 0x00  # all weights -8
+    w = w.reshape(n, -1)
+    a = np.empty((m, k // 32, 34), np.uint8)
+    a[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    a[:, :, 2:] = rng.integers(-127, 128, (m, k // 32, 32), dtype=np.int8).view(np.uint8)
+    a[0, :, 2:] = np.int8(-127).view(np.uint8)
+    a = a.reshape(m, -1)
+    got = ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
+    _, qa = wl.q8_0_split(a, k)
+    _, qw = wl.q4_0_split(w, k)
+    assert np.array_equal(got, (qa.astype(np.int64) @ qw.astype(np.int64).T).astype(np.float32))
+    assert got[0, 0] == 32512.0 * (k // 32)
+    for _ in range(3):
+        assert np.array_equal(ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0), got)
+
+
+def test_gemm_fp6_whole_tiles_on_every_workgroup(ctx, oracle):
+    # 2048 x 4096 outputs = 256 tiles of 128 x 256: the shape class the FP6 kernel takes by default; rows are checked
+    # against the oracle and against the one-row kernel
+    rng = wl.rng_for(64, 0)
+    m, k, n = 2048, 1024, 4096 + 256
+    w = wl.make_q4_0_weights(rng, n, k)
+    a = ctx.run_quantize_q8_0(wl.make_activations(rng, m, k))
+    got = ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
+    rows = [0, 127, 128, 1000, 2047]
+    want64, mag = oracle.mat_mul_q8_0_act_f64(a[rows], w, len(rows), k, n, wl.GGML_TYPE_Q4_0)
+    assert np.all(np.abs(got[rows] - want64) <= MATMUL_RTOL * mag)
+    for r in (5, 1300):
+        gemv = ctx.run_mat_mul(a[r:r + 1], w, 1, k, n, wl.GGML_TYPE_Q4_0)
+        assert np.abs(gemv[0] - got[r]).max() <= 2e-5 * np.abs(gemv).max()
+
+
 def test_gemm_weight_conversion_cache_follows_the_weights(ctx, oracle):
     # Many-row matmuls run on weights converted to MFMA operand order. For buffers the context allocated the converted
     # copy is cached and must be dropped when the buffer is rewritten; for caller-owned (registered) memory nothing is
