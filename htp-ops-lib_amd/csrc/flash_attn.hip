@@ -327,17 +327,26 @@ __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *_
     vreg[p]          = *reinterpret_cast<const v8h *>(v_ptr + off);
   }
 
-  // q for the GH heads, this lane's 8 dims, pre-scaled
+  // q for the GH heads, this lane's 8 dims. fp32 queries are pre-scaled and multiplied in fp32; fp16 queries stay
+  // fp16 pairs for v_dot2_f32_f16 (exact products, fp32 sums) and the scale is applied to the finished score.
+  typedef _Float16 v2h __attribute__((ext_vector_type(2)));
   float q[GH][8];
+  v2h   q2[GH][4];
 #pragma unroll
   for (int g = 0; g < GH; ++g) {
     const int    hg   = min(head0_in_group + g, group - 1);
     const size_t base = (size_t) (h_kv * group + hg) * D + sub * 8;
+    if (QO_F32) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const float v = QO_F32 ? reinterpret_cast<const float *>(q_ptr)[base + e] :
-                               (float) reinterpret_cast<const _Float16 *>(q_ptr)[base + e];
-      q[g][e]       = v * scale;
+      for (int e = 0; e < 8; ++e) {
+        q[g][e] = reinterpret_cast<const float *>(q_ptr)[base + e] * scale;
+      }
+    } else {
+      const v8h qv = *reinterpret_cast<const v8h *>(reinterpret_cast<const _Float16 *>(q_ptr) + base);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        q2[g][e] = (v2h){ qv[2 * e], qv[2 * e + 1] };
+      }
     }
   }
 
@@ -355,11 +364,19 @@ __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *_
 #pragma unroll
     for (int g = 0; g < GH; ++g) {
       float s = 0.0f;
+      if (QO_F32) {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        s += q[g][e] * (float) kreg[p][e];
+        for (int e = 0; e < 8; ++e) {
+          s += q[g][e] * (float) kreg[p][e];
+        }
+        s = key_group_sum<LPK>(s) + mk;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s = __builtin_amdgcn_fdot2(q2[g][e], (v2h){ kreg[p][2 * e], kreg[p][2 * e + 1] }, s, false);
+        }
+        s = key_group_sum<LPK>(s) * scale + mk;
       }
-      s        = key_group_sum<LPK>(s) + mk;
       s        = live ? s : -INFINITY;
       sc[p][g] = s;
       m_loc[g] = fmaxf(m_loc[g], s);

@@ -859,12 +859,12 @@ extern "C" int htpops_execute_op(htpops_context *ctx, const struct OpComputeRequ
 
 namespace {
 
-// Consecutive one-row matmul requests of a message that read the SAME activation row (q/k/v or gate/up of a decoder
-// layer) are collected and run as one kernel launch: the result of every request is what its own launch would have
+// Consecutive matmul requests of a message with 1 to 8 activation rows that read the SAME activation buffer (q/k/v or
+// gate/up of a decoder layer) are collected and run as one kernel launch: the result of every request is what its own launch would have
 // produced (same kernel, same arithmetic), the requests just stop paying a launch and a ramp-up each. A request
 // joins the open batch only if its output cannot feed or clobber anything the batch reads or writes.
 struct GemvBatch {
-  int                   wt = 0, k = 0, count = 0;
+  int                   wt = 0, k = 0, m = 0, count = 0;
   const void           *act = nullptr;
   struct RequestHeader *hdr[htpops::kGemvGroupMax];
   float                *out[htpops::kGemvGroupMax];
@@ -884,20 +884,31 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
   int ret = HTPOPS_OK;
   if (b.count > 1) {
     for (int i = 0; i < b.count; ++i) {
-      note_device_write(ctx, b.out[i], (size_t) b.n[i] * 4);
+      note_device_write(ctx, b.out[i], (size_t) b.m * b.n[i] * 4);
     }
-    const hipError_t e = htpops::launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k,
-                                                            (htpops::WeightType) b.wt);
+    hipError_t e;
+    if (b.m == 1) {
+      e = htpops::launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k, (htpops::WeightType) b.wt);
+    } else {
+      const size_t ws = htpops::matmul_skinny_group_workspace_bytes(b.count, b.n, b.m, b.k);
+      if (int r = ensure_workspace(ctx, ws)) {
+        ret = r;
+        e   = hipSuccess;
+      } else {
+        e = htpops::launch_matmul_skinny_group(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.m, b.k,
+                                               (htpops::WeightType) b.wt, ctx->workspace, ctx->tickets, kTicketSlots);
+      }
+    }
     if (e == hipErrorNotSupported) {
       (void) hipGetLastError();
       for (int i = 0; i < b.count; ++i) {
-        b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act, b.w[i], 1, b.k, b.n[i], b.wt);
+        b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act, b.w[i], b.m, b.k, b.n[i], b.wt);
       }
     } else if (e != hipSuccess) {
       ret = fail(ctx, HTPOPS_ERR_HIP, "grouped mat_mul launch: %s", hipGetErrorString(e));
     }
   } else {
-    ret = op_mat_mul_q8(ctx, b.out[0], b.act, b.w[0], 1, b.k, b.n[0], b.wt);
+    ret = op_mat_mul_q8(ctx, b.out[0], b.act, b.w[0], b.m, b.k, b.n[0], b.wt);
   }
   if (ret != HTPOPS_OK) {
     for (int i = 0; i < b.count; ++i) {
@@ -915,11 +926,11 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
     return false;
   }
   const auto *p = reinterpret_cast<const MatMulParams *>(req->payload);
-  if (p->m != 1 || p->k <= 0 || p->n <= 0 || p->k % 64 != 0) {
-    return false;
+  if (p->m < 1 || p->m > 8 || p->k <= 0 || p->n <= 0 || p->k % 64 != 0) {
+    return false;  // one activation row, or the few rows of the weight-streaming small-batch kernel
   }
   const int    wt        = req->op == HTP_OPS_MAT_MUL_Q4_0_Q8_0 ? htpops::kQ4_0 : htpops::kQ8_0;
-  const size_t out_bytes = (size_t) p->n * 4, act_bytes = q8_0_bytes(1, (size_t) p->k);
+  const size_t out_bytes = (size_t) p->m * p->n * 4, act_bytes = q8_0_bytes((size_t) p->m, (size_t) p->k);
   const size_t w_bytes   = weight_bytes((size_t) p->n, (size_t) p->k, wt);
   float       *out       = (float *) resolve(ctx, p->output, out_bytes);
   const void  *w         = resolve(ctx, p->weight, w_bytes);
@@ -928,15 +939,15 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
       ranges_overlap(out, out_bytes, act, act_bytes) || ranges_overlap(out, out_bytes, w, w_bytes)) {
     return false;  // the ordinary path reports what is wrong, or handles the aliasing in order
   }
-  bool join = b.count > 0 && b.count < htpops::kGemvGroupMax && b.wt == wt && b.k == p->k && b.act == act;
+  bool join = b.count > 0 && b.count < htpops::kGemvGroupMax && b.wt == wt && b.k == p->k && b.m == p->m && b.act == act;
   for (int i = 0; join && i < b.count; ++i) {
-    const size_t wi = weight_bytes((size_t) b.n[i], (size_t) b.k, b.wt);
-    join = !ranges_overlap(out, out_bytes, b.out[i], (size_t) b.n[i] * 4) && !ranges_overlap(out, out_bytes, b.w[i], wi) &&
-           !ranges_overlap(b.out[i], (size_t) b.n[i] * 4, w, w_bytes);
+    const size_t wi = weight_bytes((size_t) b.n[i], (size_t) b.k, b.wt), oi = (size_t) b.m * b.n[i] * 4;
+    join = !ranges_overlap(out, out_bytes, b.out[i], oi) && !ranges_overlap(out, out_bytes, b.w[i], wi) &&
+           !ranges_overlap(b.out[i], oi, w, w_bytes);
   }
   if (!join) {
     flush_batch(ctx, b);
-    b.wt = wt, b.k = p->k, b.act = act;
+    b.wt = wt, b.k = p->k, b.m = p->m, b.act = act;
   }
   b.hdr[b.count] = hdr, b.out[b.count] = out, b.w[b.count] = w, b.n[b.count] = p->n;
   ++b.count;

@@ -36,6 +36,12 @@ hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *cons
 size_t     matmul_skinny_workspace_bytes(int m, int k, int n);
 hipError_t launch_matmul_skinny(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
                                 int n, WeightType wt, void *workspace, unsigned *tickets, int ticket_slots);
+// several weight matrices against the same 2 <= m <= 8 activation rows in one launch; hipErrorNotSupported when the
+// shapes do not fit the K-sliced kernel (the caller then launches them one by one)
+size_t     matmul_skinny_group_workspace_bytes(int count, const int *ns, int m, int k);
+hipError_t launch_matmul_skinny_group(hipStream_t stream, int count, float *const *outs, const void *act,
+                                      const void *const *weights, const int *ns, int m, int k, WeightType wt,
+                                      void *workspace, unsigned *tickets, int ticket_slots);
 // many-row path: int8 MFMA over operands in fragment order. The weights are converted once
 // (launch_weights_to_i8_fragments into gemm_i8_weight_fragment_bytes) and can be cached by the caller; the
 // activations are converted per call into `act_fragments` (gemm_i8_act_fragment_bytes).

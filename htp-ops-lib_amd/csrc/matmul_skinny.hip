@@ -316,13 +316,28 @@ struct SliceGeom {
 typedef __attribute__((address_space(1))) const void *sk_gptr_t;
 typedef __attribute__((address_space(3))) void       *sk_lptr_t;
 
+// Several weight matrices that meet the same activation rows (the q/k/v or gate/up projections of a decoder layer)
+// share one launch: blockIdx.z picks the member, whose weight pointer, output pointer, row count and first tile
+// (for its partial tiles and ticket counters) come from the argument table.
+struct SkinnyGroupArgs {
+  const uint8_t *w[kGemvGroupMax];
+  float         *out[kGemvGroupMax];
+  int            n[kGemvGroupMax];
+  int            tile0[kGemvGroupMax];
+};
+
 template <WeightType WT, int MR>
-__global__ __launch_bounds__(kSlThreads) void matmul_skinny_slice_kernel(float *__restrict__ out,
-                                                                        const uint8_t *__restrict__ act,
-                                                                        const uint8_t *__restrict__ weight, int m,
-                                                                        int k, int n, float *__restrict__ partials,
+__global__ __launch_bounds__(kSlThreads) void matmul_skinny_slice_kernel(SkinnyGroupArgs grp,
+                                                                        const uint8_t *__restrict__ act, int m,
+                                                                        int k, float *__restrict__ partials,
                                                                         unsigned *__restrict__ tickets) {
   typedef SliceGeom<WT> G;
+  const int                     n      = grp.n[blockIdx.z];
+  float *__restrict__           out    = grp.out[blockIdx.z];
+  const uint8_t *__restrict__   weight = grp.w[blockIdx.z];
+  if ((int) (blockIdx.x * kSkRows) >= n) {
+    return;  // whole workgroup: this member has fewer rows than the widest one
+  }
   constexpr int MPAD     = 2 * MR;
   constexpr int WROW_BLK = WT == kQ4_0 ? 18 : 34;
   constexpr int ACT_BYTES = 2 * kSlPairs * ActChunk<MR>::PER_KB;
@@ -337,6 +352,7 @@ __global__ __launch_bounds__(kSlThreads) void matmul_skinny_slice_kernel(float *
   const int nl = lane & 31, half = lane >> 5;
   const int nblk    = k / 32;
   const int tile    = blockIdx.x, slice = blockIdx.y, nslices = gridDim.y;
+  const int gtile   = grp.tile0[blockIdx.z] + tile;  // among all members: partial tiles and tickets
   const int n0      = tile * kSkRows;
   const int a_slot  = min(nl, MPAD - 1);
   const int pair0   = slice * kSlPairs;
@@ -405,7 +421,7 @@ __global__ __launch_bounds__(kSlThreads) void matmul_skinny_slice_kernel(float *
     // The partials travel as device-scope atomic stores and loads (written through to / read from the level all
     // XCDs share) and the ticket is taken only after the stores are acknowledged; a device-scope fence would do the
     // same job by writing back the whole L2, which costs tens of microseconds per workgroup.
-    float *mine = partials + ((size_t) tile * nslices + slice) * (MR * 64);
+    float *mine = partials + ((size_t) gtile * nslices + slice) * (MR * 64);
 #pragma unroll
     for (int e = 0; e < EPT; ++e) {
       __hip_atomic_store(&mine[e * kSlThreads + tid], v[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -413,13 +429,13 @@ __global__ __launch_bounds__(kSlThreads) void matmul_skinny_slice_kernel(float *
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid == 0) {
-      lds_ticket = __hip_atomic_fetch_add(&tickets[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      lds_ticket = __hip_atomic_fetch_add(&tickets[gtile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (lds_ticket != (unsigned) (nslices - 1)) {
       return;
     }
-    const float *all = partials + (size_t) tile * nslices * (MR * 64);
+    const float *all = partials + (size_t) gtile * nslices * (MR * 64);
 #pragma unroll
     for (int e = 0; e < EPT; ++e) {
       v[e] = 0.0f;
@@ -432,7 +448,7 @@ __global__ __launch_bounds__(kSlThreads) void matmul_skinny_slice_kernel(float *
       }
     }
     if (tid == 0) {
-      __hip_atomic_store(&tickets[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+      __hip_atomic_store(&tickets[gtile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
     }
   }
 #pragma unroll
@@ -462,13 +478,31 @@ size_t slice_partial_bytes(int k, int n) {
 }
 
 template <WeightType WT, int MR>
-hipError_t launch_skinny_slices(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
-                                int n, void *workspace, unsigned *tickets) {
-  const unsigned tiles = (unsigned) ((n + kSkRows - 1) / kSkRows), nslices = (unsigned) ((k / 64 + kSlPairs - 1) / kSlPairs);
-  hipLaunchKernelGGL((matmul_skinny_slice_kernel<WT, MR>), dim3(tiles, nslices), dim3(kSlThreads), 0, stream, out,
-                     static_cast<const uint8_t *>(act), static_cast<const uint8_t *>(weight), m, k, n,
-                     static_cast<float *>(workspace), tickets);
+hipError_t launch_skinny_slices(hipStream_t stream, const SkinnyGroupArgs &grp, int count, const void *act, int m, int k,
+                                void *workspace, unsigned *tickets) {
+  int n_max = 0;
+  for (int i = 0; i < count; ++i) {
+    n_max = grp.n[i] > n_max ? grp.n[i] : n_max;
+  }
+  const unsigned tiles = (unsigned) ((n_max + kSkRows - 1) / kSkRows), nslices = (unsigned) ((k / 64 + kSlPairs - 1) / kSlPairs);
+  hipLaunchKernelGGL((matmul_skinny_slice_kernel<WT, MR>), dim3(tiles, nslices, (unsigned) count), dim3(kSlThreads), 0, stream,
+                     grp, static_cast<const uint8_t *>(act), m, k, static_cast<float *>(workspace), tickets);
   return hipGetLastError();
+}
+
+// true when the K-sliced kernel can take these matrices in one launch
+template <WeightType WT>
+bool slices_fit(const SkinnyGroupArgs &grp, int count, int k, const void *workspace, const unsigned *tickets, int ticket_slots) {
+  const size_t row_bytes = (size_t) (k / 32) * (WT == kQ4_0 ? 18 : 34);
+  const bool   split     = k / 64 > kSlPairs;
+  int          tiles     = 0;
+  for (int i = 0; i < count; ++i) {
+    if (reinterpret_cast<uintptr_t>(grp.w[i]) % 16 != 0 || (grp.n[i] + kSkRows - 1) / kSkRows > 65535) {
+      return false;
+    }
+    tiles += (grp.n[i] + kSkRows - 1) / kSkRows;
+  }
+  return row_bytes % 16 == 0 && (!split || (workspace && tickets && tiles <= ticket_slots));
 }
 
 template <WeightType WT, int MR>
@@ -476,12 +510,10 @@ hipError_t launch_skinny(hipStream_t stream, float *out, const void *act, const 
                          void *workspace, unsigned *tickets, int ticket_slots) {
   const int nblk = k / 32;
   static const int use_slices = env_int("HTPOPS_SKINNY_SLICES", 1);
-  const size_t row_bytes = (size_t) nblk * (WT == kQ4_0 ? 18 : 34);
-  const int    tiles     = (n + kSkRows - 1) / kSkRows;
-  const bool   split     = k / 64 > kSlPairs;
-  if (use_slices && row_bytes % 16 == 0 && reinterpret_cast<uintptr_t>(weight) % 16 == 0 && tiles <= 65535 &&
-      (!split || (workspace && tickets && tiles <= ticket_slots))) {
-    return launch_skinny_slices<WT, MR>(stream, out, act, weight, m, k, n, workspace, tickets);
+  SkinnyGroupArgs  one = {};
+  one.w[0] = static_cast<const uint8_t *>(weight), one.out[0] = out, one.n[0] = n, one.tile0[0] = 0;
+  if (use_slices && slices_fit<WT>(one, 1, k, workspace, tickets, ticket_slots)) {
+    return launch_skinny_slices<WT, MR>(stream, one, 1, act, m, k, workspace, tickets);
   }
   constexpr int per_kb = ActChunk<MR>::PER_KB;
   const size_t  budget = 96 * 1024;
@@ -524,6 +556,34 @@ size_t matmul_skinny_workspace_bytes(int m, int k, int n) {
   }
   const int rows = m < 32 ? m : 32;
   return rows <= 8 ? slice_partial_bytes<4>(k, n) : rows <= 16 ? slice_partial_bytes<8>(k, n) : slice_partial_bytes<16>(k, n);
+}
+
+size_t matmul_skinny_group_workspace_bytes(int count, const int *ns, int m, int k) {
+  size_t total = 0;
+  for (int i = 0; i < count; ++i) {
+    total += matmul_skinny_workspace_bytes(m, k, ns[i]);
+  }
+  return total;
+}
+
+hipError_t launch_matmul_skinny_group(hipStream_t stream, int count, float *const *outs, const void *act,
+                                      const void *const *weights, const int *ns, int m, int k, WeightType wt,
+                                      void *workspace, unsigned *tickets, int ticket_slots) {
+  if (count < 1 || count > kGemvGroupMax || k % 64 != 0 || m < 2 || m > 8) {
+    return hipErrorNotSupported;
+  }
+  SkinnyGroupArgs grp = {};
+  int             tile0 = 0;
+  for (int i = 0; i < count; ++i) {
+    grp.w[i] = static_cast<const uint8_t *>(weights[i]), grp.out[i] = outs[i], grp.n[i] = ns[i], grp.tile0[i] = tile0;
+    tile0 += (ns[i] + kSkRows - 1) / kSkRows;
+  }
+  if (wt == kQ4_0) {
+    return slices_fit<kQ4_0>(grp, count, k, workspace, tickets, ticket_slots) ?
+             launch_skinny_slices<kQ4_0, 4>(stream, grp, count, act, m, k, workspace, tickets) : hipErrorNotSupported;
+  }
+  return slices_fit<kQ8_0>(grp, count, k, workspace, tickets, ticket_slots) ?
+           launch_skinny_slices<kQ8_0, 4>(stream, grp, count, act, m, k, workspace, tickets) : hipErrorNotSupported;
 }
 
 hipError_t launch_matmul_skinny(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,

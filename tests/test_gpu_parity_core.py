@@ -242,6 +242,42 @@ def test_message_batches_same_activation_gemvs(ctx, oracle, wt):
             ctx.release(h)
 
 
+@pytest.mark.parametrize("wt,m,k", [(wl.GGML_TYPE_Q4_0, 8, 4096), (wl.GGML_TYPE_Q8_0, 3, 1536), (wl.GGML_TYPE_Q4_0, 2, 2048 + 64)])
+def test_message_batches_same_activation_small_batches(ctx, oracle, wt, m, k):
+    # The same grouping for 2..8 activation rows: matrices of different n on activation A run as one launch of the
+    # K-sliced kernel (each with its own partial tiles and ticket counters), then the same weights on activation B.
+    # Every request must equal its own launch bit for bit, twice in a row (the counters come back to zero).
+    rng = wl.rng_for(65, wt * 100 + m)
+    op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
+    ns = [256, 1536, 33, 640, 100]
+    ws = [wl.make_weights(rng, n, k, wt) for n in ns]
+    a = oracle.quantize_q8_0(wl.make_activations(rng, m, k))
+    b = oracle.quantize_q8_0(wl.make_activations(rng, m, k))
+    ha, hb = ctx.upload(a), ctx.upload(b)
+    hws = [ctx.upload(w) for w in ws]
+    houts_a = [ctx.alloc(m * n * 4) for n in ns]
+    houts_b = [ctx.alloc(m * n * 4) for n in ns]
+    handles = [ha, hb] + hws + houts_a + houts_b
+    try:
+        reqs = [(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, api.mat_mul_params((ho, 0), (ha, 0), (hw, 0), m, k, n)))
+                for ho, hw, n in zip(houts_a, hws, ns)]
+        reqs += [(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, api.mat_mul_params((ho, 0), (hb, 0), (hw, 0), m, k, n)))
+                 for ho, hw, n in zip(houts_b, hws, ns)]
+        msg = api.build_message(reqs)
+        for _ in range(2):
+            assert ctx.process_message(msg) == 0
+            assert all(s == 0 for s in api.message_request_states(msg))
+            for act, houts in ((a, houts_a), (b, houts_b)):
+                for ho, w, n in zip(houts, ws, ns):
+                    got = ctx.read(ho, np.float32, m * n).reshape(m, n)
+                    assert np.array_equal(got, ctx.run_mat_mul(act, w, m, k, n, wt)), "a request differs from its own launch"
+                    want64, mag = oracle.mat_mul_q8_0_act_f64(act, w, m, k, n, wt)
+                    assert np.all(np.abs(got - want64) <= MATMUL_RTOL * mag)
+    finally:
+        for h in handles:
+            ctx.release(h)
+
+
 def test_small_batch_repeated_launches_are_bit_identical(ctx):
     # K is cut into slices that are summed in a fixed order by the last workgroup of a row tile: the result must not
     # depend on which workgroup that is, and the ticket counters must come back to zero after every launch
