@@ -71,11 +71,16 @@ __global__ __launch_bounds__(kPfThreads) void flash_attn_prefill_kernel(void *__
   const int half = lane >> 5;
   const int col  = lane & 31;
 
-  const int h_kv     = blockIdx.y / sub_groups;
-  const int h_in_grp = (blockIdx.y % sub_groups) * gc + wave % gc;
+  // grid: x = (KV head, head sub-group), y = query block, LAST query block first. Workgroups are dispatched in
+  // linear order with x fastest, so under `causal` the long blocks (most visible keys) start first and the short ones
+  // fill the tail; consecutive workgroups, which go to different XCDs, work on different KV heads, so one XCD's L2
+  // keeps seeing the same K/V stream.
+  const int q_block  = (int) (gridDim.y - 1 - blockIdx.y);
+  const int h_kv     = blockIdx.x / sub_groups;
+  const int h_in_grp = (blockIdx.x % sub_groups) * gc + wave % gc;
   const bool wave_on = h_in_grp < group && wave / gc < qsub;
   const int  head    = h_kv * group + (h_in_grp < group ? h_in_grp : 0);
-  const int  q_base  = (blockIdx.x * qsub + (wave / gc < qsub ? wave / gc : 0)) * kBQ;
+  const int  q_base  = (q_block * qsub + (wave / gc < qsub ? wave / gc : 0)) * kBQ;
   const int  q_row   = q_base + col;                  // this lane's query
   const bool q_ok    = wave_on && q_row < qo_len;
   const int  q_clamp = q_row < qo_len ? q_row : qo_len - 1;
@@ -121,49 +126,107 @@ __global__ __launch_bounds__(kPfThreads) void flash_attn_prefill_kernel(void *__
   float l_run = 0.0f;       // running sum over this half's keys only; halves are added at the end
 
   // keys visible to the LAST query row of the workgroup bound the KV loop under `causal`
-  const int q_hi     = min(qo_len, (int) (blockIdx.x + 1) * qsub * kBQ) - 1;
+  const int q_hi     = min(qo_len, (q_block + 1) * qsub * kBQ) - 1;
   const int kv_limit = causal ? min(kv_len, q_hi + (kv_len - qo_len) + 1) : kv_len;
   const int q_shift  = kv_len - qo_len;
+  // last key this lane's query may see, relative to the first key this lane holds in a block (key0 = 4 * half)
+  const int vis_last = (causal ? min(kv_len - 1, q_row + q_shift) : kv_len - 1) - 4 * half;
+
+  // The next K/V block travels global memory -> registers while the current one is being used from LDS.
+  constexpr int K_PIECES = kBK * D / 8 / kPfThreads;         // 16-byte pieces of K per thread
+  constexpr int V_TASKS  = (kBK / 2) * (D / 8) / kPfThreads;  // (key pair, 8-wide d chunk) tasks of V per thread
+  v8h kreg[K_PIECES], vreg[V_TASKS][2];
+  // thread-constant element offsets inside a block; everything that changes per block is uniform (scalar registers)
+  const unsigned k_off = (unsigned) (tid / (D / 8)) * (unsigned) kv_stride + (unsigned) (tid % (D / 8)) * 8u;
+  const unsigned v_off = (unsigned) (tid / (D / 8)) * 2u * (unsigned) kv_stride + (unsigned) (tid % (D / 8)) * 8u;
+  constexpr int  ROWS  = kPfThreads / (D / 8);  // keys (K) or key pairs (V) covered by one pass of the workgroup
+  auto fetch = [&](int k0) {
+    if (k0 + kBK <= kv_len) {
+#pragma unroll
+      for (int j = 0; j < K_PIECES; ++j) {
+        const _Float16 *base = k_ptr + (size_t) h_kv * D + (size_t) (k0 + ROWS * j) * kv_stride;
+        kreg[j]              = *reinterpret_cast<const v8h *>(base + k_off);
+      }
+#pragma unroll
+      for (int j = 0; j < V_TASKS; ++j) {
+        const _Float16 *base = v_ptr + (size_t) h_kv * D + (size_t) (k0 + 2 * ROWS * j) * kv_stride;
+        vreg[j][0]           = *reinterpret_cast<const v8h *>(base + v_off);
+        vreg[j][1]           = *reinterpret_cast<const v8h *>(base + kv_stride + v_off);
+      }
+      return;
+    }
+    // last, partial block: rows past the end repeat the last key (their scores are hidden below)
+#pragma unroll
+    for (int j = 0; j < K_PIECES; ++j) {
+      const int i   = tid + j * kPfThreads;
+      const int key = i / (D / 8), part = i % (D / 8);
+      const int kg  = min(k0 + key, kv_len - 1);
+      kreg[j] = *reinterpret_cast<const v8h *>(k_ptr + (size_t) kg * kv_stride + (size_t) h_kv * D + part * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < V_TASKS; ++j) {
+      const int i = tid + j * kPfThreads;
+      const int c = i % (D / 8), kp = i / (D / 8);
+      const int kg0 = min(k0 + 2 * kp, kv_len - 1), kg1 = min(k0 + 2 * kp + 1, kv_len - 1);
+      vreg[j][0] = *reinterpret_cast<const v8h *>(v_ptr + (size_t) kg0 * kv_stride + (size_t) h_kv * D + c * 8);
+      vreg[j][1] = *reinterpret_cast<const v8h *>(v_ptr + (size_t) kg1 * kv_stride + (size_t) h_kv * D + c * 8);
+    }
+  };
+  if (kv_limit > 0) {
+    fetch(0);
+  }
 
   for (int k0 = 0; k0 < kv_limit; k0 += kBK) {
     __syncthreads();  // previous block's fragments are no longer needed
-    // ---- stage K [key][D] and V^T [d][key] ----
-    {
-      // K: 16-byte pieces, coalesced along d
-      constexpr int PIECES = kBK * D / 8;  // 8 halfs each
+    // ---- stage K [key][D] and V^T [d][key] from the registers ----
 #pragma unroll
-      for (int i = tid; i < PIECES; i += kPfThreads) {
-        const int key = i / (D / 8), part = i % (D / 8);
-        const int kg  = min(k0 + key, kv_len - 1);
-        const v8h v   = *reinterpret_cast<const v8h *>(k_ptr + (size_t) kg * kv_stride + (size_t) h_kv * D + part * 8);
-        *reinterpret_cast<v8h *>(&sm.k[key][part * 8]) = v;
-      }
-      // V^T: a task = (key pair, 8-wide d chunk): two 16-byte loads, eight 4-byte transposed stores
-      constexpr int TASKS = (kBK / 2) * (D / 8);
+    for (int j = 0; j < K_PIECES; ++j) {
+      const int i   = tid + j * kPfThreads;
+      const int key = i / (D / 8), part = i % (D / 8);
+      *reinterpret_cast<v8h *>(&sm.k[key][part * 8]) = kreg[j];
+    }
 #pragma unroll
-      for (int i = tid; i < TASKS; i += kPfThreads) {
-        const int c = i % (D / 8), kp = i / (D / 8);
-        const int kg0 = min(k0 + 2 * kp, kv_len - 1), kg1 = min(k0 + 2 * kp + 1, kv_len - 1);
-        const v8h a = *reinterpret_cast<const v8h *>(v_ptr + (size_t) kg0 * kv_stride + (size_t) h_kv * D + c * 8);
-        const v8h b = *reinterpret_cast<const v8h *>(v_ptr + (size_t) kg1 * kv_stride + (size_t) h_kv * D + c * 8);
+    for (int j = 0; j < V_TASKS; ++j) {
+      // two keys of one 8-wide d chunk: eight 4-byte transposed stores
+      const int i = tid + j * kPfThreads;
+      const int c = i % (D / 8), kp = i / (D / 8);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int d   = c * 8 + e;
-          const int pos = (2 * kp + 8 * (d / 32)) % kBK;
-          v2h       pr  = { a[e], b[e] };
-          *reinterpret_cast<v2h *>(&sm.vt[d][pos]) = pr;
-        }
+      for (int e = 0; e < 8; ++e) {
+        const int d   = c * 8 + e;
+        const int pos = (2 * kp + 8 * (d / 32)) % kBK;
+        v2h       pr  = { vreg[j][0][e], vreg[j][1][e] };
+        *reinterpret_cast<v2h *>(&sm.vt[d][pos]) = pr;
       }
     }
     __syncthreads();
+    if (k0 + kBK < kv_limit) {
+      fetch(k0 + kBK);
+    }
 
-    // ---- S^T = K Q^T: two 32-key tiles ----
+    // ---- S^T - m = K Q^T - m: two 32-key tiles, accumulated on top of minus the running maximum ----
+    // Scores come out of the MFMA already relative to the maximum seen so far, so a block that brings no new maximum
+    // to any query of the wave (the usual case after the first few blocks) needs no subtraction and no rescaling.
+    // additive mask values of this lane's 2 x 16 keys, requested before the products so that they arrive meanwhile
+    v4h mreg[2][4];
+    if (mask) {
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          // four consecutive keys: one 8-byte load (rows are padded to a multiple of 64 keys)
+          mreg[kt][rg] = *reinterpret_cast<const v4h *>(mask + (size_t) q_clamp * mask_ld + k0 + 32 * kt + 8 * rg +
+                                                        4 * half);
+        }
+      }
+    }
+    const bool  fresh = m_run == -INFINITY;  // nothing visible yet for this query
+    const float m_ref = fresh ? 0.0f : m_run;
     v16f st[2];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        st[kt][r] = 0.0f;
+        st[kt][r] = -m_ref;
       }
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
@@ -172,47 +235,76 @@ __global__ __launch_bounds__(kPfThreads) void flash_attn_prefill_kernel(void *__
       }
     }
 
-    // ---- mask, online softmax (lane = query; register r of tile kt is key 32 kt + 8 (r / 4) + 4 half + r % 4) ----
+    // ---- mask (lane = query; register r of tile kt is key k0 + 32 kt + 8 (r / 4) + 4 half + r % 4) ----
+    // Only blocks that a mask, the causal diagonal or the end of the keys touches pay for it (the same for the
+    // whole wave).
+    if (mask != nullptr || k0 + kBK > kv_len || (causal && k0 + kBK - 1 > q_base + q_shift)) {
+      const int last = vis_last - k0;  // registers whose key offset 32 kt + 8 (r / 4) + r % 4 exceeds it are hidden
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          float add[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+          if (mask) {
+            const v4h mv = mreg[kt][rg];
+            add[0] = (float) mv[0], add[1] = (float) mv[1], add[2] = (float) mv[2], add[3] = (float) mv[3];
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int r = 4 * rg + e;
+            st[kt][r]   = (32 * kt + 8 * rg + e > last) ? -INFINITY : st[kt][r] + add[e];
+          }
+        }
+      }
+    }
+
+    // ---- online softmax on scores relative to m_ref ----
     float mx = -INFINITY;
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int key = k0 + 32 * kt + 8 * (r >> 2) + 4 * half + (r & 3);
-        float     s   = st[kt][r];
-        if (mask) {
-          s += (float) mask[(size_t) q_clamp * mask_ld + (size_t) min(key, (int) mask_ld - 1)];
-        }
-        if (key >= kv_len || (causal && key > q_row + q_shift)) {
-          s = -INFINITY;
-        }
-        st[kt][r] = s;
-        mx        = fmaxf(mx, s);
+        mx = fmaxf(mx, st[kt][r]);
       }
     }
-    mx                 = fmaxf(mx, __shfl_xor(mx, 32, kWave));
-    const float m_new  = fmaxf(m_run, mx);
-    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // a fully masked prefix keeps exp2 arguments finite
-    const float alpha  = fast_exp2(m_run - m_safe);            // exp2(-inf) = 0 on the first visible block
-    float       psum   = 0.0f;
+    {
+      // both 32-lane halves of the wave hold the same queries: v_permlane32_swap hands each the other's maximum
+      const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+      mx            = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    }
+    // the first visible block of a query sets its maximum (either sign), later blocks only raise it
+    const bool move = fresh ? (mx != -INFINITY) : (mx > 0.0f);
+    if (__builtin_amdgcn_ballot_w64(move) != 0) {
+      const float delta = move ? mx : 0.0f;
+      const float alpha = fresh ? 0.0f : fast_exp2(-delta);  // O and l of a fresh query are still zero
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          st[kt][r] -= delta;
+        }
+      }
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          oacc[t][r] *= alpha;
+        }
+      }
+      l_run *= alpha;
+      m_run = move ? m_ref + mx : m_run;
+    }
+    float psum = 0.0f;
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float p = fast_exp2(st[kt][r] - m_safe);
+        const float p = fast_exp2(st[kt][r]);
         st[kt][r]     = p;
         psum += p;
       }
     }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-#pragma unroll
-    for (int t = 0; t < DT; ++t) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        oacc[t][r] *= alpha;
-      }
-    }
+    l_run += psum;
 
     // ---- O^T += V^T P^T ----
     // MFMA (kt, u) covers keys 32 kt + 16 u + {4 half + 0..3, 8 + 4 half + 0..3}: exactly registers 8 u .. 8 u + 7
@@ -514,7 +606,11 @@ hipError_t launch_prefill(hipStream_t stream, void *o, const void *q, const void
   const int gc         = group < 4 ? group : 4;
   const int qsub       = 4 / gc;
   const int sub_groups = (group + gc - 1) / gc;
-  const dim3 grid((unsigned) ((qo_len + qsub * kBQ - 1) / (qsub * kBQ)), (unsigned) (n_kv_heads * sub_groups));
+  const unsigned q_blocks = (unsigned) ((qo_len + qsub * kBQ - 1) / (qsub * kBQ));
+  if (q_blocks > 65535u) {
+    return hipErrorInvalidValue;
+  }
+  const dim3 grid((unsigned) (n_kv_heads * sub_groups), q_blocks);
   hipLaunchKernelGGL((flash_attn_prefill_kernel<D, QO_F32>), grid, dim3(kPfThreads), 0, stream, o, q,
                      (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, qo_len, kv_len, n_heads,
                      n_kv_heads, causal ? 1 : 0);
