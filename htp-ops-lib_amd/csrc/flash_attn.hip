@@ -599,6 +599,149 @@ __global__ __launch_bounds__(D) void flash_attn_decode_merge_kernel(void *__rest
   }
 }
 
+// ------------------------------------------------------------------------------------------------ any even head_dim
+
+// Head dims the MFMA kernels above are not built for (anything but 64 and 128; the reference routes head_dim % 64 != 0
+// to its own variant, src/dsp/ops/flash_attn_sp_hdim.c:782-832, which only asks for an even head_dim). One workgroup
+// per (query row, head); its four waves take every fourth 64-key block, with one key per lane for the scores (dot
+// products of fp16 pairs, v_dot2_f32_f16) and one output column per lane (d = lane + 64 i) for O += p V, then merge their
+// (max, sum, O) through LDS. Built for coverage, not speed: K rows are read straight from global memory.
+constexpr int kGenThreads = 256;
+constexpr int kGenMaxD    = 256;
+
+template <bool QO_F32>
+__global__ __launch_bounds__(kGenThreads) void flash_attn_any_dim_kernel(void *__restrict__ o_ptr,
+                                                                         const void *__restrict__ q_ptr,
+                                                                         const _Float16 *__restrict__ k_ptr,
+                                                                         const _Float16 *__restrict__ v_ptr,
+                                                                         const _Float16 *__restrict__ mask, int qo_len,
+                                                                         int kv_len, int n_heads, int n_kv_heads,
+                                                                         int head_dim, int causal) {
+  __shared__ v2h   q_sh[kGenMaxD / 2];
+  __shared__ float part_o[4][kGenMaxD];
+  __shared__ float part_ml[4][2];
+
+  const int D     = head_dim;
+  const int tid   = threadIdx.x;
+  const int lane  = tid & 63;
+  const int wave  = tid >> 6;
+  const int row   = blockIdx.x;
+  const int head  = blockIdx.y;
+  const int h_kv  = head / (n_heads / n_kv_heads);
+  const float scale = (1.0f / sqrtf((float) D)) * kLog2e;
+  const size_t qo_base   = ((size_t) row * n_heads + head) * D;
+  const size_t kv_stride = (size_t) n_kv_heads * D;
+  const size_t mask_ld   = ((size_t) kv_len + 63) / 64 * 64;
+
+  // the scaled query, rounded to fp16 like the MFMA kernels' B operand
+  for (int i = tid; i < D / 2; i += kGenThreads) {
+    float a, b;
+    if (QO_F32) {
+      a = reinterpret_cast<const float *>(q_ptr)[qo_base + 2 * i];
+      b = reinterpret_cast<const float *>(q_ptr)[qo_base + 2 * i + 1];
+    } else {
+      a = (float) reinterpret_cast<const _Float16 *>(q_ptr)[qo_base + 2 * i];
+      b = (float) reinterpret_cast<const _Float16 *>(q_ptr)[qo_base + 2 * i + 1];
+    }
+    q_sh[i] = v2h{ (_Float16) (a * scale), (_Float16) (b * scale) };
+  }
+  __syncthreads();
+
+  const int kv_vis = causal ? min(kv_len, row + (kv_len - qo_len) + 1) : kv_len;  // keys 0 .. kv_vis - 1 are visible
+  float m_run = -INFINITY, l_run = 0.0f;
+  float acc[kGenMaxD / 64] = { 0.0f, 0.0f, 0.0f, 0.0f };
+  for (int k0 = wave * 64; k0 < kv_vis; k0 += 4 * 64) {
+    const int  key = k0 + lane;
+    const bool on  = key < kv_vis;
+    float      s   = -INFINITY;
+    if (on) {
+      const v2h *kr = reinterpret_cast<const v2h *>(k_ptr + (size_t) key * kv_stride + (size_t) h_kv * D);
+      float      d0 = 0.0f, d1 = 0.0f;
+      int        i  = 0;
+      for (; i + 1 < D / 2; i += 2) {
+        d0 = __builtin_amdgcn_fdot2(q_sh[i], kr[i], d0, false);
+        d1 = __builtin_amdgcn_fdot2(q_sh[i + 1], kr[i + 1], d1, false);
+      }
+      if (i < D / 2) {
+        d0 = __builtin_amdgcn_fdot2(q_sh[i], kr[i], d0, false);
+      }
+      s = d0 + d1;
+      if (mask) {
+        s += (float) mask[(size_t) row * mask_ld + key];
+      }
+    }
+    float mx = s;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+    }
+    const float m_new  = fmaxf(m_run, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;  // everything masked so far: keep exp2 arguments finite
+    const float alpha  = fast_exp2(m_run - m_safe);
+    const float p      = fast_exp2(s - m_safe);  // 0 for hidden keys
+    float       psum   = p;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+      psum += __shfl_xor(psum, off, kWave);
+    }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+#pragma unroll
+    for (int i = 0; i < kGenMaxD / 64; ++i) {
+      acc[i] *= alpha;
+    }
+    const int n_keys = min(64, kv_vis - k0);
+    for (int j = 0; j < n_keys; ++j) {
+      const float     pj = __shfl(p, j, kWave);
+      const _Float16 *vr = v_ptr + (size_t) (k0 + j) * kv_stride + (size_t) h_kv * D;
+#pragma unroll
+      for (int i = 0; i < kGenMaxD / 64; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) {
+          acc[i] += pj * (float) vr[d];
+        }
+      }
+    }
+  }
+
+  // merge the four waves
+  if (lane == 0) {
+    part_ml[wave][0] = m_run;
+    part_ml[wave][1] = l_run;
+  }
+#pragma unroll
+  for (int i = 0; i < kGenMaxD / 64; ++i) {
+    part_o[wave][lane + 64 * i] = acc[i];
+  }
+  __syncthreads();
+  float m_all = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    m_all = fmaxf(m_all, part_ml[w][0]);
+  }
+  const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
+  float       l_all  = 0.0f;
+  float       wgt[4];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    wgt[w] = fast_exp2(part_ml[w][0] - m_safe);
+    l_all += wgt[w] * part_ml[w][1];
+  }
+  for (int d = tid; d < D; d += kGenThreads) {
+    float o = 0.0f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      o += wgt[w] * part_o[w][d];
+    }
+    o /= l_all;
+    if (QO_F32) {
+      reinterpret_cast<float *>(o_ptr)[qo_base + d] = o;
+    } else {
+      reinterpret_cast<_Float16 *>(o_ptr)[qo_base + d] = (_Float16) o;
+    }
+  }
+}
+
 template <int D, bool QO_F32>
 hipError_t launch_prefill(hipStream_t stream, void *o, const void *q, const void *k, const void *v, const void *mask,
                           int qo_len, int kv_len, int n_heads, int n_kv_heads, bool causal) {
@@ -650,7 +793,7 @@ hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void 
 }  // namespace
 
 size_t flash_attn_workspace_bytes(int qo_len, int kv_len, int n_heads, int head_dim) {
-  if (qo_len != 1) {
+  if (qo_len != 1 || (head_dim != 64 && head_dim != 128)) {
     return 0;
   }
   const size_t n_splits = ((size_t) kv_len + kDecSplit - 1) / kDecSplit;
@@ -661,7 +804,20 @@ hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const v
                              const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
                              bool qo_is_f32, bool causal, void *workspace) {
   if (head_dim != 64 && head_dim != 128) {
-    return hipErrorNotSupported;
+    if (head_dim <= 0 || head_dim % 2 != 0 || head_dim > kGenMaxD || qo_len > 0x7fffffff || n_heads > 65535) {
+      return hipErrorNotSupported;
+    }
+    const dim3 grid((unsigned) qo_len, (unsigned) n_heads);
+    if (qo_is_f32) {
+      hipLaunchKernelGGL(flash_attn_any_dim_kernel<true>, grid, dim3(kGenThreads), 0, stream, o, q,
+                         (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, qo_len, kv_len, n_heads,
+                         n_kv_heads, head_dim, causal ? 1 : 0);
+    } else {
+      hipLaunchKernelGGL(flash_attn_any_dim_kernel<false>, grid, dim3(kGenThreads), 0, stream, o, q,
+                         (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, qo_len, kv_len, n_heads,
+                         n_kv_heads, head_dim, causal ? 1 : 0);
+    }
+    return hipGetLastError();
   }
   // with a single query row the causal rule (key j visible iff j <= kv_len - 1) hides nothing
   if (qo_len == 1) {

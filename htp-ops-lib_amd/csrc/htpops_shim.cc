@@ -513,11 +513,13 @@ int op_flash_attn(htpops_context *ctx, void *o, const void *q, const void *k, co
     return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: n_heads=%d is not a multiple of n_kv_heads=%d", n_heads,
                 n_kv_heads);
   }
-  if (head_dim != 64 && head_dim != 128) {
-    return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: head_dim=%d (64 and 128 are built)", head_dim);
+  // reference: flash_attn_sp_hdim.c:785-788 (an odd head_dim is refused); 64 and 128 take the MFMA kernels, every
+  // other even head_dim up to 256 the general one
+  if (head_dim % 2 != 0 || head_dim > 256) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: head_dim=%d (even values up to 256 are built)", head_dim);
   }
-  if (!aligned(o, 16) || !aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || (mask && !aligned(mask, 2))) {
-    return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: q/k/v/o must be 16-byte aligned");
+  if (!aligned(o, 16) || !aligned(q, 16) || !aligned(k, 16) || !aligned(v, 16) || (mask && !aligned(mask, 8))) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: q/k/v/o must be 16-byte aligned, the mask 8-byte aligned");
   }
   if (int r = need_device(ctx)) {
     return r;

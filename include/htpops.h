@@ -140,7 +140,9 @@ int htpops_mat_mul_f32_act_ptr(htpops_context *ctx, float *dst, const float *act
 
 /* simple_flash_attn (src/dsp/ops/flash_attn.c:1368-1420). Q/O [qo_len][n_heads][head_dim] as fp32
  * (qo_is_f32 = 1, the reference op) or fp16; K/V fp16 [kv_len][n_kv_heads][head_dim]; mask fp16
- * [qo_len][align_up(kv_len, 64)] added to the scaled scores, or NULL; causal as in FlashAttnExParams. */
+ * [qo_len][align_up(kv_len, 64)] added to the scaled scores, or NULL; causal as in FlashAttnExParams.
+ * head_dim: any even value up to 256 (the reference sends head_dim % 64 != 0 to simple_flash_attn_sp_hdim,
+ * src/dsp/ops/flash_attn_sp_hdim.c:782-832, and refuses odd values, :785). */
 int htpops_flash_attn_ptr(htpops_context *ctx, void *o, const void *q, const void *k, const void *v,
                           const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
                           int qo_is_f32, int causal);

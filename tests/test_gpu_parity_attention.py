@@ -26,6 +26,9 @@ CASES = [
     (1, 300, 8, 2, 128), (1, 4096, 32, 8, 128), (1, 70, 4, 4, 64), (1, 129, 16, 1, 128), (1, 1, 4, 2, 64),
     (5, 70, 4, 2, 64), (40, 300, 4, 1, 128), (33, 517, 4, 4, 128), (64, 64, 2, 1, 64), (128, 128, 8, 2, 128),
     (100, 260, 6, 2, 128), (31, 95, 3, 1, 64), (2, 2, 2, 2, 64), (96, 200, 8, 1, 128),
+    # head dims other than 64 and 128 (the reference's flash_attn_sp_hdim.c domain: any even head_dim)
+    (1, 300, 8, 2, 80), (7, 133, 4, 2, 96), (33, 70, 6, 3, 40), (1, 1, 2, 1, 2), (20, 517, 4, 1, 256), (3, 64, 2, 2, 112),
+    (1, 1000, 4, 4, 192), (65, 65, 2, 1, 30),
 ]
 
 
@@ -107,8 +110,10 @@ def test_rejections(ctx):
     R = api.HTPOPS_ERR_REJECTED
     p = api.flash_attn_params((q, 0), (q, 0), (k, 0), (k, 0), (-1, 0), 1, 64, 8, 3, 128)
     assert ctx.execute(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16, p) == R     # n_heads % n_kv_heads
-    p = api.flash_attn_params((q, 0), (q, 0), (k, 0), (k, 0), (-1, 0), 1, 64, 4, 2, 96)
-    assert ctx.execute(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16, p) == R     # head_dim not built
+    p = api.flash_attn_params((q, 0), (q, 0), (k, 0), (k, 0), (-1, 0), 1, 64, 4, 2, 95)
+    assert ctx.execute(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16, p) == R     # odd head_dim (flash_attn_sp_hdim.c:785)
+    p = api.flash_attn_params((q, 0), (q, 0), (k, 0), (k, 0), (-1, 0), 1, 2, 2, 2, 258)
+    assert ctx.execute(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16, p) == R     # head_dim above what is built
     p = api.flash_attn_params((q, 0), (q, 0), (k, 0), (k, 0), (-1, 0), 1, 4096, 8, 2, 128)
     assert ctx.execute(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16, p) == R     # K/V buffer too small
     ctx.release(q), ctx.release(k)
