@@ -440,11 +440,27 @@ __global__ __launch_bounds__(kSlThreads) void matmul_skinny_slice_kernel(SkinnyG
     for (int e = 0; e < EPT; ++e) {
       v[e] = 0.0f;
     }
-    for (int sl = 0; sl < nslices; ++sl) {
+    // eight slices are requested together (each load travels to the level all XCDs share and back), then added in
+    // slice order
+    for (int sl0 = 0; sl0 < nslices; sl0 += 8) {
+      float x[8][EPT];
 #pragma unroll
-      for (int e = 0; e < EPT; ++e) {
-        v[e] += __hip_atomic_load(&all[(size_t) sl * (MR * 64) + e * kSlThreads + tid], __ATOMIC_RELAXED,
-                                  __HIP_MEMORY_SCOPE_AGENT);
+      for (int u = 0; u < 8; ++u) {
+        const int sl = min(sl0 + u, nslices - 1);
+#pragma unroll
+        for (int e = 0; e < EPT; ++e) {
+          x[u][e] = __hip_atomic_load(&all[(size_t) sl * (MR * 64) + e * kSlThreads + tid], __ATOMIC_RELAXED,
+                                      __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (sl0 + u < nslices) {
+#pragma unroll
+          for (int e = 0; e < EPT; ++e) {
+            v[e] += x[u][e];
+          }
+        }
       }
     }
     if (tid == 0) {
