@@ -6,15 +6,18 @@
 // [kv_len][n_kv_heads][D]; the optional fp16 mask [qo_len][align_up(kv_len, 64)] is ADDED to the scaled scores (the
 // scalar routine's convention, reference :1505-1512); `causal` hides key j from query i when j > i + kv_len - qo_len.
 //
-// Two kernels:
-//  * prefill (any qo_len): one workgroup = 32 query rows x up to 4 query heads of one KV head (one wave per head,
-//    so a K/V tile staged in LDS serves the whole GQA group). Scores are computed transposed, S^T = K Q^T with
-//    v_mfma_f32_32x32x16_f16, which puts one query per lane: row max / row sum are register reductions plus one
-//    exchange between the two lane halves. O^T += V^T P^T uses V transposed on its way into LDS; P goes from the
-//    score registers straight into the MFMA B operand. Under `causal`, KV blocks above the diagonal are skipped.
-//  * decode (qo_len == 1): bandwidth bound. The KV range is split across workgroups (n_kv_heads alone would leave
-//    the GPU idle); 16 lanes share a key (16 bytes of K and V each), all heads of the GQA group are scored against
-//    the same K/V registers, and a second tiny kernel merges the per-split (max, sum, O) partials.
+// Three kernels:
+//  * prefill (any qo_len, head_dim 64 or 128): one workgroup = 32 query rows x up to 4 query heads of one KV head (one
+//    wave per head, so a K/V tile staged in LDS serves the whole GQA group). Scores are computed transposed,
+//    S^T = K Q^T with v_mfma_f32_32x32x16_f16, which puts one query per lane: row max / row sum are register
+//    reductions plus one exchange between the two lane halves. O^T += V^T P^T uses V transposed on its way into LDS;
+//    P goes from the score registers straight into the MFMA B operand. The next K/V block is fetched into registers
+//    while the current one is used; scores are accumulated on top of minus the running maximum, so most blocks need
+//    no rescaling. Under `causal`, KV blocks above the diagonal are skipped and the longest query blocks start first.
+//  * decode (qo_len == 1, head_dim 64 or 128): bandwidth bound. The KV range is split across workgroups (n_kv_heads
+//    alone would leave the GPU idle); 16 lanes share a key (16 bytes of K and V each), all heads of the GQA group are
+//    scored against the same K/V registers, and a second tiny kernel merges the per-split (max, sum, O) partials.
+//  * any other even head_dim up to 256 (the reference's flash_attn_sp_hdim.c domain): a plain kernel without MFMA.
 #include "device_utils.h"
 #include "kernels.h"
 
