@@ -347,6 +347,38 @@ constexpr int kFragKindRowLayout = 100;  // + ggml type, to keep apart from the 
 // How one quantized matmul will run and how much of the context's workspace it needs.
 constexpr int kFragKindFp6Panel  = 200;  // + ggml type: FP6 operand panels of the many-row Q4_0 matmul
 
+constexpr int kFragKindLaneOrder = 300;  // + ggml type: Q4_0 weights in matrix-core operand order (2..8 activation rows)
+
+// The repacked copy of `weight` for the few-row kernel: from the cache, or made now and cached. nullptr when this
+// matmul does not take that kernel (shape, weight type, weights in memory the context does not own and so cannot
+// watch for writes) or when the copy cannot be made; the caller then uses the kernels that read the weights as they are.
+const void *lane_order_weights(htpops_context *ctx, const void *weight, int m, int k, int n, int wt) {
+  if (htpops::env_int("HTPOPS_LANE_ORDER", 1) == 0 || !htpops::matmul_lane_order_fits(n, m, k, (htpops::WeightType) wt)) {
+    return nullptr;
+  }
+  const int kind = kFragKindLaneOrder + wt;
+  for (const auto &e : ctx->frag_cache) {
+    if (e.src == weight && e.kind == kind && e.k == k && e.n == n) {
+      return e.frag;
+    }
+  }
+  if (!in_owned_buffer(ctx, weight, weight_bytes((size_t) n, (size_t) k, wt))) {
+    return nullptr;
+  }
+  void *fresh = nullptr;
+  if (hipMalloc(&fresh, htpops::matmul_lane_order_weight_bytes(k, n)) != hipSuccess) {
+    (void) hipGetLastError();
+    return nullptr;
+  }
+  if (htpops::launch_q4_0_to_lane_order(ctx->stream, fresh, weight, k, n) != hipSuccess) {
+    (void) hipGetLastError();
+    (void) hipFree(fresh);
+    return nullptr;
+  }
+  ctx->frag_cache.push_back({ weight, weight_bytes((size_t) n, (size_t) k, wt), kind, k, n, fresh });
+  return fresh;
+}
+
 struct MatMulPlan {
   bool        fragments = false;  // many rows: matrix-core kernels over converted operands
   bool        fp6       = false;  // Q4_0 weights: FP6 panels; otherwise int8 fragments
@@ -391,6 +423,10 @@ int run_mat_mul(htpops_context *ctx, MatMulPlan &plan, float *dst, const void *a
                 int n, int wt, uint8_t *ws) {
   note_device_write(ctx, dst, (size_t) m * n * 4);
   if (!plan.fragments) {
+    if (const void *lw = lane_order_weights(ctx, weight, m, k, n, wt)) {
+      HTPOPS_HIP(ctx, htpops::launch_matmul_lane_order_group(ctx->stream, 1, &dst, act, &lw, &n, m, k));
+      return HTPOPS_OK;
+    }
     HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, act, weight, m, k, n, (htpops::WeightType) wt, ws,
                                                     ctx->tickets, kTicketSlots));
     return HTPOPS_OK;
@@ -892,13 +928,31 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
     if (b.m == 1) {
       e = htpops::launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k, (htpops::WeightType) b.wt);
     } else {
-      const size_t ws = htpops::matmul_skinny_group_workspace_bytes(b.count, b.n, b.m, b.k);
-      if (int r = ensure_workspace(ctx, ws)) {
-        ret = r;
-        e   = hipSuccess;
-      } else {
-        e = htpops::launch_matmul_skinny_group(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.m, b.k,
-                                               (htpops::WeightType) b.wt, ctx->workspace, ctx->tickets, kTicketSlots);
+      // Members whose weights have (or get) a repacked copy go to the kernel that streams it, the others to the
+      // K-sliced kernel: which kernel a matrix gets depends on that matrix alone, so a request gives the same bits
+      // grouped or alone.
+      float      *out_a[htpops::kGemvGroupMax], *out_b[htpops::kGemvGroupMax];
+      const void *w_a[htpops::kGemvGroupMax], *w_b[htpops::kGemvGroupMax];
+      int         n_a[htpops::kGemvGroupMax], n_b[htpops::kGemvGroupMax], count_a = 0, count_b = 0;
+      for (int i = 0; i < b.count; ++i) {
+        if (const void *lw = lane_order_weights(ctx, b.w[i], b.m, b.k, b.n[i], b.wt)) {
+          out_a[count_a] = b.out[i], w_a[count_a] = lw, n_a[count_a++] = b.n[i];
+        } else {
+          out_b[count_b] = b.out[i], w_b[count_b] = b.w[i], n_b[count_b++] = b.n[i];
+        }
+      }
+      e = hipSuccess;
+      if (count_a > 0) {
+        e = htpops::launch_matmul_lane_order_group(ctx->stream, count_a, out_a, b.act, w_a, n_a, b.m, b.k);
+      }
+      if (e == hipSuccess && count_b > 0) {
+        const size_t ws = htpops::matmul_skinny_group_workspace_bytes(count_b, n_b, b.m, b.k);
+        if (int r = ensure_workspace(ctx, ws)) {
+          ret = r;
+        } else {
+          e = htpops::launch_matmul_skinny_group(ctx->stream, count_b, out_b, b.act, w_b, n_b, b.m, b.k,
+                                                 (htpops::WeightType) b.wt, ctx->workspace, ctx->tickets, kTicketSlots);
+        }
       }
     }
     if (e == hipErrorNotSupported) {

@@ -1,0 +1,294 @@
+// Q4_0 x Q8_0 matmul for 2..8 activation rows over weights repacked once into the order the matrix core wants:
+// out[m][n] = sum over 32-wide blocks of (int dot of the block) * d_act * d_weight (reference: src/dsp/ops/mat_mul.c:572-640,
+// block formats include/dsp/quants.h:8-14, ggml block_q4_0 / block_q8_0).
+//
+// The decode kernel streams Q4_0 rows as they are because one lane can own a whole block. With several activation
+// rows the block dots belong on v_mfma_i32_16x16x32_i8 (activation rows x 16 weight rows x 32 k), whose weight operand
+// wants, per lane (row n = lane % 16, group g = lane / 16), the 4 nibble bytes 4 g .. 4 g + 3 of row n's block: 4-byte
+// pickings from 16 rows, which no wide load delivers from the row layout. So the weights are repacked once per weight
+// buffer (same size, cached by the caller): for a tile of 16 rows and a quad of 4 consecutive blocks,
+//   1024 B: lane l's 16 bytes = its 4 nibble bytes of blocks 4 q .. 4 q + 3
+//    128 B: row n's 4 fp16 scales of those blocks
+// so that a wave fetches a quad with one 16-byte and one 8-byte load per lane, fully coalesced, straight into the
+// registers the MFMA reads. A workgroup owns one tile over the whole of K (its 8 waves take every eighth quad and add
+// up through LDS), so nothing is exchanged between workgroups and a 4096-row matrix still gives 256 of them.
+//
+// Every workgroup needs all activation rows, as many bytes as its weights. They come as they are (block_q8_0 rows)
+// by global_load_lds DMA in 16-byte pieces - no registers, no vector ALU work, in flight together with the first weight
+// loads - into LDS with the 8 rows interleaved piece by piece (the 8 rows a wave reads at one byte offset lie in 8
+// different bank groups); the lanes pick their operand bytes out of that image (a funnel shift where a block starts
+// 2 bytes off a dword) and the block scales out of a float table made once after the DMA has landed. Measured: laying
+// the rows out in operand order with the vector ALU instead cost as much as streaming the weights.
+#include "device_utils.h"
+#include "kernels.h"
+
+#include <stdint.h>
+
+namespace htpops {
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+
+constexpr int kLoThreads  = 512;
+constexpr int kLoWaves    = kLoThreads / kWave;
+constexpr int kLoRows     = 16;                       // weight rows per tile
+constexpr int kLoActRows  = 8;                        // activation rows in the LDS panel (m <= 8)
+constexpr int kLoQuadBytes = 64 * 16 + kLoRows * 8;   // 1152 = 16 rows x 4 blocks x 18 B
+constexpr int kLoScaleBlk = kLoActRows * 4;           // bytes of the scale table per block (8 floats)
+constexpr int kLoChunk    = 4;                        // quads a wave fetches at a time
+constexpr size_t kLoLdsLimit = 160 * 1024;
+
+// ---- repack: one thread per (tile, quad, lane) writes its 16 nibble bytes; lanes 0..15 also write the scales ----
+__global__ __launch_bounds__(256) void q4_0_to_lane_order_kernel(uint8_t *__restrict__ dst,
+                                                                const uint8_t *__restrict__ src, int nblk, int n) {
+  const int    nquads = nblk / 4;
+  const size_t item   = (size_t) blockIdx.x * 256 + threadIdx.x;  // (tile * nquads + quad) * 64 + lane
+  const size_t total  = (size_t) (n / kLoRows) * nquads * 64;
+  if (item >= total) {
+    return;
+  }
+  const int    lane = (int) (item & 63), nl = lane & 15, g = lane >> 4;
+  const size_t tq   = item >> 6;
+  const int    quad = (int) (tq % nquads);
+  const size_t tile = tq / nquads;
+  const uint8_t *row = src + ((size_t) (tile * kLoRows + nl) * nblk + 4 * (size_t) quad) * 18;
+  uint8_t       *out = dst + tq * kLoQuadBytes;
+  uint32_t       w[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint8_t *q = row + j * 18 + 2 + 4 * g;
+    w[j] = (uint32_t) q[0] | ((uint32_t) q[1] << 8) | ((uint32_t) q[2] << 16) | ((uint32_t) q[3] << 24);
+  }
+  *reinterpret_cast<uint4 *>(out + lane * 16) = make_uint4(w[0], w[1], w[2], w[3]);
+  if (g == 0) {
+    uint16_t s[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      s[j] = (uint16_t) (row[j * 18] | (row[j * 18 + 1] << 8));
+    }
+    *reinterpret_cast<uint2 *>(out + 1024 + nl * 8) =
+      make_uint2((uint32_t) s[0] | ((uint32_t) s[1] << 16), (uint32_t) s[2] | ((uint32_t) s[3] << 16));
+  }
+}
+
+struct LaneOrderGroupArgs {
+  const uint8_t *w[kGemvGroupMax];  // repacked weights
+  float         *out[kGemvGroupMax];
+  int            n[kGemvGroupMax];
+};
+
+struct QuadRegs {
+  uint4 q;  // this lane's nibble bytes of the 4 blocks
+  uint2 d;  // the 4 fp16 scales of this lane's row
+};
+
+__global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrderGroupArgs grp,
+                                                                       const uint8_t *__restrict__ act, int m, int k) {
+  extern __shared__ __align__(16) uint8_t lo_lds[];  // activation panel, later the waves' sums
+  const int n = grp.n[blockIdx.y];
+  if ((int) (blockIdx.x * kLoRows) >= n) {
+    return;  // whole workgroup: this member has fewer rows than the widest one
+  }
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int nl = lane & 15, g = lane >> 4;
+  const int nblk = k / 32, nquads = nblk / 4;
+  const uint8_t *__restrict__ wt = grp.w[blockIdx.y] + (size_t) blockIdx.x * nquads * kLoQuadBytes;
+  float *__restrict__         out = grp.out[blockIdx.y];
+  const int                   n0  = blockIdx.x * kLoRows;
+
+  auto fetch = [&](QuadRegs (&r)[kLoChunk], int q0) {  // quads q0, q0 + 8, ... of this wave (clamped: extra ones unused)
+#pragma unroll
+    for (int c = 0; c < kLoChunk; ++c) {
+      const int      q = min(q0 + c * kLoWaves, nquads - 1);
+      const uint8_t *p = wt + (size_t) q * kLoQuadBytes;
+      r[c].q           = *reinterpret_cast<const uint4 *>(p + lane * 16);
+      r[c].d           = *reinterpret_cast<const uint2 *>(p + 1024 + nl * 8);
+    }
+  };
+  // ---- the activation rows, as they are, by DMA: piece pc of row r goes to piece slot pc * 8 + r. Rows past m repeat
+  // row m - 1 (their results are never stored). The DMA instruction is written out so that the compiler does not make
+  // every later LDS read wait for all loads in flight. ----
+  const int      a_row    = nblk * 34;                 // bytes of an activation row, a multiple of 16
+  const int      a_pieces = kLoActRows * (a_row / 16);
+  const int      a_bytes  = (a_pieces * 16 + 1023) & ~1023;  // image size: whole DMA instructions
+  const uint32_t lds0     = (uint32_t) (uintptr_t) lo_lds;
+  for (int i = wave; i * kWave < a_pieces; i += kLoWaves) {
+    const int      s   = min(i * kWave + lane, a_pieces - 1), row = min(s % kLoActRows, m - 1), pc = s / kLoActRows;
+    const uint8_t *p   = act + (size_t) row * a_row + (size_t) pc * 16;
+    const uint32_t to  = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t) i * kWave * 16);
+    asm volatile("s_mov_b32 m0, %1\n s_nop 0\n global_load_lds_dwordx4 %0, off" ::"v"(p), "s"(to) : "memory");
+  }
+  QuadRegs cur[kLoChunk], nxt[kLoChunk];
+  fetch(cur, wave);  // 2 kLoChunk loads, in flight behind the DMA
+  // the DMA pieces of this wave have landed once only the weight loads issued after them are outstanding
+  // (s_waitcnt operand: vmcnt in bits 3:0 and 15:14, expcnt (7 = no wait) in 6:4, lgkmcnt in 11:8)
+  static_assert(2 * kLoChunk == 8, "the wait below leaves exactly the weight loads in flight");
+  __builtin_amdgcn_s_waitcnt(0x0070 | 8);
+  __builtin_amdgcn_s_barrier();  // (bare barriers: __syncthreads would also wait for the weight loads)
+  // block scales of all rows as floats: [block][row]
+  float *s_tab = reinterpret_cast<float *>(lo_lds + a_bytes);
+  for (int i = tid; i < nblk * kLoActRows; i += kLoThreads) {
+    const int blk = i / kLoActRows, row = i % kLoActRows, o = blk * 34;
+    s_tab[i]      = (float) *reinterpret_cast<const _Float16 *>(lo_lds + ((o >> 4) * kLoActRows + row) * 16 + (o & 15));
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the table is written; vmcnt untouched
+  __builtin_amdgcn_s_barrier();
+
+  // ---- this wave's quads, kLoChunk at a time, the next chunk in flight behind the current one ----
+  // LDS byte offsets of this lane's operand dwords in its first quad (row nl % 8, elements {4 g .., 16 + 4 g ..} of
+  // the quad's 4 blocks); the wave's next quad is 8 quads = 1088 B = 68 pieces of every row further on. Even blocks
+  // of a quad start 2 bytes off a dword (34 b + 2 with b even): two dwords and a funnel shift; odd blocks are aligned.
+  auto a_addr = [&](int o) { return ((o >> 4) * kLoActRows + (nl & 7)) * 16 + (o & 15); };
+  int  a_off[4][4];  // [block of the quad][dword]: even blocks use 4, odd blocks 2
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int o = (4 * wave + j) * 34 + 4 * g;  // byte 4 g of the block's row segment (its scale is bytes 0..1)
+    if (j % 2 == 0) {
+      a_off[j][0] = a_addr(o), a_off[j][1] = a_addr(o + 4), a_off[j][2] = a_addr(o + 16), a_off[j][3] = a_addr(o + 20);
+    } else {
+      a_off[j][0] = a_addr(o + 2), a_off[j][1] = a_addr(o + 18), a_off[j][2] = 0, a_off[j][3] = 0;
+    }
+  }
+  constexpr int kQuadStep  = kLoWaves * 4 * 34 / 16 * kLoActRows * 16;  // 8 quads further on in the image: 8704 B
+  constexpr int kScaleStep = kLoWaves * 4 * kLoScaleBlk;                // and in the scale table: 1024 B
+  static_assert(kLoWaves * 4 * 34 % 16 == 0, "a wave's quads are whole pieces apart");
+  const uint8_t *s_lane = lo_lds + a_bytes + 4 * wave * kLoScaleBlk + (g & 1) * 16;  // scales of rows 4 (g & 1) ..
+  float          acc[4] = { 0.0f, 0.0f, 0.0f, 0.0f };  // rows 4 g + j, column nl (lanes with g >= 2: unused rows)
+  // nibble -> int8 minus 8 without carries between bytes: (q + 0x78) ^ 0x80 per byte
+  auto lo = [](uint32_t q) { return ((q & 0x0f0f0f0fu) + 0x78787878u) ^ 0x80808080u; };
+  auto hi = [](uint32_t q) { return (((q >> 4) & 0x0f0f0f0fu) + 0x78787878u) ^ 0x80808080u; };
+  for (int q0 = wave; q0 < nquads; q0 += kLoChunk * kLoWaves) {
+    const bool more = q0 + kLoChunk * kLoWaves < nquads;
+    if (more) {
+      fetch(nxt, q0 + kLoChunk * kLoWaves);
+    }
+#pragma unroll
+    for (int c = 0; c < kLoChunk; ++c) {
+      const int quad = q0 + c * kLoWaves;
+      if (quad < nquads) {
+        const uint32_t wq[4] = { cur[c].q.x, cur[c].q.y, cur[c].q.z, cur[c].q.w };
+        union {
+          uint2    u;
+          _Float16 h[4];
+        } sc;
+        sc.u = cur[c].d;
+        const int      it  = (quad - wave) / kLoWaves;  // this quad is the wave's it-th
+        const uint8_t *img = lo_lds + (size_t) it * kQuadStep;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint32_t e0, e1;  // elements 4 g .. 4 g + 3 and 16 + 4 g .. 16 + 4 g + 3 of this lane's activation row
+          if (j % 2 == 0) {
+            e0 = __builtin_amdgcn_alignbyte(*reinterpret_cast<const uint32_t *>(img + a_off[j][1]),
+                                            *reinterpret_cast<const uint32_t *>(img + a_off[j][0]), 2);
+            e1 = __builtin_amdgcn_alignbyte(*reinterpret_cast<const uint32_t *>(img + a_off[j][3]),
+                                            *reinterpret_cast<const uint32_t *>(img + a_off[j][2]), 2);
+          } else {
+            e0 = *reinterpret_cast<const uint32_t *>(img + a_off[j][0]);
+            e1 = *reinterpret_cast<const uint32_t *>(img + a_off[j][1]);
+          }
+          const long   a = (long) (((uint64_t) e1 << 32) | e0);
+          const float4 s = *reinterpret_cast<const float4 *>(s_lane + (size_t) it * kScaleStep + j * kLoScaleBlk);
+          const long   b = (long) (((uint64_t) hi(wq[j]) << 32) | lo(wq[j]));
+          const v4i    zero = { 0, 0, 0, 0 };
+          const v4i    p    = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, zero, 0, 0, 0);
+          const float  dw   = (float) sc.h[j];
+          acc[0] += (float) p[0] * (s.x * dw);
+          acc[1] += (float) p[1] * (s.y * dw);
+          acc[2] += (float) p[2] * (s.z * dw);
+          acc[3] += (float) p[3] * (s.w * dw);
+        }
+      }
+    }
+    if (more) {
+#pragma unroll
+      for (int c = 0; c < kLoChunk; ++c) {
+        cur[c] = nxt[c];
+      }
+    }
+  }
+
+  // ---- add the eight waves in wave order (the panel is no longer needed) ----
+  __syncthreads();
+  float *red = reinterpret_cast<float *>(lo_lds);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    red[(wave * 4 + j) * kWave + lane] = acc[j];
+  }
+  __syncthreads();
+  if (tid < 4 * kWave) {
+    const int j = tid >> 6, l = tid & 63, row = 4 * (l >> 4) + j;
+    float     v = 0.0f;
+#pragma unroll
+    for (int w = 0; w < kLoWaves; ++w) {
+      v += red[(w * 4 + j) * kWave + l];
+    }
+    if ((l >> 4) < 2 && row < m) {
+      out[(size_t) row * n + n0 + (l & 15)] = v;
+    }
+  }
+}
+
+// LDS of a workgroup: the activation rows in whole DMA instructions, the scale table; later the waves' sums
+size_t panel_bytes(int k) {
+  const size_t nblk  = (size_t) k / 32;
+  const size_t image = ((kLoActRows * (nblk * 34 / 16) * 16) + 1023) & ~(size_t) 1023;
+  const size_t panel = image + nblk * kLoScaleBlk, red = (size_t) kLoWaves * 4 * kWave * sizeof(float);
+  return panel > red ? panel : red;
+}
+
+}  // namespace
+
+bool matmul_lane_order_fits(int n, int m, int k, WeightType wt) {
+  // k % 256: activation rows (34 B per 32 elements) are whole 16-byte pieces, weight rows whole quads of blocks
+  return wt == kQ4_0 && m >= 2 && m <= kLoActRows && k > 0 && k % 256 == 0 && n > 0 && n % kLoRows == 0 &&
+         panel_bytes(k) <= kLoLdsLimit && n / kLoRows <= 0x7fffffff;
+}
+
+size_t matmul_lane_order_weight_bytes(int k, int n) {
+  return (size_t) (n / kLoRows) * (size_t) (k / 128) * kLoQuadBytes;
+}
+
+hipError_t launch_q4_0_to_lane_order(hipStream_t stream, void *dst, const void *weight, int k, int n) {
+  if (k % 128 != 0 || n % kLoRows != 0) {
+    return hipErrorNotSupported;
+  }
+  const size_t items = (size_t) (n / kLoRows) * (size_t) (k / 128) * 64;
+  hipLaunchKernelGGL(q4_0_to_lane_order_kernel, dim3((unsigned) ((items + 255) / 256)), dim3(256), 0, stream,
+                     static_cast<uint8_t *>(dst), static_cast<const uint8_t *>(weight), k / 32, n);
+  return hipGetLastError();
+}
+
+hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *const *outs, const void *act,
+                                          const void *const *lane_order_weights, const int *ns, int m, int k) {
+  if (count < 1 || count > kGemvGroupMax) {
+    return hipErrorNotSupported;
+  }
+  LaneOrderGroupArgs grp = {};
+  int                n_max = 0;
+  for (int i = 0; i < count; ++i) {
+    if (!matmul_lane_order_fits(ns[i], m, k, kQ4_0) || (reinterpret_cast<uintptr_t>(lane_order_weights[i]) & 15) != 0 ||
+        (reinterpret_cast<uintptr_t>(act) & 15) != 0) {
+      return hipErrorNotSupported;
+    }
+    grp.w[i]   = static_cast<const uint8_t *>(lane_order_weights[i]);
+    grp.out[i] = outs[i];
+    grp.n[i]   = ns[i];
+    n_max      = ns[i] > n_max ? ns[i] : n_max;
+  }
+  static bool attr_set = false;  // more than the default 64 KiB of dynamic LDS for long rows
+  if (!attr_set) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(matmul_lane_order_kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int) kLoLdsLimit);
+    if (e != hipSuccess) {
+      return e;
+    }
+    attr_set = true;
+  }
+  const dim3 grid((unsigned) (n_max / kLoRows), (unsigned) count);
+  hipLaunchKernelGGL(matmul_lane_order_kernel, grid, dim3(kLoThreads), panel_bytes(k), stream, grp,
+                     static_cast<const uint8_t *>(act), m, k);
+  return hipGetLastError();
+}
+
+}  // namespace htpops
