@@ -322,6 +322,54 @@ def test_gemm_mfma_integer_exact(ctx, wt):
     assert np.array_equal(got, (qa.astype(np.int64) @ qw.astype(np.int64).T).astype(np.float32))
 
 
+@pytest.mark.parametrize("m,k,n", [(2, 256, 16), (8, 256, 48), (3, 512, 4096), (8, 4096, 4096), (5, 11008, 272), (8, 2048 + 256, 1024),
+                                   (7, 8960, 1536)])
+def test_few_rows_over_repacked_weights(ctx, oracle, monkeypatch, m, k, n):
+    # 2..8 rows against Q4_0 weights with n % 16 == 0, k % 256 == 0 run on a copy of the weights repacked into
+    # matrix-core operand order. It must meet the oracle, agree with the kernels that read the weights as they are
+    # (switch HTPOPS_LANE_ORDER=0) to summation order, and repeat bit for bit.
+    rng = wl.rng_for(66, m * 17 + k + n)
+    got, x, w = check_mat_mul(ctx, oracle, rng, m, k, n, wl.GGML_TYPE_Q4_0)
+    a = oracle.quantize_q8_0(x)
+    assert np.array_equal(ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0), got)
+    _, mag = oracle.mat_mul_q8_0_act_f64(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
+    monkeypatch.setenv("HTPOPS_LANE_ORDER", "0")
+    plain = ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
+    assert np.all(np.abs(plain - got) <= 2 * MATMUL_RTOL * mag)
+
+
+def test_few_rows_repacked_weights_extremes_and_cache(ctx, oracle):
+    # every weight -8 against every activation -127 with unit scales: 32512 per block, exact in fp32 for k = 512;
+    # then the cached repacked copy must follow a rewrite of the weight buffer, and caller-owned memory (nothing
+    # cached, the weights are read as they are) must give the same values
+    m, k, n = 8, 512, 64
+    one = np.array([1.0], np.float16).view(np.uint8)
+    w = np.zeros((n, k // 32, 18), np.uint8)
+    w[:, :, 0:2] = one
+    a = np.empty((m, k // 32, 34), np.uint8)
+    a[:, :, 0:2] = one
+    a[:, :, 2:] = np.int8(-127).view(np.uint8)
+    w, a = w.reshape(n, -1), a.reshape(m, -1)
+    ha, hw, ho = ctx.upload(a), ctx.upload(w), ctx.alloc(m * n * 4)
+    alias = ctx.register(ctx.device_ptr(hw), w.nbytes)
+    try:
+        def run(h):
+            assert ctx.execute(api.HTP_OPS_MAT_MUL_Q4_0_Q8_0, api.mat_mul_params((ho, 0), (ha, 0), (h, 0), m, k, n)) == 0
+            ctx.synchronize()
+            return ctx.read(ho, np.float32, m * n).reshape(m, n)
+        assert np.array_equal(run(hw), np.full((m, n), 32512.0 * (k // 32), np.float32))
+        rng = wl.rng_for(67, 0)
+        w2 = wl.make_q4_0_weights(rng, n, k)
+        a2 = oracle.quantize_q8_0(wl.make_activations(rng, m, k))
+        ctx.write(hw, w2), ctx.write(ha, a2)
+        want, mag = oracle.mat_mul_q8_0_act_f64(a2, w2, m, k, n, wl.GGML_TYPE_Q4_0)
+        assert np.all(np.abs(run(hw) - want) <= MATMUL_RTOL * mag)
+        assert np.all(np.abs(run(alias) - want) <= MATMUL_RTOL * mag)
+    finally:
+        for h in (alias, ha, hw, ho):
+            ctx.release(h)
+
+
 @pytest.fixture
 def fp6_kernel(monkeypatch):
     """Forces the FP6 many-row kernel (by default it only takes shapes that fill the device with whole tiles)."""
