@@ -38,7 +38,7 @@ __device__ __forceinline__ float fast_exp2(float x) {
 
 // ------------------------------------------------------------------------------------------------ prefill
 
-constexpr int kPfThreads = 256;
+constexpr int kPfThreads = 256;  // threads of one key group: 4 waves, one per query head
 constexpr int kBQ        = 32;  // query rows per wave tile
 constexpr int kBK        = 64;  // keys per KV block
 
@@ -51,24 +51,31 @@ struct PrefillSmem {
   _Float16 vt[D][kBK + 4];
 };
 
-template <int D, bool QO_F32>
-__global__ __launch_bounds__(kPfThreads) void flash_attn_prefill_kernel(void *__restrict__ o_ptr,
+// GROUPS = 1 or 2 key groups per workgroup (4 waves each); with 2 they take alternate KV blocks of the same queries
+template <int D, bool QO_F32, int GROUPS>
+__global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(void *__restrict__ o_ptr,
                                                                         const void *__restrict__ q_ptr,
                                                                         const _Float16 *__restrict__ k_ptr,
                                                                         const _Float16 *__restrict__ v_ptr,
                                                                         const _Float16 *__restrict__ mask, int qo_len,
                                                                         int kv_len, int n_heads, int n_kv_heads,
                                                                         int causal) {
-  __shared__ PrefillSmem<D> sm;
+  __shared__ PrefillSmem<D> sm_all[GROUPS];
   constexpr int KSTEPS = D / 16;  // MFMA k-steps over the head dimension
   constexpr int DT     = D / 32;  // 32-row tiles of O^T
+  // With GROUPS = 2, two groups of 4 waves work on the same queries and heads: group g takes KV blocks g, g + 2, ...
+  // with its own K/V tiles in LDS and its own running (max, sum, O); the two states are merged through LDS at the
+  // end. The longest workgroup then walks half as many iterations, which pays when the grid is too small to keep two
+  // independent workgroups on every CU busy to the end (few query blocks, or the uneven lengths under `causal`).
+  const int           grp = threadIdx.x / kPfThreads;
+  PrefillSmem<D>     &sm  = sm_all[grp];
 
   const int group = n_heads / n_kv_heads;
   const int gc    = group < 4 ? group : 4;  // heads handled by one workgroup
   const int qsub  = 4 / gc;                 // query sub-blocks per workgroup (waves left over when group < 4)
   const int sub_groups = (group + gc - 1) / gc;
 
-  const int tid  = threadIdx.x;
+  const int tid  = threadIdx.x % kPfThreads;  // within the key group
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int half = lane >> 5;
@@ -175,35 +182,42 @@ __global__ __launch_bounds__(kPfThreads) void flash_attn_prefill_kernel(void *__
       vreg[j][1] = *reinterpret_cast<const v8h *>(v_ptr + (size_t) kg1 * kv_stride + (size_t) h_kv * D + c * 8);
     }
   };
-  if (kv_limit > 0) {
-    fetch(0);
+  if (grp * kBK < kv_limit) {
+    fetch(grp * kBK);
   }
 
-  for (int k0 = 0; k0 < kv_limit; k0 += kBK) {
+  for (int kk = 0; kk < kv_limit; kk += GROUPS * kBK) {
+    const int  k0   = kk + grp * kBK;  // this key group's block of the iteration
+    const bool live = k0 < kv_limit;   // (the last iteration may have a block for the first group only)
     __syncthreads();  // previous block's fragments are no longer needed
     // ---- stage K [key][D] and V^T [d][key] from the registers ----
+    if (live) {
 #pragma unroll
-    for (int j = 0; j < K_PIECES; ++j) {
-      const int i   = tid + j * kPfThreads;
-      const int key = i / (D / 8), part = i % (D / 8);
-      *reinterpret_cast<v8h *>(&sm.k[key][part * 8]) = kreg[j];
-    }
+      for (int j = 0; j < K_PIECES; ++j) {
+        const int i   = tid + j * kPfThreads;
+        const int key = i / (D / 8), part = i % (D / 8);
+        *reinterpret_cast<v8h *>(&sm.k[key][part * 8]) = kreg[j];
+      }
 #pragma unroll
-    for (int j = 0; j < V_TASKS; ++j) {
-      // two keys of one 8-wide d chunk: eight 4-byte transposed stores
-      const int i = tid + j * kPfThreads;
-      const int c = i % (D / 8), kp = i / (D / 8);
+      for (int j = 0; j < V_TASKS; ++j) {
+        // two keys of one 8-wide d chunk: eight 4-byte transposed stores
+        const int i = tid + j * kPfThreads;
+        const int c = i % (D / 8), kp = i / (D / 8);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int d   = c * 8 + e;
-        const int pos = (2 * kp + 8 * (d / 32)) % kBK;
-        v2h       pr  = { vreg[j][0][e], vreg[j][1][e] };
-        *reinterpret_cast<v2h *>(&sm.vt[d][pos]) = pr;
+        for (int e = 0; e < 8; ++e) {
+          const int d   = c * 8 + e;
+          const int pos = (2 * kp + 8 * (d / 32)) % kBK;
+          v2h       pr  = { vreg[j][0][e], vreg[j][1][e] };
+          *reinterpret_cast<v2h *>(&sm.vt[d][pos]) = pr;
+        }
       }
     }
     __syncthreads();
-    if (k0 + kBK < kv_limit) {
-      fetch(k0 + kBK);
+    if (k0 + GROUPS * kBK < kv_limit) {
+      fetch(k0 + GROUPS * kBK);
+    }
+    if (!live) {
+      continue;
     }
 
     // ---- S^T - m = K Q^T - m: two 32-key tiles, accumulated on top of minus the running maximum ----
@@ -334,8 +348,43 @@ __global__ __launch_bounds__(kPfThreads) void flash_attn_prefill_kernel(void *__
     }
   }
 
+  // ---- the second key group hands its state over: m, l and O of the same query, lane for lane ----
+  float l_tot = l_run + __shfl_xor(l_run, 32, kWave);
+  if constexpr (GROUPS == 2) {
+    constexpr int STATE = 16 * DT + 2;  // floats per lane
+    static_assert((size_t) (kPfThreads / kWave) * STATE * kWave * sizeof(float) <= sizeof(sm_all),
+                  "the handed-over state fits the K/V tiles");
+    float *xch = reinterpret_cast<float *>(&sm_all[0]) + (size_t) wave * STATE * kWave + lane;
+    __syncthreads();  // everybody is done with the tiles
+    if (grp == 1) {
+      xch[0] = m_run, xch[kWave] = l_tot;
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          xch[(2 + 16 * t + r) * kWave] = oacc[t][r];
+        }
+      }
+    }
+    __syncthreads();
+    if (grp == 1) {
+      return;
+    }
+    const float m1 = xch[0], l1 = xch[kWave];
+    const float m_all  = fmaxf(m_run, m1);
+    const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;  // nothing visible at all: keep the exponents finite
+    const float a0 = fast_exp2(m_run - m_safe), a1 = fast_exp2(m1 - m_safe);
+    l_tot          = a0 * l_tot + a1 * l1;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        oacc[t][r] = a0 * oacc[t][r] + a1 * xch[(2 + 16 * t + r) * kWave];
+      }
+    }
+  }
+
   // ---- finish: O = O^T / l, one query per lane; register r of tile t is d = 32 t + 8 (r / 4) + 4 half + r % 4 ----
-  const float l_tot = l_run + __shfl_xor(l_run, 32, kWave);
   const float inv   = 1.0f / l_tot;
   if (q_ok) {
     const size_t base = (size_t) q_row * qo_stride + (size_t) head * D;
@@ -757,9 +806,23 @@ hipError_t launch_prefill(hipStream_t stream, void *o, const void *q, const void
     return hipErrorInvalidValue;
   }
   const dim3 grid((unsigned) (n_kv_heads * sub_groups), q_blocks);
-  hipLaunchKernelGGL((flash_attn_prefill_kernel<D, QO_F32>), grid, dim3(kPfThreads), 0, stream, o, q,
-                     (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, qo_len, kv_len, n_heads,
-                     n_kv_heads, causal ? 1 : 0);
+  // Two key groups per workgroup when the grid leaves CUs without a second workgroup, or (causal) when the workgroups
+  // all fit at once and their uneven lengths would leave the long ones running alone. Measured on the 256-CU device,
+  // 32 query / 8 KV heads of 128: 2048 x 2048 causal 67 us against 73 us, 1024 x 2048 65 against 72 us; but
+  // 2048 x 2048 without `causal` 117 against 107 us and 4096 x 4096 causal 242 against 214 us.
+  constexpr unsigned kCus = 256;
+  const unsigned     wgs  = grid.x * grid.y;
+  const int          forced = env_int("HTPOPS_ATTN_KEY_GROUPS", 0);  // 1 or 2: for tests and measurements
+  const bool         two  = forced ? forced == 2 : (wgs <= kCus || (causal && wgs <= 2 * kCus));
+  if (two) {
+    hipLaunchKernelGGL((flash_attn_prefill_kernel<D, QO_F32, 2>), grid, dim3(kPfThreads * 2), 0, stream, o, q,
+                       (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, qo_len, kv_len, n_heads,
+                       n_kv_heads, causal ? 1 : 0);
+  } else {
+    hipLaunchKernelGGL((flash_attn_prefill_kernel<D, QO_F32, 1>), grid, dim3(kPfThreads), 0, stream, o, q,
+                       (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, qo_len, kv_len, n_heads,
+                       n_kv_heads, causal ? 1 : 0);
+  }
   return hipGetLastError();
 }
 

@@ -57,6 +57,21 @@ def test_fp16_op_with_causal_flag(ctx, oracle, qo, kv, nh, nkv, d):
     assert np.abs(got.astype(np.float32) - masked.astype(np.float32)).max() <= 1e-3
 
 
+@pytest.mark.parametrize("groups", ["1", "2"])
+@pytest.mark.parametrize("qo,kv,nh,nkv,d", [(40, 300, 4, 1, 128), (33, 517, 4, 4, 128), (64, 96, 2, 1, 64), (70, 200, 8, 2, 128),
+                                            (128, 129, 8, 2, 128)])
+def test_prefill_with_one_and_two_key_groups(ctx, oracle, monkeypatch, groups, qo, kv, nh, nkv, d):
+    # the prefill kernel runs its KV blocks in one or two key groups per workgroup depending on the grid; both must
+    # meet the oracle on every shape (odd block counts leave the second group idle in the last iteration)
+    monkeypatch.setenv("HTPOPS_ATTN_KEY_GROUPS", groups)
+    rng = wl.rng_for(63, qo * 1000 + kv + nh)
+    q, k, v = wl.make_attention_inputs(rng, qo, kv, nh, nkv, d)
+    for causal, mask in ((True, None), (False, wl.make_causal_mask(qo, kv)), (False, None)):
+        got = ctx.run_flash_attn(q, k, v, mask, nh, nkv, d, causal=causal)
+        want = oracle.flash_attn(q, k, v, mask, nh, nkv, d, causal)
+        assert np.abs(got.astype(np.float32) - want.astype(np.float32)).max() <= ATOL
+
+
 def test_fixtures_from_the_reference_routine(ctx, golden_dir):
     files = sorted(glob.glob(os.path.join(golden_dir, "naive_flash_attn_*.npz")))
     assert len(files) >= 3
