@@ -13,7 +13,7 @@ The same run also measures, and reports inside the JSON line:
                 against 8 TB/s
   prefill_gemm  m = 512 Q4_0 GEMM, both shapes of config 2, in int8 Tera-ops/s (2 m n k per launch)
   small_batch   the same layer at m = 8
-  q8_0_block    the Qwen2-1.5B-like Q8_0 block of config 4 at m = 1
+  q8_0_block    the Qwen2-1.5B-like Q8_0 block of config 4 at m = 1 and m = 128
   attention     config 3: decode (1 x 4096) and causal prefill (2048 x 2048), 32 query / 8 KV heads of 128, fp16
   launches      the four kernel launches of the step one by one (q+k+v, o, gate+up, down) on cold weights
   cpu_baseline  the scalar C oracle (a port of the same arithmetic) on the host cores, same layer, m = 1
@@ -232,7 +232,7 @@ def main():
         log("prefill GEMM m=512 n=%d k=%d: %.1f us  %.1f Tops (%.1f%% of 5 Pop/s)" % (n, k, us, tops, tops / 50))
         ctx.release(ha), ctx.release(ho)
 
-    # ------------------------------------------------------------------ Q8_0 block (config 4), m = 1
+    # ------------------------------------------------------------------ Q8_0 block (config 4), m = 1 and m = 128
     # same protocol as the headline step: one message per layer, 8 layers of distinct weights (8 x 49.7 MB) rotated
     rng4 = wl.rng_for(4, 0)
     shapes8 = wl.QWEN2_1P5B_LAYER
@@ -240,34 +240,43 @@ def main():
     for _, n, k in shapes8:
         if (n, k) not in uniq8:
             uniq8[(n, k)] = wl.make_q8_0_weights(rng4, n, k)
-    act8 = {g: ctx.run_quantize_q8_0(wl.make_activations(rng4, 1, k)) for g, k in {0: 1536, 1: 1536, 2: 1536, 3: 8960}.items()}
-    h_act8 = {g: ctx.upload(a) for g, a in act8.items()}
     layers8 = [[ctx.upload(uniq8[(n, k)]) for _, n, k in shapes8] for _ in range(LAYERS)]
-    h_out8 = [ctx.alloc(n * 4) for _, n, _ in shapes8]
-    msgs8 = [api.build_message([(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
-        api.HTP_OPS_MAT_MUL_Q8_0_Q8_0,
-        api.mat_mul_params((h_out8[i], 0), (h_act8[ACT_OF[name]], 0), (layers8[l][i], 0), 1, k, n)))
-        for i, (name, n, k) in enumerate(shapes8)]) for l in range(LAYERS)]
-    assert ctx.process_message(msgs8[0]) == 0
-    check_states(msgs8[0])
-    for i, (name, n, k) in enumerate(shapes8):
-        got = ctx.read(h_out8[i], np.float32, n)
-        rows = np.unique(np.linspace(0, n - 1, 64).astype(int))
-        want, mag = orc.mat_mul_q8_0_act_f64(act8[ACT_OF[name]], uniq8[(n, k)][rows], 1, k, len(rows), Q8)
-        assert np.all(np.abs(got[rows] - want[0]) <= 1e-5 * mag[0]), "Q8_0 matmul %s outside 1e-5 relative" % name
-    for s_ in range(20):
-        ctx.enqueue_message(msgs8[s_ % LAYERS])
-    ctx.synchronize()
-    ctx.timer_start()
-    for s_ in range(200):
-        ctx.enqueue_message(msgs8[s_ % LAYERS])
-    q8_us = ctx.timer_stop_ms() * 1e3 / 200
-    for msg in msgs8:
-        ctx.finish_message(msg)
-        check_states(msg)
-    q8_bytes = sum(wl.matmul_algorithmic_bytes(1, k, n, Q8) for _, n, k in shapes8)
-    log("Q8_0 block m=1: %.1f us/step (7 GEMVs in 4 launches), %.0f GB/s" % (q8_us, q8_bytes / q8_us / 1e3))
-    for h in [h for l in layers8 for h in l] + h_out8 + list(h_act8.values()):
+    q8_block = {}
+    for m8, steps8 in ((1, 200), (128, 40)):
+        act8 = {g: ctx.run_quantize_q8_0(wl.make_activations(rng4, m8, k)) for g, k in {0: 1536, 1: 1536, 2: 1536, 3: 8960}.items()}
+        h_act8 = {g: ctx.upload(a) for g, a in act8.items()}
+        h_out8 = [ctx.alloc(m8 * n * 4) for _, n, _ in shapes8]
+        msgs8 = [api.build_message([(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
+            api.HTP_OPS_MAT_MUL_Q8_0_Q8_0,
+            api.mat_mul_params((h_out8[i], 0), (h_act8[ACT_OF[name]], 0), (layers8[l][i], 0), m8, k, n)))
+            for i, (name, n, k) in enumerate(shapes8)]) for l in range(LAYERS)]
+        assert ctx.process_message(msgs8[0]) == 0
+        check_states(msgs8[0])
+        for i, (name, n, k) in enumerate(shapes8):
+            got = ctx.read(h_out8[i], np.float32, m8 * n).reshape(m8, n)
+            rows = np.unique(np.linspace(0, n - 1, 64).astype(int))
+            arow = np.unique(np.linspace(0, m8 - 1, 4).astype(int))
+            want, mag = orc.mat_mul_q8_0_act_f64(act8[ACT_OF[name]][arow], uniq8[(n, k)][rows], len(arow), k, len(rows), Q8)
+            assert np.all(np.abs(got[np.ix_(arow, rows)] - want) <= 1e-5 * mag), "Q8_0 matmul %s outside 1e-5 relative" % name
+        for s_ in range(max(LAYERS, steps8 // 10)):  # every layer once before the clock (converted weight copies)
+            ctx.enqueue_message(msgs8[s_ % LAYERS])
+        ctx.synchronize()
+        ctx.timer_start()
+        for s_ in range(steps8):
+            ctx.enqueue_message(msgs8[s_ % LAYERS])
+        q8_us = ctx.timer_stop_ms() * 1e3 / steps8
+        for msg in msgs8:
+            ctx.finish_message(msg)
+            check_states(msg)
+        q8_bytes = sum(wl.matmul_algorithmic_bytes(m8, k, n, Q8) for _, n, k in shapes8)
+        q8_ops = sum(2.0 * m8 * k * n for _, n, k in shapes8)
+        q8_block[m8] = {"m": m8, "us_per_step": round(q8_us, 2), "GBps": round(q8_bytes / q8_us / 1e3, 1),
+                        "tera_ops": round(q8_ops / q8_us / 1e6, 2)}
+        log("Q8_0 block m=%d: %.1f us/step (7 matmuls), %.0f GB/s, %.1f Tops" % (m8, q8_us, q8_bytes / q8_us / 1e3,
+                                                                               q8_ops / q8_us / 1e6))
+        for h in h_out8 + list(h_act8.values()):
+            ctx.release(h)
+    for h in [h for l in layers8 for h in l]:
         ctx.release(h)
 
     # ------------------------------------------------------------------ attention (config 3): 32 query / 8 KV heads, D = 128
@@ -371,7 +380,7 @@ def main():
         "small_batch": {"m": 8, "us_per_step": round(ms_step8 * 1e3, 2),
                         "GBps": round(layer_bytes[8] / ms_step8 / 1e6, 1)},
         "attention": attention,
-        "q8_0_block": {"m": 1, "us_per_step": round(q8_us, 2), "GBps": round(q8_bytes / q8_us / 1e3, 1)},
+        "q8_0_block": [q8_block[1], q8_block[128]],
         "peaks": peaks,
     }
     ctx.close()
