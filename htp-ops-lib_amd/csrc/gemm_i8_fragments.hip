@@ -16,7 +16,8 @@
 //             and block) and cached by the caller; Q4_0 grows from 0.5625 to 1.125 bytes per weight in that cache
 //   act       converted per call from block_q8_0 rows (a pure re-ordering)
 // A wave owns 64 x 64 outputs (2 x 2 units per block) and a share of K; the KSPLIT waves of one tile are summed
-// through LDS in a fixed order.
+// through LDS in a fixed order. Launches with too few such tiles to fill the chip use 32 x 32 tiles (one unit per
+// block) instead: four times the workgroups, each with a quarter of the vector-ALU work.
 #include "device_utils.h"
 #include "kernels.h"
 
@@ -106,57 +107,65 @@ __global__ __launch_bounds__(256) void act_to_i8_fragments_kernel(uint4 *__restr
 
 constexpr int kGiThreads = 256;
 constexpr int kGiWaves   = 4;
-constexpr int kGiDepth   = 2;  // fragment sets in flight per wave
+#ifndef GI_DEPTH_U1
+#define GI_DEPTH_U1 6
+#endif
+#ifndef GI_DEPTH_U2
+#define GI_DEPTH_U2 2
+#endif
 
+template <int U>
 struct FragSet {
-  uint4    a[2], b[2];
-  uint32_t da[2], dw[2];
+  uint4    a[U], b[U];
+  uint32_t da[U], dw[U];
 };
 
-// KSPLIT waves share one 64 x 64 tile (each takes every KSPLIT-th block); a workgroup holds 4 / KSPLIT tiles that are
-// neighbours along n (they read the same activation fragments).
-template <int KSPLIT>
+// KSPLIT waves share one tile of U x U units (each takes every KSPLIT-th block); a workgroup holds 4 / KSPLIT tiles
+// that are neighbours along n (they read the same activation fragments).
+template <int KSPLIT, int U>
 __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__restrict__ out,
                                                                        const uint4 *__restrict__ a_frag,
                                                                        const uint32_t *__restrict__ a_scale,
                                                                        const uint4 *__restrict__ b_frag,
                                                                        const uint32_t *__restrict__ b_scale, int m, int n,
                                                                        int nblk, int m_tiles, int n_tiles) {
+  // fragment sets in flight per wave: small tiles run one wave per SIMD and must cover the memory latency alone
+  constexpr int kGiDepth = U == 1 ? GI_DEPTH_U1 : GI_DEPTH_U2;
   constexpr int TILES = kGiWaves / KSPLIT;
-  __shared__ float red[TILES][KSPLIT - 1][4][16][64];  // partial accumulators of the waves with ks > 0
+  __shared__ float red[TILES][KSPLIT - 1][U * U][16][64];  // partial accumulators of the waves with ks > 0
 
   // the wave index (and everything derived from it) is made scalar so that fragment addresses are scalar base +
   // per-lane offset and cost no vector instructions in the loop
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ks = wave % KSPLIT, tw = wave / KSPLIT;
   const int c = lane & 31, h = lane >> 5;
-  // 64 x 64 tile of this wave, in units of 32: m tiles mt0, mt0 + 1; n tiles nt0, nt0 + 1
+  // tile of this wave, in units of 32: m tiles mt0 .. mt0 + U - 1; n tiles nt0 .. nt0 + U - 1
   // Workgroup ids go round-robin over the 8 XCDs (each with its own L2). All row blocks of one column group are
   // given consecutive slots of ONE XCD, so the weight fragments they share are fetched into that L2 once.
-  const int gy = (m_tiles + 1) / 2, gx = (n_tiles + 2 * TILES - 1) / (2 * TILES);
+  const int gy = (m_tiles + U - 1) / U, gx = (n_tiles + U * TILES - 1) / (U * TILES);
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
   const int by = slot % gy, bx = (slot / gy) * 8 + xcd;
   if (bx >= gx) {
     return;  // whole workgroup (the grid is padded to a multiple of 8 column groups)
   }
-  const int mt0 = by * 2, nt0 = (bx * TILES + tw) * 2;
+  const int mt0 = by * U, nt0 = (bx * TILES + tw) * U;
   const bool tile_ok = nt0 < n_tiles;  // mt0 < m_tiles by construction
 
-  const uint4    *ap[2], *bp[2];
-  const uint32_t *asp[2], *bsp[2];
+  const uint4    *ap[U], *bp[U];
+  const uint32_t *asp[U], *bsp[U];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < U; ++i) {
     const size_t mt = (size_t) min(mt0 + i, m_tiles - 1), nt = (size_t) min(nt0 + i, n_tiles - 1);
     ap[i]  = a_frag + mt * nblk * 64;
     bp[i]  = b_frag + nt * nblk * 64;
     asp[i] = a_scale + mt * nblk * 32;
     bsp[i] = b_scale + nt * nblk * 32;
   }
-  auto load = [&](FragSet &s, int kb_raw) {
+  auto load = [&](FragSet<U> &s, int kb_raw) {
     const size_t kb = (size_t) min(kb_raw, nblk - 1);  // branch-free: blocks past the end repeat the last one ...
     const uint32_t live = kb_raw < nblk ? 0xffffffffu : 0u;  // ... with activation scales of zero: they add nothing
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < U; ++i) {
       s.a[i]  = (ap[i] + kb * 64)[lane];
       s.b[i]  = (bp[i] + kb * 64)[lane];
       s.da[i] = (asp[i] + kb * 32)[c] & live;
@@ -164,11 +173,11 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__
     }
   };
 
-  v16f acc[2][2];
+  v16f acc[U][U];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < U; ++i) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < U; ++j) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         acc[i][j][r] = 0.0f;
@@ -176,7 +185,7 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__
     }
   }
 
-  FragSet ring[kGiDepth];
+  FragSet<U> ring[kGiDepth];
 #pragma unroll
   for (int d = 0; d < kGiDepth; ++d) {
     load(ring[d], ks + d * KSPLIT);
@@ -188,12 +197,12 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__
     const uint2 u = make_uint2(h == 0 ? packed : 0u, 0u);
     return __builtin_bit_cast(v4h, u);
   };
-  auto mfma_sum = [&](const FragSet &s, int i, int j) {
+  auto mfma_sum = [&](const FragSet<U> &s, int i, int j) {
     const v4i af = { (int) s.a[i].x, (int) s.a[i].y, (int) s.a[i].z, (int) s.a[i].w };
     const v4i bf = { (int) s.b[j].x, (int) s.b[j].y, (int) s.b[j].z, (int) s.b[j].w };
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, zi, 0, 0, 0);
   };
-  auto mfma_scale = [&](const FragSet &s, int i, int j) {
+  auto mfma_scale = [&](const FragSet<U> &s, int i, int j) {
     return __builtin_amdgcn_mfma_f32_32x32x8f16(scale_operand(s.da[i]), scale_operand(s.dw[j]), zf, 0, 0, 0);
   };
 
@@ -206,12 +215,13 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__
 #pragma unroll
     for (int d = 0; d < kGiDepth; ++d) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int      i = u >> 1, j = u & 1;
-        const v16i     sum_cur = sum_next;
-        const v16f     scl_cur = scl_next;
-        const FragSet &nx = u < 3 ? ring[d] : ring[(d + 1) % kGiDepth];
-        const int      ni = u < 3 ? (u + 1) >> 1 : 0, nj = u < 3 ? (u + 1) & 1 : 0;
+      for (int u = 0; u < U * U; ++u) {
+        constexpr int     LAST = U * U - 1;
+        const int         i = u / U, j = u % U;
+        const v16i        sum_cur = sum_next;
+        const v16f        scl_cur = scl_next;
+        const FragSet<U> &nx = u < LAST ? ring[d] : ring[(d + 1) % kGiDepth];
+        const int         ni = u < LAST ? (u + 1) / U : 0, nj = u < LAST ? (u + 1) % U : 0;
         // The empty volatile asm statements keep their program order and each pins the value it names: the next
         // unit's block sums exist (in registers of their own) before this unit's converts and fmas are done.
         sum_next = mfma_sum(nx, ni, nj);
@@ -238,12 +248,12 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__
   // ---- the waves of a tile: ks > 0 park their sums in LDS, ks == 0 adds them in order and stores ----
   if (ks > 0) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < U; ++i) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < U; ++j) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          red[tw][ks - 1][i * 2 + j][r][lane] = acc[i][j][r];
+          red[tw][ks - 1][i * U + j][r][lane] = acc[i][j][r];
         }
       }
     }
@@ -251,9 +261,9 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__
   __syncthreads();
   if (ks == 0 && tile_ok) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < U; ++i) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < U; ++j) {
         if (mt0 + i < m_tiles && nt0 + j < n_tiles) {
           const int col = (nt0 + j) * 32 + c;
 #pragma unroll
@@ -261,7 +271,7 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__
             float v = acc[i][j][r];
 #pragma unroll
             for (int s = 0; s < KSPLIT - 1; ++s) {
-              v += red[tw][s][i * 2 + j][r][lane];
+              v += red[tw][s][i * U + j][r][lane];
             }
             // D[row][col]: col = lane % 32, row = 8 (r / 4) + 4 (lane / 32) + r % 4
             const int row = (mt0 + i) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
@@ -313,7 +323,7 @@ hipError_t launch_weights_to_i8_fragments(hipStream_t stream, void *dst, const v
 }
 
 hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_fragments,
-                                    int m, int k, int n, void *act_fragments) {
+                                    int m, int k, int n, void *act_fragments, bool act_fragments_ready) {
   if (k % 32 != 0 || m <= 0 || n <= 0) {
     return hipErrorInvalidValue;
   }
@@ -323,27 +333,35 @@ hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *
   const uint4 *bf  = static_cast<const uint4 *>(weight_fragments);
   const uint32_t *bs = reinterpret_cast<const uint32_t *>(static_cast<const uint8_t *>(weight_fragments) +
                                                           round256((size_t) n_tiles * nblk * 1024));
-  const size_t a_pieces = (size_t) m_tiles * nblk * 64;
-  hipLaunchKernelGGL(act_to_i8_fragments_kernel, dim3((unsigned) ((a_pieces + 255) / 256)), dim3(256), 0, stream, af, as,
-                     static_cast<const uint16_t *>(act_q8_0), m, nblk, m_tiles);
-  if (hipError_t e = hipGetLastError(); e != hipSuccess) {
-    return e;
+  if (!act_fragments_ready) {
+    const size_t a_pieces = (size_t) m_tiles * nblk * 64;
+    hipLaunchKernelGGL(act_to_i8_fragments_kernel, dim3((unsigned) ((a_pieces + 255) / 256)), dim3(256), 0, stream, af,
+                       as, static_cast<const uint16_t *>(act_q8_0), m, nblk, m_tiles);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) {
+      return e;
+    }
   }
-  // enough waves for two per SIMD: split K four ways when the tile count alone gives fewer than ~1500 waves
+  // enough waves for two per SIMD: split K four ways when the tile count alone gives fewer than ~1500 waves; when even
+  // that leaves fewer than two workgroups per CU, 32 x 32 tiles
   const int    wave_tiles = ((m_tiles + 1) / 2) * ((n_tiles + 1) / 2);
   static const int forced = env_int("HTPOPS_GEMM_KSPLIT", 0);
-  const int    ksplit = forced ? forced : (wave_tiles * 2 < 1536 ? 4 : 2);
-  const unsigned gy = (unsigned) ((m_tiles + 1) / 2);
+  const int    forced_unit = env_int("HTPOPS_GEMM_TILE_UNITS", 0);  // read per call: tests run both tile sizes
+  const int    unit = forced_unit == 1 || forced_unit == 2 ? forced_unit : (wave_tiles < 512 ? 1 : 2);
+  const int    ksplit = unit == 1 ? 4 : forced ? forced : (wave_tiles * 2 < 1536 ? 4 : 2);
+  const unsigned gy = (unsigned) ((m_tiles + unit - 1) / unit);
   auto grid = [&](int tiles_per_wg) {
-    const unsigned gx = (unsigned) ((n_tiles + 2 * tiles_per_wg - 1) / (2 * tiles_per_wg));
+    const unsigned gx = (unsigned) ((n_tiles + unit * tiles_per_wg - 1) / (unit * tiles_per_wg));
     return dim3((gx + 7) / 8 * 8 * gy);
   };
-  if (ksplit == 4) {
-    hipLaunchKernelGGL(gemm_i8_fragments_kernel<4>, grid(1), dim3(kGiThreads), 0, stream, out, af, as, bf, bs, m, n, nblk,
-                       m_tiles, n_tiles);
+  if (unit == 1) {
+    hipLaunchKernelGGL((gemm_i8_fragments_kernel<4, 1>), grid(1), dim3(kGiThreads), 0, stream, out, af, as, bf, bs, m, n,
+                       nblk, m_tiles, n_tiles);
+  } else if (ksplit == 4) {
+    hipLaunchKernelGGL((gemm_i8_fragments_kernel<4, 2>), grid(1), dim3(kGiThreads), 0, stream, out, af, as, bf, bs, m, n,
+                       nblk, m_tiles, n_tiles);
   } else {
-    hipLaunchKernelGGL(gemm_i8_fragments_kernel<2>, grid(2), dim3(kGiThreads), 0, stream, out, af, as, bf, bs, m, n, nblk,
-                       m_tiles, n_tiles);
+    hipLaunchKernelGGL((gemm_i8_fragments_kernel<2, 2>), grid(2), dim3(kGiThreads), 0, stream, out, af, as, bf, bs, m, n,
+                       nblk, m_tiles, n_tiles);
   }
   return hipGetLastError();
 }

@@ -58,6 +58,16 @@ struct htpops_context {
   };
   std::vector<FragEntry> frag_cache;
 
+  // Which activations the int8 fragments at the start of `workspace` were made from. Only kept while one message is
+  // walked (requests of a message that multiply the same activations share one conversion); any other use of the
+  // workspace and any write into the source range clears it.
+  struct ActFragments {
+    const void *src       = nullptr;
+    size_t      src_bytes = 0;
+    int         m = 0, k = 0;
+  } act_fragments;
+  bool in_message = false;
+
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
 
   // mailbox channel
@@ -184,7 +194,10 @@ bool mul3(size_t a, size_t b, size_t c, size_t *out) {
   return true;
 }
 
-int ensure_workspace(htpops_context *ctx, size_t bytes) {
+int ensure_workspace(htpops_context *ctx, size_t bytes, bool keep_act_fragments = false) {
+  if (!keep_act_fragments || bytes > ctx->workspace_bytes) {
+    ctx->act_fragments.src = nullptr;
+  }
   if (bytes <= ctx->workspace_bytes) {
     return HTPOPS_OK;
   }
@@ -203,6 +216,12 @@ int ensure_workspace(htpops_context *ctx, size_t bytes) {
 
 void drop_fragments(htpops_context *ctx, const void *ptr, size_t bytes) {
   const uintptr_t lo = reinterpret_cast<uintptr_t>(ptr), hi = lo + bytes;
+  if (ctx->act_fragments.src) {
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(ctx->act_fragments.src);
+    if (a0 < hi && lo < a0 + ctx->act_fragments.src_bytes) {
+      ctx->act_fragments.src = nullptr;
+    }
+  }
   bool            synced = false;
   for (size_t i = 0; i < ctx->frag_cache.size();) {
     const auto     &e  = ctx->frag_cache[i];
@@ -223,7 +242,7 @@ void drop_fragments(htpops_context *ctx, const void *ptr, size_t bytes) {
 
 // an op is about to write [ptr, ptr + bytes): converted weights made from that range are stale
 void note_device_write(htpops_context *ctx, const void *ptr, size_t bytes) {
-  if (!ctx->frag_cache.empty() && ptr) {
+  if ((!ctx->frag_cache.empty() || ctx->act_fragments.src) && ptr) {
     drop_fragments(ctx, ptr, bytes);
   }
 }
@@ -342,6 +361,11 @@ bool in_owned_buffer(htpops_context *ctx, const void *ptr, size_t bytes) {
   return false;
 }
 
+bool ranges_overlap(const void *a, size_t a_bytes, const void *b, size_t b_bytes) {
+  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+  return a0 < b0 + b_bytes && b0 < a0 + a_bytes;
+}
+
 constexpr int kFragKindRowLayout = 100;  // + ggml type, to keep apart from the tile-permuted kinds 1..4
 
 // How one quantized matmul will run and how much of the context's workspace it needs.
@@ -422,6 +446,9 @@ MatMulPlan plan_mat_mul(htpops_context *ctx, const void *weight, int m, int k, i
 int run_mat_mul(htpops_context *ctx, MatMulPlan &plan, float *dst, const void *act, const void *weight, int m, int k,
                 int n, int wt, uint8_t *ws) {
   note_device_write(ctx, dst, (size_t) m * n * 4);
+  if (!plan.fragments || plan.fp6) {
+    ctx->act_fragments.src = nullptr;  // these kernels put something else at the start of the workspace
+  }
   if (!plan.fragments) {
     if (const void *lw = lane_order_weights(ctx, weight, m, k, n, wt)) {
       HTPOPS_HIP(ctx, htpops::launch_matmul_lane_order_group(ctx->stream, 1, &dst, act, &lw, &n, m, k));
@@ -456,7 +483,17 @@ int run_mat_mul(htpops_context *ctx, MatMulPlan &plan, float *dst, const void *a
     HTPOPS_HIP(ctx, htpops::launch_gemm_fp6_panels(ctx->stream, dst, act, frags, m, k, n, ws, partials, ctx->tickets, kTicketSlots));
     return HTPOPS_OK;
   }
-  HTPOPS_HIP(ctx, htpops::launch_gemm_i8_fragments(ctx->stream, dst, act, frags, m, k, n, ws));
+  // note_device_write above has already cleared the record if this matmul writes into its own activations
+  auto      &af    = ctx->act_fragments;
+  const bool ready = af.src == act && af.m == m && af.k == k && ws == ctx->workspace;
+  const bool keep  = ready || (ctx->in_message && ws == ctx->workspace &&
+                               in_owned_buffer(ctx, act, q8_0_bytes((size_t) m, (size_t) k)) &&
+                               !ranges_overlap(dst, (size_t) m * n * 4, act, q8_0_bytes((size_t) m, (size_t) k)));
+  af.src = nullptr;
+  HTPOPS_HIP(ctx, htpops::launch_gemm_i8_fragments(ctx->stream, dst, act, frags, m, k, n, ws, ready));
+  if (keep) {
+    af.src = act, af.src_bytes = q8_0_bytes((size_t) m, (size_t) k), af.m = m, af.k = k;
+  }
   return HTPOPS_OK;
 }
 
@@ -469,7 +506,7 @@ int op_mat_mul_q8(htpops_context *ctx, float *dst, const void *act, const void *
     return r;
   }
   MatMulPlan plan = plan_mat_mul(ctx, weight, m, k, n, weight_type);
-  if (int r = ensure_workspace(ctx, plan.ws_bytes)) {
+  if (int r = ensure_workspace(ctx, plan.ws_bytes, /*keep_act_fragments=*/true)) {
     return r;
   }
   return run_mat_mul(ctx, plan, dst, act, weight, m, k, n, weight_type, static_cast<uint8_t *>(ctx->workspace));
@@ -910,11 +947,6 @@ struct GemvBatch {
   int                   n[htpops::kGemvGroupMax];
 };
 
-bool ranges_overlap(const void *a, size_t a_bytes, const void *b, size_t b_bytes) {
-  const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
-  return a0 < b0 + b_bytes && b0 < a0 + a_bytes;
-}
-
 void flush_batch(htpops_context *ctx, GemvBatch &b) {
   if (b.count == 0) {
     return;
@@ -1033,6 +1065,8 @@ int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_b
     }
   }
   GemvBatch batch;
+  ctx->act_fragments.src = nullptr;
+  ctx->in_message        = true;
   for (int i = 0; i < n_reqs; ++i) {
     struct RequestHeader *hdr  = message_header_get_request_ptr(msg, i);
     const size_t          size = message_header_get_request_size(msg, i);
@@ -1073,6 +1107,8 @@ int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_b
     }
   }
   flush_batch(ctx, batch);
+  ctx->in_message        = false;
+  ctx->act_fragments.src = nullptr;
   return HTPOPS_OK;
 }
 

@@ -54,13 +54,14 @@ hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *
                                           const void *const *lane_order_weights, const int *ns, int m, int k);
 // many-row path: int8 MFMA over operands in fragment order. The weights are converted once
 // (launch_weights_to_i8_fragments into gemm_i8_weight_fragment_bytes) and can be cached by the caller; the
-// activations are converted per call into `act_fragments` (gemm_i8_act_fragment_bytes).
+// activations are converted per call into `act_fragments` (gemm_i8_act_fragment_bytes), unless the caller says that
+// buffer already holds the conversion of the same activations (`act_fragments_ready`).
 size_t     gemm_i8_weight_fragment_bytes(int k, int n);
 size_t     gemm_i8_act_fragment_bytes(int m, int k);
 hipError_t launch_weights_to_i8_fragments(hipStream_t stream, void *dst, const void *weight, int k, int n,
                                           WeightType wt);
 hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_fragments,
-                                    int m, int k, int n, void *act_fragments);
+                                    int m, int k, int n, void *act_fragments, bool act_fragments_ready);
 // many-row path for Q4_0 weights: FP6 scaled MFMA over operand panels (exact: int8 = 16 hi + lo, all parts |t| <= 15).
 // The weight panel (gemm_fp6_weight_panel_bytes) is converted once and can be cached by the caller; the activation
 // panel (gemm_fp6_act_panel_bytes) is scratch written per call.

@@ -322,6 +322,71 @@ def test_gemm_mfma_integer_exact(ctx, wt):
     assert np.array_equal(got, (qa.astype(np.int64) @ qw.astype(np.int64).T).astype(np.float32))
 
 
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+@pytest.mark.parametrize("m,k,n", [(128, 1536, 256), (129, 320, 65), (100, 11008, 96), (33, 2048, 70), (256, 4096, 512)])
+def test_gemm_mfma_with_small_and_large_tiles(ctx, oracle, monkeypatch, wt, m, k, n):
+    # launches with few output tiles run 32 x 32 tiles per workgroup, the others 64 x 64 (HTPOPS_GEMM_TILE_UNITS forces
+    # one or the other): both must meet the oracle on the same inputs
+    monkeypatch.setenv("HTPOPS_GEMM_FP6", "0")
+    got = {}
+    for units in ("1", "2"):
+        monkeypatch.setenv("HTPOPS_GEMM_TILE_UNITS", units)
+        got[units], _, _ = check_mat_mul(ctx, oracle, wl.rng_for(58, m * 131 + k + n + wt), m, k, n, wt)
+    scale = np.abs(got["1"]).max()
+    assert np.abs(got["1"] - got["2"]).max() <= 2e-5 * scale
+
+
+def test_message_shares_one_activation_conversion_between_many_row_matmuls(ctx, oracle):
+    # Many-row matmuls of one message that multiply the same activations reuse the converted copy of those
+    # activations. The copy must be dropped when a request of the message rewrites the activations, when another
+    # activation (or another kernel) takes the workspace, and at the end of the message. Every request must equal its
+    # own launch bit for bit.
+    rng = wl.rng_for(66, 0)
+    m, k = 96, 1536
+    wt = wl.GGML_TYPE_Q8_0
+    op = api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
+    ns = [256, 1536, 320]
+    ws = [wl.make_weights(rng, n, k, wt) for n in ns]
+    x1, x2, xb = (wl.make_activations(rng, m, k) for _ in range(3))
+    a1, a2, b = (oracle.quantize_q8_0(x) for x in (x1, x2, xb))
+    hx2 = ctx.upload(x2)
+    ha, hb = ctx.upload(a1), ctx.upload(b)
+    hws = [ctx.upload(w) for w in ws]
+    w1row = wl.make_weights(rng, 64, k, wt)  # a one-row matmul in between uses the workspace for something else
+    hw1 = ctx.upload(w1row)
+    ho1 = ctx.alloc(64 * 4)
+    # outputs: 0..2 = A (first contents) x W0..W2, 3..5 = A (second contents) x W0..W2, 6 = B x W0, 7 = A x W1, 8 = A x W2
+    out_ns = ns + ns + [ns[0], ns[1], ns[2]]
+    houts = [ctx.alloc(m * n * 4) for n in out_ns]
+    handles = [hx2, ha, hb, hw1, ho1] + hws + houts
+    mm = lambda ho, hact, hw, n: (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, api.mat_mul_params((ho, 0), (hact, 0), (hw, 0), m, k, n)))
+    try:
+        reqs = [mm(houts[i], ha, hws[i], ns[i]) for i in range(3)]
+        reqs += [(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(api.HTP_OPS_QUANTIZE_Q8_0, api.rms_norm_params((ha, 0), (hx2, 0), k, m)))]
+        reqs += [mm(houts[3 + i], ha, hws[i], ns[i]) for i in range(3)]
+        reqs += [mm(houts[6], hb, hws[0], ns[0]), mm(houts[7], ha, hws[1], ns[1])]
+        reqs += [(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, api.mat_mul_params((ho1, 0), (ha, 0), (hw1, 0), 1, k, 64)))]
+        reqs += [mm(houts[8], ha, hws[2], ns[2])]
+        msg = api.build_message(reqs)
+        for _ in range(2):
+            ctx.write(ha, a1)
+            assert ctx.process_message(msg) == 0
+            assert all(s == 0 for s in api.message_request_states(msg))
+            acts = [a1] * 3 + [a2] * 3 + [b, a2, a2]
+            wsel = [0, 1, 2, 0, 1, 2, 0, 1, 2]
+            for ho, act, wi, n in zip(houts, acts, wsel, out_ns):
+                got = ctx.read(ho, np.float32, m * n).reshape(m, n)
+                assert np.array_equal(got, ctx.run_mat_mul(act, ws[wi], m, k, n, wt)), "a request differs from its own launch"
+            assert np.array_equal(ctx.read(ha, np.uint8, a2.size).reshape(a2.shape), a2)
+            assert np.array_equal(ctx.read(ho1, np.float32, 64), ctx.run_mat_mul(a2[:1], w1row, 1, k, 64, wt)[0])
+        want64, mag = oracle.mat_mul_q8_0_act_f64(a2, ws[1], m, k, ns[1], wt)
+        got = ctx.read(houts[7], np.float32, m * ns[1]).reshape(m, ns[1])
+        assert np.all(np.abs(got - want64) <= MATMUL_RTOL * mag)
+    finally:
+        for h in handles:
+            ctx.release(h)
+
+
 @pytest.mark.parametrize("m,k,n", [(2, 256, 16), (8, 256, 48), (3, 512, 4096), (8, 4096, 4096), (5, 11008, 272), (8, 2048 + 256, 1024),
                                    (7, 8960, 1536)])
 def test_few_rows_over_repacked_weights(ctx, oracle, monkeypatch, m, k, n):
