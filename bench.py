@@ -13,6 +13,8 @@ The same run also measures, and reports inside the JSON line:
                 against 8 TB/s
   prefill_gemm  m = 512 Q4_0 GEMM, both shapes of config 2, in int8 Tera-ops/s (2 m n k per launch)
   small_batch   the same layer at m = 8
+  recorded_message_us_per_step   the m = 1 and m = 8 steps again, each layer's message recorded once into a HIP graph
+                and replayed (reported beside `value`, which is the ordinary message walk)
   q8_0_block    the Qwen2-1.5B-like Q8_0 block of config 4 at m = 1 and m = 128
   attention     config 3: decode (1 x 4096) and causal prefill (2048 x 2048), 32 query / 8 KV heads of 128, fp16
   launches      the four kernel launches of the step one by one (q+k+v, o, gate+up, down) on cold weights
@@ -153,9 +155,32 @@ def main():
             check_states(msg)
         return ev_ms / steps, wall_ms / steps
 
+    def time_recorded_layers(m, steps, warmup):
+        # the same steps, each layer's message recorded once into a HIP graph and re-enqueued with one call
+        msgs = [layer_message(l, m) for l in range(LAYERS)]
+        recs = []
+        for msg in msgs:
+            ret, rec = ctx.record_message(msg)
+            if ret != 0:
+                raise RuntimeError("record_message: %d %s" % (ret, ctx.last_error()))
+            check_states(msg)
+            recs.append(rec)
+        for s in range(warmup):
+            ctx.launch_recorded_message(recs[s % LAYERS])
+        ctx.synchronize()
+        ctx.timer_start()
+        for s in range(steps):
+            ctx.launch_recorded_message(recs[s % LAYERS])
+        ev_ms = ctx.timer_stop_ms()
+        for rec in recs:
+            ctx.release_recorded_message(rec)
+        return ev_ms / steps
+
     ms_step, wall_step = time_layers(1, args.steps, args.warmup)
+    rec_step = {1: time_recorded_layers(1, args.steps, args.warmup)}
     value = layer_bytes[1] / (ms_step * 1e-3) / 1e9
     log("layer m=1: %.2f us/step (events) %.2f us/step (wall)  %.0f GB/s" % (ms_step * 1e3, wall_step * 1e3, value))
+    log("layer m=1 as recorded messages: %.2f us/step" % (rec_step[1] * 1e3))
 
     # ------------------------------------------------------------------ the step's four launches, one by one
     def time_single(n, k, m, wt, handles, h_a, h_o, reps, op):
@@ -209,6 +234,8 @@ def main():
     # (every layer is touched before the clock starts: the first few-row use of a weight buffer repacks it once)
     ms_step8, _ = time_layers(8, max(20, args.steps // 4), LAYERS)
     log("layer m=8: %.2f us/step  %.0f GB/s" % (ms_step8 * 1e3, layer_bytes[8] / ms_step8 / 1e6))
+    rec_step[8] = time_recorded_layers(8, max(20, args.steps // 4), LAYERS)
+    log("layer m=8 as recorded messages: %.2f us/step" % (rec_step[8] * 1e3))
 
     # ------------------------------------------------------------------ prefill GEMM (config 2)
     prefill = []
@@ -379,6 +406,7 @@ def main():
         "prefill_gemm": prefill,
         "small_batch": {"m": 8, "us_per_step": round(ms_step8 * 1e3, 2),
                         "GBps": round(layer_bytes[8] / ms_step8 / 1e6, 1)},
+        "recorded_message_us_per_step": {"m1": round(rec_step[1] * 1e3, 2), "m8": round(rec_step[8] * 1e3, 2)},
         "attention": attention,
         "q8_0_block": [q8_block[1], q8_block[128]],
         "peaks": peaks,

@@ -16,6 +16,7 @@
 #include <cstring>
 #include <string>
 #include <thread>
+#include <utility>
 #include <vector>
 
 #include "kernels.h"
@@ -33,6 +34,14 @@ constexpr int kMaxHandles  = 1 << 20;
 constexpr int kTicketSlots = 1 << 16;
 
 }  // namespace
+
+struct htpops_recorded_message {
+  htpops_context *ctx   = nullptr;
+  hipGraph_t      graph = nullptr;
+  hipGraphExec_t  exec  = nullptr;  // null for a message without launches
+  bool            stale = false;
+  std::vector<std::pair<uintptr_t, size_t>> ranges;
+};
 
 struct htpops_context {
   int                 device     = HTPOPS_DEVICE_NONE;
@@ -67,6 +76,14 @@ struct htpops_context {
     int         m = 0, k = 0;
   } act_fragments;
   bool in_message = false;
+
+  // Recorded messages hold device addresses. Each keeps the buffer ranges its requests resolved to (collected through
+  // `collect_ranges` while it is recorded) and is marked stale when one of them is released, when a converted copy of
+  // weights in one of them is dropped, or when the workspace is replaced. `memory_generation` counts those events, so
+  // that a recording can tell whether one happened during its own recorded walk.
+  std::vector<htpops_recorded_message *>     recordings;
+  std::vector<std::pair<uintptr_t, size_t>> *collect_ranges = nullptr;
+  uint64_t                                   memory_generation = 0;
 
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
 
@@ -147,7 +164,24 @@ void *resolve(htpops_context *ctx, const struct RpcmemBufAddr &addr, size_t need
   if (off > b->size || need > b->size - off) {
     return nullptr;
   }
+  if (ctx->collect_ranges) {
+    ctx->collect_ranges->emplace_back(reinterpret_cast<uintptr_t>(b->ptr) + off, need);
+  }
   return static_cast<uint8_t *>(b->ptr) + off;
+}
+
+// memory in [ptr, ptr + bytes) is about to go (bytes = 0: the workspace, which every recording may use)
+void mark_recordings_stale(htpops_context *ctx, const void *ptr, size_t bytes) {
+  ++ctx->memory_generation;
+  const uintptr_t lo = reinterpret_cast<uintptr_t>(ptr);
+  for (htpops_recorded_message *rec : ctx->recordings) {
+    if (bytes == 0) {
+      rec->stale = true;
+    }
+    for (size_t i = 0; !rec->stale && i < rec->ranges.size(); ++i) {
+      rec->stale = rec->ranges[i].first < lo + bytes && lo < rec->ranges[i].first + rec->ranges[i].second;
+    }
+  }
 }
 
 bool aligned(const void *p, size_t a) {
@@ -201,6 +235,7 @@ int ensure_workspace(htpops_context *ctx, size_t bytes, bool keep_act_fragments 
   if (bytes <= ctx->workspace_bytes) {
     return HTPOPS_OK;
   }
+  mark_recordings_stale(ctx, nullptr, 0);
   if (ctx->workspace) {
     // kernels already enqueued may still use the old block
     HTPOPS_HIP(ctx, hipStreamSynchronize(ctx->stream));
@@ -232,6 +267,7 @@ void drop_fragments(htpops_context *ctx, const void *ptr, size_t bytes) {
         synced = true;
       }
       (void) hipFree(e.frag);
+      mark_recordings_stale(ctx, e.src, e.src_bytes);
       ctx->frag_cache[i] = ctx->frag_cache.back();
       ctx->frag_cache.pop_back();
     } else {
@@ -745,6 +781,7 @@ extern "C" int htpops_buffer_release(htpops_context *ctx, int handle) {
   }
   int ret = HTPOPS_OK;
   drop_fragments(ctx, b->ptr, b->size);
+  mark_recordings_stale(ctx, b->ptr, b->size);
   if (b->owned) {
     if (ctx->has_device) {
       hipError_t e = hipFree(b->ptr);  // waits for work that may still use the block
@@ -1043,9 +1080,8 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
   return true;
 }
 
-// Walks a message and enqueues every request in order (reference: src/dsp/commu.c:91-114). Returns 0 or the
-// framing error; per-request results go to RequestHeader.state.
-int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes) {
+// 0, or the error if the request table does not fit `msg_bytes` (0 = unknown size, offsets are trusted)
+int check_message_framing(htpops_context *ctx, const struct MessageHeader *msg, size_t msg_bytes) {
   const int n_reqs = msg->n_reqs;
   if (n_reqs < 0 || n_reqs > (1 << 20)) {
     return fail(ctx, HTPOPS_ERR_REJECTED, "message: n_reqs=%d", n_reqs);
@@ -1064,6 +1100,16 @@ int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_b
       prev = off;
     }
   }
+  return HTPOPS_OK;
+}
+
+// Walks a message and enqueues every request in order (reference: src/dsp/commu.c:91-114). Returns 0 or the
+// framing error; per-request results go to RequestHeader.state.
+int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes) {
+  if (int r = check_message_framing(ctx, msg, msg_bytes)) {
+    return r;
+  }
+  const int n_reqs = msg->n_reqs;
   GemvBatch batch;
   ctx->act_fragments.src = nullptr;
   ctx->in_message        = true;
@@ -1149,6 +1195,121 @@ extern "C" int htpops_process_message(htpops_context *ctx, struct MessageHeader 
     return ret;
   }
   return htpops_finish_message(ctx, msg);
+}
+
+// ------------------------------------------------------------------------------------------------ recorded messages
+
+extern "C" int htpops_record_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes,
+                                     htpops_recorded_message **out) {
+  if (!ctx || !msg || !out) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  *out = nullptr;
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  if (ctx->poller.joinable()) {
+    return fail(ctx, HTPOPS_ERR_BUSY, "record_message: the channel's consumer thread owns the stream");
+  }
+  if (int r = check_message_framing(ctx, msg, msg_bytes)) {
+    return r;
+  }
+  for (int i = 0; i < msg->n_reqs; ++i) {
+    // releasing handles is not something a replay could repeat
+    if (message_header_get_request_ptr(msg, i)->type == REQUEST_TYPE_RPCMEM_MAP) {
+      return fail(ctx, HTPOPS_ERR_REJECTED, "record_message: request %d releases buffers; only ops can be recorded", i);
+    }
+  }
+  // First walk, executed: sizes the workspace and makes every converted weight copy, so that the recorded walk
+  // allocates nothing.
+  if (int r = enqueue_message(ctx, msg, msg_bytes)) {
+    return r;
+  }
+  for (int i = 0; i < msg->n_reqs; ++i) {
+    const struct RequestHeader *hdr = message_header_get_request_ptr(msg, i);
+    if (hdr->type == REQUEST_TYPE_OP_COMPUTE && hdr->state != HTPOPS_OK) {
+      return fail(ctx, HTPOPS_ERR_REJECTED, "record_message: request %d failed with %d", i, (int) hdr->state);
+    }
+  }
+  HTPOPS_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  const uint64_t generation = ctx->memory_generation;
+  std::vector<std::pair<uintptr_t, size_t>> ranges;
+  HTPOPS_HIP(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+  ctx->collect_ranges = &ranges;
+  const int  walked   = enqueue_message(ctx, msg, 0);
+  ctx->collect_ranges = nullptr;
+  hipGraph_t graph    = nullptr;
+  hipError_t e        = hipStreamEndCapture(ctx->stream, &graph);
+  bool       all_ok = walked == HTPOPS_OK;
+  for (int i = 0; all_ok && i < msg->n_reqs; ++i) {
+    const struct RequestHeader *hdr = message_header_get_request_ptr(msg, i);
+    all_ok = hdr->type != REQUEST_TYPE_OP_COMPUTE || hdr->state == HTPOPS_OK;
+  }
+  if (e != hipSuccess || !all_ok || generation != ctx->memory_generation) {
+    (void) hipGetLastError();
+    if (graph) {
+      (void) hipGraphDestroy(graph);
+    }
+    return fail(ctx, HTPOPS_ERR_HIP, "record_message: the launches could not be captured (%s)",
+                e != hipSuccess ? hipGetErrorString(e) : "a request failed or memory moved during the recorded walk");
+  }
+  hipGraphExec_t exec = nullptr;  // stays null for a message without launches
+  size_t         nodes = 0;
+  if (graph && (hipGraphGetNodes(graph, nullptr, &nodes) != hipSuccess || nodes == 0)) {
+    (void) hipGetLastError();
+    (void) hipGraphDestroy(graph);
+    graph = nullptr;
+  }
+  if (graph) {
+    e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    if (e != hipSuccess) {
+      (void) hipGraphDestroy(graph);
+      return hip_fail(ctx, e, "hipGraphInstantiate");
+    }
+  }
+  auto *rec   = new htpops_recorded_message;
+  rec->ctx    = ctx;
+  rec->graph  = graph;
+  rec->exec   = exec;
+  rec->ranges = std::move(ranges);
+  ctx->recordings.push_back(rec);
+  *out = rec;
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_launch_recorded_message(htpops_context *ctx, htpops_recorded_message *rec) {
+  if (!ctx || !rec || rec->ctx != ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (rec->stale) {
+    return fail(ctx, HTPOPS_ERR_REJECTED,
+                "launch_recorded_message: buffers were released or rewritten since the message was recorded; record it again");
+  }
+  ctx->act_fragments.src = nullptr;
+  if (rec->exec) {
+    HTPOPS_HIP(ctx, hipGraphLaunch(rec->exec, ctx->stream));
+  }
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_release_recorded_message(htpops_context *ctx, htpops_recorded_message *rec) {
+  if (!ctx || !rec || rec->ctx != ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  (void) hipStreamSynchronize(ctx->stream);
+  if (rec->exec) {
+    (void) hipGraphExecDestroy(rec->exec);
+    (void) hipGraphDestroy(rec->graph);
+  }
+  for (size_t i = 0; i < ctx->recordings.size(); ++i) {
+    if (ctx->recordings[i] == rec) {
+      ctx->recordings[i] = ctx->recordings.back();
+      ctx->recordings.pop_back();
+      break;
+    }
+  }
+  delete rec;
+  return HTPOPS_OK;
 }
 
 // ------------------------------------------------------------------------------------------------ channel

@@ -50,7 +50,8 @@ EXPORTED_SYMBOLS = [
     "htpops_init_backend", "htpops_close", "htpops_last_error", "htpops_synchronize", "htpops_get_stream",
     "htpops_buffer_alloc", "htpops_buffer_register", "htpops_buffer_release", "htpops_buffer_device_ptr",
     "htpops_buffer_size", "htpops_buffer_write", "htpops_buffer_read", "htpops_execute_op",
-    "htpops_process_message", "htpops_enqueue_message", "htpops_finish_message", "htpops_create_channel", "htpops_destroy_channel", "htpops_rms_norm_f32",
+    "htpops_process_message", "htpops_enqueue_message", "htpops_finish_message",
+    "htpops_record_message", "htpops_launch_recorded_message", "htpops_release_recorded_message", "htpops_create_channel", "htpops_destroy_channel", "htpops_rms_norm_f32",
     "htpops_mat_mul_permuted_w16a32", "htpops_rms_norm_f32_ex_ptr", "htpops_quantize_q8_0_ptr",
     "htpops_rms_norm_quantize_q8_0_ptr", "htpops_mat_mul_q8_0_act_ptr", "htpops_mat_mul_f32_act_ptr",
     "htpops_flash_attn_ptr", "htpops_timer_start", "htpops_timer_stop", "htpops_timer_elapsed_ms",
@@ -88,6 +89,9 @@ def load_library(path=None):
         "htpops_process_message": (ci, [vp, vp, sz]),
         "htpops_enqueue_message": (ci, [vp, vp, sz]),
         "htpops_finish_message": (ci, [vp, vp]),
+        "htpops_record_message": (ci, [vp, vp, sz, ctypes.POINTER(vp)]),
+        "htpops_launch_recorded_message": (ci, [vp, vp]),
+        "htpops_release_recorded_message": (ci, [vp, vp]),
         "htpops_create_channel": (ci, [vp, vp, sz]),
         "htpops_destroy_channel": (ci, [vp]),
         "htpops_rms_norm_f32": (ci, [vp, ci, ci, ci, ci, ci, ci]),
@@ -259,6 +263,19 @@ class Context:
     def finish_message(self, msg):
         buf = (ctypes.c_char * len(msg)).from_buffer(msg)
         return self.lib.htpops_finish_message(self._ctx, ctypes.cast(buf, ctypes.c_void_p))
+
+    def record_message(self, msg):
+        """htpops_record_message: runs `msg` once and returns (code, recording); the recording is None on failure."""
+        buf = (ctypes.c_char * len(msg)).from_buffer(msg)
+        rec = ctypes.c_void_p()
+        ret = self.lib.htpops_record_message(self._ctx, ctypes.cast(buf, ctypes.c_void_p), len(msg), ctypes.byref(rec))
+        return ret, (rec if ret == 0 else None)
+
+    def launch_recorded_message(self, rec):
+        return self.lib.htpops_launch_recorded_message(self._ctx, rec)
+
+    def release_recorded_message(self, rec):
+        return self.lib.htpops_release_recorded_message(self._ctx, rec)
 
     # -- timing --
     def timer_start(self):

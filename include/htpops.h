@@ -96,6 +96,25 @@ int htpops_process_message(htpops_context *ctx, struct MessageHeader *msg, size_
 int htpops_enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes);
 int htpops_finish_message(htpops_context *ctx, struct MessageHeader *msg);
 
+/* A message recorded once and replayed many times: the kernel launches of a whole message (a decoder block that is
+ * submitted again for every token, reference: src/dsp/commu.c:91-114 walks it anew each time) are captured into one
+ * HIP graph and re-enqueued on the context's stream with a single call.
+ * htpops_record_message runs the message once (request states are stored as usual, converted weight copies are made,
+ * the workspace is sized), then records a second walk without running it. It rejects messages with an RPCMEM_MAP
+ * request or a failing op, and contexts whose channel thread is active. A recording holds device addresses: it refuses
+ * to launch (HTPOPS_ERR_REJECTED, record again) once a buffer that its requests name has been released, weights it
+ * uses have been rewritten through htpops_buffer_write (their converted copies are dropped), or a later op has needed
+ * a larger workspace than the context had. Activations, KV rows and other buffer CONTENTS may change between launches
+ * (written by ops, by htpops_buffer_write or by the caller's own kernels); sizes, handles and offsets are those of
+ * the recorded message.
+ * Request states and the done byte are not touched by a launch; order against other work is stream order.
+ * Release every recording before htpops_close. */
+typedef struct htpops_recorded_message htpops_recorded_message;
+int htpops_record_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes,
+                          htpops_recorded_message **out);
+int htpops_launch_recorded_message(htpops_context *ctx, htpops_recorded_message *rec);
+int htpops_release_recorded_message(htpops_context *ctx, htpops_recorded_message *rec);
+
 /* Replaces htp_ops_create_channel / htp_ops_destroy_channel (reference: include/htp_ops.idl:11-12,
  * src/dsp/commu.c:151-212): starts a consumer thread that polls msg->state exactly as
  * msg_receiver_loop does (run when v[0] != 0 && v[1] == 0) and calls htpops_process_message.
