@@ -64,6 +64,7 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--skip-recorded", action="store_true", help="skip the replays of recorded messages (HIP graphs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (every box of this pool has one); --gpus %d is not "
@@ -177,10 +178,11 @@ def main():
         return ev_ms / steps
 
     ms_step, wall_step = time_layers(1, args.steps, args.warmup)
-    rec_step = {1: time_recorded_layers(1, args.steps, args.warmup)}
+    rec_step = {1: None if args.skip_recorded else time_recorded_layers(1, args.steps, args.warmup)}
     value = layer_bytes[1] / (ms_step * 1e-3) / 1e9
     log("layer m=1: %.2f us/step (events) %.2f us/step (wall)  %.0f GB/s" % (ms_step * 1e3, wall_step * 1e3, value))
-    log("layer m=1 as recorded messages: %.2f us/step" % (rec_step[1] * 1e3))
+    if rec_step[1] is not None:
+        log("layer m=1 as recorded messages: %.2f us/step" % (rec_step[1] * 1e3))
 
     # ------------------------------------------------------------------ the step's four launches, one by one
     def time_single(n, k, m, wt, handles, h_a, h_o, reps, op):
@@ -234,8 +236,9 @@ def main():
     # (every layer is touched before the clock starts: the first few-row use of a weight buffer repacks it once)
     ms_step8, _ = time_layers(8, max(20, args.steps // 4), LAYERS)
     log("layer m=8: %.2f us/step  %.0f GB/s" % (ms_step8 * 1e3, layer_bytes[8] / ms_step8 / 1e6))
-    rec_step[8] = time_recorded_layers(8, max(20, args.steps // 4), LAYERS)
-    log("layer m=8 as recorded messages: %.2f us/step" % (rec_step[8] * 1e3))
+    rec_step[8] = None if args.skip_recorded else time_recorded_layers(8, max(20, args.steps // 4), LAYERS)
+    if rec_step[8] is not None:
+        log("layer m=8 as recorded messages: %.2f us/step" % (rec_step[8] * 1e3))
 
     # ------------------------------------------------------------------ prefill GEMM (config 2)
     prefill = []
@@ -406,7 +409,8 @@ def main():
         "prefill_gemm": prefill,
         "small_batch": {"m": 8, "us_per_step": round(ms_step8 * 1e3, 2),
                         "GBps": round(layer_bytes[8] / ms_step8 / 1e6, 1)},
-        "recorded_message_us_per_step": {"m1": round(rec_step[1] * 1e3, 2), "m8": round(rec_step[8] * 1e3, 2)},
+        "recorded_message_us_per_step": None if args.skip_recorded else
+        {"m1": round(rec_step[1] * 1e3, 2), "m8": round(rec_step[8] * 1e3, 2)},
         "attention": attention,
         "q8_0_block": [q8_block[1], q8_block[128]],
         "peaks": peaks,
