@@ -397,6 +397,9 @@ bool in_owned_buffer(htpops_context *ctx, const void *ptr, size_t bytes) {
   return false;
 }
 
+constexpr int kSkinnyGroupMaxM = 8;   // rows of the K-sliced kernel's grouped launch
+constexpr int kBatchMaxM       = 16;  // rows up to which same-activation requests of a message are grouped
+
 bool ranges_overlap(const void *a, size_t a_bytes, const void *b, size_t b_bytes) {
   const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
   return a0 < b0 + b_bytes && b0 < a0 + a_bytes;
@@ -407,7 +410,7 @@ constexpr int kFragKindRowLayout = 100;  // + ggml type, to keep apart from the 
 // How one quantized matmul will run and how much of the context's workspace it needs.
 constexpr int kFragKindFp6Panel  = 200;  // + ggml type: FP6 operand panels of the many-row Q4_0 matmul
 
-constexpr int kFragKindLaneOrder = 300;  // + ggml type: Q4_0 weights in matrix-core operand order (2..8 activation rows)
+constexpr int kFragKindLaneOrder = 300;  // + ggml type: Q4_0 weights in matrix-core operand order (2..16 activation rows)
 
 // The repacked copy of `weight` for the few-row kernel: from the cache, or made now and cached. nullptr when this
 // matmul does not take that kernel (shape, weight type, weights in memory the context does not own and so cannot
@@ -1006,8 +1009,11 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
       for (int i = 0; i < b.count; ++i) {
         if (const void *lw = lane_order_weights(ctx, b.w[i], b.m, b.k, b.n[i], b.wt)) {
           out_a[count_a] = b.out[i], w_a[count_a] = lw, n_a[count_a++] = b.n[i];
-        } else {
+        } else if (b.m <= kSkinnyGroupMaxM) {
           out_b[count_b] = b.out[i], w_b[count_b] = b.w[i], n_b[count_b++] = b.n[i];
+        } else {
+          // more rows than the K-sliced group launch takes: on its own
+          b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act, b.w[i], b.m, b.k, b.n[i], b.wt);
         }
       }
       e = hipSuccess;
@@ -1051,8 +1057,8 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
     return false;
   }
   const auto *p = reinterpret_cast<const MatMulParams *>(req->payload);
-  if (p->m < 1 || p->m > 8 || p->k <= 0 || p->n <= 0 || p->k % 64 != 0) {
-    return false;  // one activation row, or the few rows of the weight-streaming small-batch kernel
+  if (p->m < 1 || p->m > kBatchMaxM || p->k <= 0 || p->n <= 0 || p->k % 64 != 0) {
+    return false;  // one activation row, or the few rows of the weight-streaming small-batch kernels
   }
   const int    wt        = req->op == HTP_OPS_MAT_MUL_Q4_0_Q8_0 ? htpops::kQ4_0 : htpops::kQ8_0;
   const size_t out_bytes = (size_t) p->m * p->n * 4, act_bytes = q8_0_bytes((size_t) p->m, (size_t) p->k);

@@ -1,4 +1,4 @@
-// Q4_0 x Q8_0 matmul for 2..8 activation rows over weights repacked once into the order the matrix core wants:
+// Q4_0 x Q8_0 matmul for 2..16 activation rows over weights repacked once into the order the matrix core wants:
 // out[m][n] = sum over 32-wide blocks of (int dot of the block) * d_act * d_weight (reference: src/dsp/ops/mat_mul.c:572-640,
 // block formats include/dsp/quants.h:8-14, ggml block_q4_0 / block_q8_0).
 //
@@ -15,8 +15,8 @@
 //
 // Every workgroup needs all activation rows, as many bytes as its weights. They come as they are (block_q8_0 rows)
 // by global_load_lds DMA in 16-byte pieces - no registers, no vector ALU work, in flight together with the first weight
-// loads - into LDS with the 8 rows interleaved piece by piece (the 8 rows a wave reads at one byte offset lie in 8
-// different bank groups); the lanes pick their operand bytes out of that image (a funnel shift where a block starts
+// loads - into LDS with the 8 (or, for m > 8, 16) rows interleaved piece by piece (the rows a wave reads at one byte
+// offset lie in different bank groups); the lanes pick their operand bytes out of that image (a funnel shift where a block starts
 // 2 bytes off a dword) and the block scales out of a float table made once after the DMA has landed. Measured: laying
 // the rows out in operand order with the vector ALU instead cost as much as streaming the weights.
 #include "device_utils.h"
@@ -33,9 +33,8 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 constexpr int kLoThreads  = 512;
 constexpr int kLoWaves    = kLoThreads / kWave;
 constexpr int kLoRows     = 16;                       // weight rows per tile
-constexpr int kLoActRows  = 8;                        // activation rows in the LDS panel (m <= 8)
+constexpr int kLoMaxActRows = 16;                     // the matrix instruction's other side: 16 activation rows
 constexpr int kLoQuadBytes = 64 * 16 + kLoRows * 8;   // 1152 = 16 rows x 4 blocks x 18 B
-constexpr int kLoScaleBlk = kLoActRows * 4;           // bytes of the scale table per block (8 floats)
 constexpr int kLoChunk    = 4;                        // quads a wave fetches at a time
 constexpr size_t kLoLdsLimit = 160 * 1024;
 
@@ -83,8 +82,12 @@ struct QuadRegs {
   uint2 d;  // the 4 fp16 scales of this lane's row
 };
 
+// ROWS: activation rows in the LDS panel, 8 (m <= 8: lanes 32..63 repeat rows 0..7 and their results are dropped) or 16
+template <int ROWS>
 __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrderGroupArgs grp,
                                                                        const uint8_t *__restrict__ act, int m, int k) {
+  constexpr int kLoActRows  = ROWS;
+  constexpr int kLoScaleBlk = ROWS * 4;  // bytes of the scale table per block (one float per row)
   extern __shared__ __align__(16) uint8_t lo_lds[];  // activation panel, later the waves' sums
   const int n = grp.n[blockIdx.y];
   if ((int) (blockIdx.x * kLoRows) >= n) {
@@ -139,7 +142,7 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
   // LDS byte offsets of this lane's operand dwords in its first quad (row nl % 8, elements {4 g .., 16 + 4 g ..} of
   // the quad's 4 blocks); the wave's next quad is 8 quads = 1088 B = 68 pieces of every row further on. Even blocks
   // of a quad start 2 bytes off a dword (34 b + 2 with b even): two dwords and a funnel shift; odd blocks are aligned.
-  auto a_addr = [&](int o) { return ((o >> 4) * kLoActRows + (nl & 7)) * 16 + (o & 15); };
+  auto a_addr = [&](int o) { return ((o >> 4) * kLoActRows + (nl & (ROWS - 1))) * 16 + (o & 15); };
   int  a_off[4][4];  // [block of the quad][dword]: even blocks use 4, odd blocks 2
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -153,8 +156,8 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
   constexpr int kQuadStep  = kLoWaves * 4 * 34 / 16 * kLoActRows * 16;  // 8 quads further on in the image: 8704 B
   constexpr int kScaleStep = kLoWaves * 4 * kLoScaleBlk;                // and in the scale table: 1024 B
   static_assert(kLoWaves * 4 * 34 % 16 == 0, "a wave's quads are whole pieces apart");
-  const uint8_t *s_lane = lo_lds + a_bytes + 4 * wave * kLoScaleBlk + (g & 1) * 16;  // scales of rows 4 (g & 1) ..
-  float          acc[4] = { 0.0f, 0.0f, 0.0f, 0.0f };  // rows 4 g + j, column nl (lanes with g >= 2: unused rows)
+  const uint8_t *s_lane = lo_lds + a_bytes + 4 * wave * kLoScaleBlk + (g & (ROWS / 4 - 1)) * 16;  // scales of rows 4 g ..
+  float          acc[4] = { 0.0f, 0.0f, 0.0f, 0.0f };  // rows 4 g + j, column nl (ROWS = 8, lanes with g >= 2: unused rows)
   // nibble -> int8 minus 8 without carries between bytes: (q + 0x78) ^ 0x80 per byte
   auto lo = [](uint32_t q) { return ((q & 0x0f0f0f0fu) + 0x78787878u) ^ 0x80808080u; };
   auto hi = [](uint32_t q) { return (((q >> 4) & 0x0f0f0f0fu) + 0x78787878u) ^ 0x80808080u; };
@@ -223,17 +226,21 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
     for (int w = 0; w < kLoWaves; ++w) {
       v += red[(w * 4 + j) * kWave + l];
     }
-    if ((l >> 4) < 2 && row < m) {
+    if ((l >> 4) < ROWS / 4 && row < m) {
       out[(size_t) row * n + n0 + (l & 15)] = v;
     }
   }
 }
 
 // LDS of a workgroup: the activation rows in whole DMA instructions, the scale table; later the waves' sums
-size_t panel_bytes(int k) {
+int panel_rows(int m) {
+  return m <= 8 ? 8 : kLoMaxActRows;
+}
+
+size_t panel_bytes(int k, int rows) {
   const size_t nblk  = (size_t) k / 32;
-  const size_t image = ((kLoActRows * (nblk * 34 / 16) * 16) + 1023) & ~(size_t) 1023;
-  const size_t panel = image + nblk * kLoScaleBlk, red = (size_t) kLoWaves * 4 * kWave * sizeof(float);
+  const size_t image = (((size_t) rows * (nblk * 34 / 16) * 16) + 1023) & ~(size_t) 1023;
+  const size_t panel = image + nblk * (size_t) rows * 4, red = (size_t) kLoWaves * 4 * kWave * sizeof(float);
   return panel > red ? panel : red;
 }
 
@@ -241,8 +248,8 @@ size_t panel_bytes(int k) {
 
 bool matmul_lane_order_fits(int n, int m, int k, WeightType wt) {
   // k % 256: activation rows (34 B per 32 elements) are whole 16-byte pieces, weight rows whole quads of blocks
-  return wt == kQ4_0 && m >= 2 && m <= kLoActRows && k > 0 && k % 256 == 0 && n > 0 && n % kLoRows == 0 &&
-         panel_bytes(k) <= kLoLdsLimit && n / kLoRows <= 0x7fffffff;
+  return wt == kQ4_0 && m >= 2 && m <= kLoMaxActRows && k > 0 && k % 256 == 0 && n > 0 && n % kLoRows == 0 &&
+         panel_bytes(k, panel_rows(m)) <= kLoLdsLimit && n / kLoRows <= 0x7fffffff;
 }
 
 size_t matmul_lane_order_weight_bytes(int k, int n) {
@@ -278,16 +285,25 @@ hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *
   }
   static bool attr_set = false;  // more than the default 64 KiB of dynamic LDS for long rows
   if (!attr_set) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(matmul_lane_order_kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int) kLoLdsLimit);
-    if (e != hipSuccess) {
-      return e;
+    for (const void *kernel : { reinterpret_cast<const void *>(matmul_lane_order_kernel<8>),
+                                reinterpret_cast<const void *>(matmul_lane_order_kernel<16>) }) {
+      const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int) kLoLdsLimit);
+      if (e != hipSuccess) {
+        return e;
+      }
     }
     attr_set = true;
   }
-  const dim3 grid((unsigned) (n_max / kLoRows), (unsigned) count);
-  hipLaunchKernelGGL(matmul_lane_order_kernel, grid, dim3(kLoThreads), panel_bytes(k), stream, grp,
-                     static_cast<const uint8_t *>(act), m, k);
+  const dim3   grid((unsigned) (n_max / kLoRows), (unsigned) count);
+  const int    rows = panel_rows(m);
+  const size_t lds  = panel_bytes(k, rows);
+  if (rows == 8) {
+    hipLaunchKernelGGL(matmul_lane_order_kernel<8>, grid, dim3(kLoThreads), lds, stream, grp,
+                       static_cast<const uint8_t *>(act), m, k);
+  } else {
+    hipLaunchKernelGGL(matmul_lane_order_kernel<16>, grid, dim3(kLoThreads), lds, stream, grp,
+                       static_cast<const uint8_t *>(act), m, k);
+  }
   return hipGetLastError();
 }
 

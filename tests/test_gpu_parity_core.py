@@ -242,7 +242,8 @@ def test_message_batches_same_activation_gemvs(ctx, oracle, wt):
             ctx.release(h)
 
 
-@pytest.mark.parametrize("wt,m,k", [(wl.GGML_TYPE_Q4_0, 8, 4096), (wl.GGML_TYPE_Q8_0, 3, 1536), (wl.GGML_TYPE_Q4_0, 2, 2048 + 64)])
+@pytest.mark.parametrize("wt,m,k", [(wl.GGML_TYPE_Q4_0, 8, 4096), (wl.GGML_TYPE_Q8_0, 3, 1536), (wl.GGML_TYPE_Q4_0, 2, 2048 + 64),
+                                    (wl.GGML_TYPE_Q4_0, 12, 4096), (wl.GGML_TYPE_Q8_0, 10, 1536), (wl.GGML_TYPE_Q4_0, 16, 2048 + 64)])
 def test_message_batches_same_activation_small_batches(ctx, oracle, wt, m, k):
     # The same grouping for 2..8 activation rows: matrices of different n on activation A run as one launch of the
     # K-sliced kernel (each with its own partial tiles and ticket counters), then the same weights on activation B.
@@ -388,10 +389,12 @@ def test_message_shares_one_activation_conversion_between_many_row_matmuls(ctx, 
 
 
 @pytest.mark.parametrize("m,k,n", [(2, 256, 16), (8, 256, 48), (3, 512, 4096), (8, 4096, 4096), (5, 11008, 272), (8, 2048 + 256, 1024),
-                                   (7, 8960, 1536)])
+                                   (7, 8960, 1536), (9, 256, 32), (16, 4096, 4096), (12, 2048 + 256, 1040), (13, 8192, 48),
+                                   (16, 8960, 64), (11, 11008, 64)])
 def test_few_rows_over_repacked_weights(ctx, oracle, monkeypatch, m, k, n):
-    # 2..8 rows against Q4_0 weights with n % 16 == 0, k % 256 == 0 run on a copy of the weights repacked into
-    # matrix-core operand order. It must meet the oracle, agree with the kernels that read the weights as they are
+    # 2..16 rows against Q4_0 weights with n % 16 == 0, k % 256 == 0 run on a copy of the weights repacked into
+    # matrix-core operand order (9..16 rows only while 16 activation rows fit the LDS panel: k = 8960 does not,
+    # nor 11008; they take the K-sliced kernel). It must meet the oracle, agree with the kernels that read the weights as they are
     # (switch HTPOPS_LANE_ORDER=0) to summation order, and repeat bit for bit.
     rng = wl.rng_for(66, m * 17 + k + n)
     got, x, w = check_mat_mul(ctx, oracle, rng, m, k, n, wl.GGML_TYPE_Q4_0)
