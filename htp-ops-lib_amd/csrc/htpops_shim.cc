@@ -693,6 +693,14 @@ extern "C" int htpops_close(htpops_context *ctx) {
     (void) hipSetDevice(ctx->device);
     (void) hipStreamSynchronize(ctx->stream);
   }
+  for (htpops_recorded_message *rec : ctx->recordings) {  // recordings the caller did not release
+    if (rec->exec) {
+      (void) hipGraphExecDestroy(rec->exec);
+      (void) hipGraphDestroy(rec->graph);
+    }
+    delete rec;
+  }
+  ctx->recordings.clear();
   for (size_t h = 1; h < ctx->buffers.size(); ++h) {
     Buffer &b = ctx->buffers[h];
     if (b.live && b.owned) {

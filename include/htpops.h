@@ -108,7 +108,7 @@ int htpops_finish_message(htpops_context *ctx, struct MessageHeader *msg);
  * (written by ops, by htpops_buffer_write or by the caller's own kernels); sizes, handles and offsets are those of
  * the recorded message.
  * Request states and the done byte are not touched by a launch; order against other work is stream order.
- * Release every recording before htpops_close. */
+ * htpops_close releases the recordings that are still alive; their pointers must not be used afterwards. */
 typedef struct htpops_recorded_message htpops_recorded_message;
 int htpops_record_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes,
                           htpops_recorded_message **out);

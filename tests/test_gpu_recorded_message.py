@@ -167,3 +167,15 @@ def test_messages_that_cannot_be_recorded(ctx):
     finally:
         for h in (spare, hx, hy):
             ctx.release(h)
+
+
+def test_close_releases_recordings_left_alive():
+    c = api.Context(device=0)
+    rng = wl.rng_for(73, 0)
+    hx = c.upload(wl.make_activations(rng, 4, 1024))
+    hy = c.alloc(4 * 1024 * 4)
+    msg = api.build_message([op(api.HTP_OPS_RMS_NORM_F32, api.rms_norm_params((hy, 0), (hx, 0), 1024, 4))])
+    ret, rec = c.record_message(msg)
+    assert ret == 0 and rec is not None
+    assert c.launch_recorded_message(rec) == 0
+    c.close()  # neither the recording nor the buffers were released by hand
