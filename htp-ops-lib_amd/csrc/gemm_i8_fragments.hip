@@ -118,6 +118,7 @@ template <int U>
 struct FragSet {
   uint4    a[U], b[U];
   uint32_t da[U], dw[U];
+  uint32_t live;  // all ones, or zero for a block past the end of K (wave-uniform)
 };
 
 // KSPLIT waves share one tile of U x U units (each takes every KSPLIT-th block); a workgroup holds 4 / KSPLIT tiles
@@ -163,12 +164,14 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__
   }
   auto load = [&](FragSet<U> &s, int kb_raw) {
     const size_t kb = (size_t) min(kb_raw, nblk - 1);  // branch-free: blocks past the end repeat the last one ...
-    const uint32_t live = kb_raw < nblk ? 0xffffffffu : 0u;  // ... with activation scales of zero: they add nothing
+    // ... with activation scales of zero: they add nothing. The mask is applied where the scale is used, not here: an
+    // instruction on a freshly loaded register here would make the wave wait for the loads it has just issued.
+    s.live = kb_raw < nblk ? 0xffffffffu : 0u;
 #pragma unroll
     for (int i = 0; i < U; ++i) {
       s.a[i]  = (ap[i] + kb * 64)[lane];
       s.b[i]  = (bp[i] + kb * 64)[lane];
-      s.da[i] = (asp[i] + kb * 32)[c] & live;
+      s.da[i] = (asp[i] + kb * 32)[c];
       s.dw[i] = (bsp[i] + kb * 32)[c];
     }
   };
@@ -203,7 +206,7 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, zi, 0, 0, 0);
   };
   auto mfma_scale = [&](const FragSet<U> &s, int i, int j) {
-    return __builtin_amdgcn_mfma_f32_32x32x8f16(scale_operand(s.da[i]), scale_operand(s.dw[j]), zf, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x8f16(scale_operand(s.da[i] & s.live), scale_operand(s.dw[j]), zf, 0, 0, 0);
   };
 
   // Software pipeline over units (block, i, j): the two matrix instructions of the NEXT unit are issued between the
