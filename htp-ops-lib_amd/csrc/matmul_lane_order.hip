@@ -83,27 +83,33 @@ struct QuadRegs {
 };
 
 // ROWS: activation rows in the LDS panel, 8 (m <= 8: lanes 32..63 repeat rows 0..7 and their results are dropped) or 16
-template <int ROWS>
+// TPW:  16-row weight tiles per workgroup, 1 (8 waves per tile) or 2 (4 waves per tile). The activation panel is as
+//       many bytes as a tile's weights and every workgroup fetches it from L2, so two tiles per workgroup cut the
+//       traffic into a CU by a quarter; used when that still leaves enough workgroups.
+template <int ROWS, int TPW>
 __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrderGroupArgs grp,
                                                                        const uint8_t *__restrict__ act, int m, int k) {
   constexpr int kLoActRows  = ROWS;
   constexpr int kLoScaleBlk = ROWS * 4;  // bytes of the scale table per block (one float per row)
   extern __shared__ __align__(16) uint8_t lo_lds[];  // activation panel, later the waves' sums
   const int n = grp.n[blockIdx.y];
-  if ((int) (blockIdx.x * kLoRows) >= n) {
+  if ((int) (blockIdx.x * kLoRows * TPW) >= n) {
     return;  // whole workgroup: this member has fewer rows than the widest one
   }
+  constexpr int WQ = kLoWaves / TPW;  // waves that share a tile
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wph = wave % WQ, tw = wave / WQ;
   const int nl = lane & 15, g = lane >> 4;
+  // a second tile past the end of an odd tile count repeats the last one (never stored)
+  const int tile = min((int) blockIdx.x * TPW + tw, n / kLoRows - 1);
   const int nblk = k / 32, nquads = nblk / 4;
-  const uint8_t *__restrict__ wt = grp.w[blockIdx.y] + (size_t) blockIdx.x * nquads * kLoQuadBytes;
+  const uint8_t *__restrict__ wt = grp.w[blockIdx.y] + (size_t) tile * nquads * kLoQuadBytes;
   float *__restrict__         out = grp.out[blockIdx.y];
-  const int                   n0  = blockIdx.x * kLoRows;
 
   auto fetch = [&](QuadRegs (&r)[kLoChunk], int q0) {  // quads q0, q0 + 8, ... of this wave (clamped: extra ones unused)
 #pragma unroll
     for (int c = 0; c < kLoChunk; ++c) {
-      const int      q = min(q0 + c * kLoWaves, nquads - 1);
+      const int      q = min(q0 + c * WQ, nquads - 1);
       const uint8_t *p = wt + (size_t) q * kLoQuadBytes;
       r[c].q           = *reinterpret_cast<const uint4 *>(p + lane * 16);
       r[c].d           = *reinterpret_cast<const uint2 *>(p + 1024 + nl * 8);
@@ -123,7 +129,7 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
     asm volatile("s_mov_b32 m0, %1\n s_nop 0\n global_load_lds_dwordx4 %0, off" ::"v"(p), "s"(to) : "memory");
   }
   QuadRegs cur[kLoChunk], nxt[kLoChunk];
-  fetch(cur, wave);  // 2 kLoChunk loads, in flight behind the DMA
+  fetch(cur, wph);  // 2 kLoChunk loads, in flight behind the DMA
   // the DMA pieces of this wave have landed once only the weight loads issued after them are outstanding
   // (s_waitcnt operand: vmcnt in bits 3:0 and 15:14, expcnt (7 = no wait) in 6:4, lgkmcnt in 11:8)
   static_assert(2 * kLoChunk == 8, "the wait below leaves exactly the weight loads in flight");
@@ -146,29 +152,29 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
   int  a_off[4][4];  // [block of the quad][dword]: even blocks use 4, odd blocks 2
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const int o = (4 * wave + j) * 34 + 4 * g;  // byte 4 g of the block's row segment (its scale is bytes 0..1)
+    const int o = (4 * wph + j) * 34 + 4 * g;  // byte 4 g of the block's row segment (its scale is bytes 0..1)
     if (j % 2 == 0) {
       a_off[j][0] = a_addr(o), a_off[j][1] = a_addr(o + 4), a_off[j][2] = a_addr(o + 16), a_off[j][3] = a_addr(o + 20);
     } else {
       a_off[j][0] = a_addr(o + 2), a_off[j][1] = a_addr(o + 18), a_off[j][2] = 0, a_off[j][3] = 0;
     }
   }
-  constexpr int kQuadStep  = kLoWaves * 4 * 34 / 16 * kLoActRows * 16;  // 8 quads further on in the image: 8704 B
-  constexpr int kScaleStep = kLoWaves * 4 * kLoScaleBlk;                // and in the scale table: 1024 B
-  static_assert(kLoWaves * 4 * 34 % 16 == 0, "a wave's quads are whole pieces apart");
-  const uint8_t *s_lane = lo_lds + a_bytes + 4 * wave * kLoScaleBlk + (g & (ROWS / 4 - 1)) * 16;  // scales of rows 4 g ..
+  constexpr int kQuadStep  = WQ * 4 * 34 / 16 * kLoActRows * 16;  // WQ quads further on in the image
+  constexpr int kScaleStep = WQ * 4 * kLoScaleBlk;                // and in the scale table
+  static_assert(WQ * 4 * 34 % 16 == 0, "a wave's quads are whole pieces apart");
+  const uint8_t *s_lane = lo_lds + a_bytes + 4 * wph * kLoScaleBlk + (g & (ROWS / 4 - 1)) * 16;  // scales of rows 4 g ..
   float          acc[4] = { 0.0f, 0.0f, 0.0f, 0.0f };  // rows 4 g + j, column nl (ROWS = 8, lanes with g >= 2: unused rows)
   // nibble -> int8 minus 8 without carries between bytes: (q + 0x78) ^ 0x80 per byte
   auto lo = [](uint32_t q) { return ((q & 0x0f0f0f0fu) + 0x78787878u) ^ 0x80808080u; };
   auto hi = [](uint32_t q) { return (((q >> 4) & 0x0f0f0f0fu) + 0x78787878u) ^ 0x80808080u; };
-  for (int q0 = wave; q0 < nquads; q0 += kLoChunk * kLoWaves) {
-    const bool more = q0 + kLoChunk * kLoWaves < nquads;
+  for (int q0 = wph; q0 < nquads; q0 += kLoChunk * WQ) {
+    const bool more = q0 + kLoChunk * WQ < nquads;
     if (more) {
-      fetch(nxt, q0 + kLoChunk * kLoWaves);
+      fetch(nxt, q0 + kLoChunk * WQ);
     }
 #pragma unroll
     for (int c = 0; c < kLoChunk; ++c) {
-      const int quad = q0 + c * kLoWaves;
+      const int quad = q0 + c * WQ;
       if (quad < nquads) {
         const uint32_t wq[4] = { cur[c].q.x, cur[c].q.y, cur[c].q.z, cur[c].q.w };
         union {
@@ -176,7 +182,7 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
           _Float16 h[4];
         } sc;
         sc.u = cur[c].d;
-        const int      it  = (quad - wave) / kLoWaves;  // this quad is the wave's it-th
+        const int      it  = (quad - wph) / WQ;  // this quad is the wave's it-th
         const uint8_t *img = lo_lds + (size_t) it * kQuadStep;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -211,7 +217,7 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
     }
   }
 
-  // ---- add the eight waves in wave order (the panel is no longer needed) ----
+  // ---- add the waves of a tile in wave order (the panel is no longer needed) ----
   __syncthreads();
   float *red = reinterpret_cast<float *>(lo_lds);
 #pragma unroll
@@ -219,14 +225,15 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
     red[(wave * 4 + j) * kWave + lane] = acc[j];
   }
   __syncthreads();
-  if (tid < 4 * kWave) {
-    const int j = tid >> 6, l = tid & 63, row = 4 * (l >> 4) + j;
+  if (tid < 4 * kWave * TPW) {
+    const int t = tid / (4 * kWave), j = (tid >> 6) & 3, l = tid & 63, row = 4 * (l >> 4) + j;
     float     v = 0.0f;
 #pragma unroll
-    for (int w = 0; w < kLoWaves; ++w) {
-      v += red[(w * 4 + j) * kWave + l];
+    for (int w = 0; w < WQ; ++w) {
+      v += red[((t * WQ + w) * 4 + j) * kWave + l];
     }
-    if ((l >> 4) < ROWS / 4 && row < m) {
+    const int n0 = ((int) blockIdx.x * TPW + t) * kLoRows;
+    if ((l >> 4) < ROWS / 4 && row < m && n0 < n) {
       out[(size_t) row * n + n0 + (l & 15)] = v;
     }
   }
@@ -283,27 +290,33 @@ hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *
     grp.n[i]   = ns[i];
     n_max      = ns[i] > n_max ? ns[i] : n_max;
   }
+  typedef void (*Kernel)(LaneOrderGroupArgs, const uint8_t *, int, int);
+  static const Kernel kernels[2][2] = { { matmul_lane_order_kernel<8, 1>, matmul_lane_order_kernel<8, 2> },
+                                        { matmul_lane_order_kernel<16, 1>, matmul_lane_order_kernel<16, 2> } };
   static bool attr_set = false;  // more than the default 64 KiB of dynamic LDS for long rows
   if (!attr_set) {
-    for (const void *kernel : { reinterpret_cast<const void *>(matmul_lane_order_kernel<8>),
-                                reinterpret_cast<const void *>(matmul_lane_order_kernel<16>) }) {
-      const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int) kLoLdsLimit);
+    for (int i = 0; i < 4; ++i) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernels[i / 2][i % 2]),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int) kLoLdsLimit);
       if (e != hipSuccess) {
         return e;
       }
     }
     attr_set = true;
   }
-  const dim3   grid((unsigned) (n_max / kLoRows), (unsigned) count);
+  // two tiles per workgroup when that still gives every CU two workgroups (measured at m = 8: gate + up, 688 pairs,
+  // 19.6 -> 17.6 us; q + k + v, 384 pairs, no gain; single 4096-row matrices lose)
+  long pairs = 0;
+  for (int i = 0; i < count; ++i) {
+    pairs += (ns[i] / kLoRows + 1) / 2;
+  }
+  const int    forced = env_int("HTPOPS_LANE_ORDER_TILES", 0);  // read per call: tests run both
+  const int    tpw    = forced == 1 || forced == 2 ? forced : (pairs >= 512 ? 2 : 1);
+  const dim3   grid((unsigned) ((n_max / kLoRows + tpw - 1) / tpw), (unsigned) count);
   const int    rows = panel_rows(m);
   const size_t lds  = panel_bytes(k, rows);
-  if (rows == 8) {
-    hipLaunchKernelGGL(matmul_lane_order_kernel<8>, grid, dim3(kLoThreads), lds, stream, grp,
-                       static_cast<const uint8_t *>(act), m, k);
-  } else {
-    hipLaunchKernelGGL(matmul_lane_order_kernel<16>, grid, dim3(kLoThreads), lds, stream, grp,
-                       static_cast<const uint8_t *>(act), m, k);
-  }
+  hipLaunchKernelGGL(kernels[rows == 16][tpw - 1], grid, dim3(kLoThreads), lds, stream, grp,
+                     static_cast<const uint8_t *>(act), m, k);
   return hipGetLastError();
 }
 

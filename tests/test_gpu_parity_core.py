@@ -401,6 +401,14 @@ def test_few_rows_over_repacked_weights(ctx, oracle, monkeypatch, m, k, n):
     a = oracle.quantize_q8_0(x)
     assert np.array_equal(ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0), got)
     _, mag = oracle.mat_mul_q8_0_act_f64(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
+    # one and two weight tiles per workgroup (the launcher picks by the number of tiles) sum the same blocks in
+    # different wave order
+    for tiles in ("1", "2"):
+        monkeypatch.setenv("HTPOPS_LANE_ORDER_TILES", tiles)
+        forced = ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
+        assert np.all(np.abs(forced - got) <= 2 * MATMUL_RTOL * mag)
+        assert np.array_equal(forced, ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0))
+    monkeypatch.delenv("HTPOPS_LANE_ORDER_TILES")
     monkeypatch.setenv("HTPOPS_LANE_ORDER", "0")
     plain = ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
     assert np.all(np.abs(plain - got) <= 2 * MATMUL_RTOL * mag)
