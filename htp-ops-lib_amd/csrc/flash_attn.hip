@@ -413,7 +413,8 @@ __global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(
 
 constexpr int kDecThreads  = 256;
 constexpr int kDecMaxGroup = 8;   // query heads scored per pass against one K/V stream
-constexpr int kDecSplit    = 128; // keys per workgroup
+constexpr int kDecSplit    = 128; // keys per workgroup ...
+constexpr int kDecSplitShort = 64;  // ... and for short contexts, where 128 would leave most CUs without a workgroup
 
 // sum over the 16 (or 8) consecutive lanes of a key group with DPP row operations; every lane gets the sum
 template <int LPK>
@@ -430,10 +431,10 @@ __device__ __forceinline__ float key_group_sum(float v) {
 }
 
 // partial record per (head, split): m, l, then D floats of un-normalised O.
-// A workgroup owns kDecSplit consecutive keys of one KV head. LPK = D / 8 lanes share a key (16 bytes of K and of
+// A workgroup owns SPLIT consecutive keys of one KV head. LPK = D / 8 lanes share a key (16 bytes of K and of
 // V each); every K and V load of the wave is issued before the first use, the scores of all GH heads are formed
 // against the same registers, and the per-slot (max, sum, O) partials are merged through LDS.
-template <int D, int GH, bool QO_F32>
+template <int D, int GH, bool QO_F32, int SPLIT>
 __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *__restrict__ part,
                                                                         const void *__restrict__ q_ptr,
                                                                         const _Float16 *__restrict__ k_ptr,
@@ -445,7 +446,8 @@ __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *_
   constexpr int KPW    = kWave / LPK;  // keys per wave per pass
   constexpr int WAVES  = kDecThreads / kWave;
   constexpr int SLOTS  = WAVES * KPW;  // independent partial streams in the workgroup
-  constexpr int PASSES = kDecSplit / SLOTS;
+  constexpr int PASSES = SPLIT / SLOTS;
+  static_assert(SPLIT % SLOTS == 0, "whole passes");
   __shared__ float red_m[SLOTS][GH], red_l[SLOTS][GH], red_o[SLOTS][GH][D];
 
   const int group = n_heads / n_kv_heads;
@@ -458,8 +460,8 @@ __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *_
   const float scale = (1.0f / sqrtf((float) D)) * kLog2e;
   const size_t kv_stride = (size_t) n_kv_heads * D;
 
-  const int k_begin = split * kDecSplit;
-  const int k_end   = min(kv_len, k_begin + kDecSplit);
+  const int k_begin = split * SPLIT;
+  const int k_end   = min(kv_len, k_begin + SPLIT);
 
   // all K and V of this lane, requested up front (keys of a pass are consecutive across slots)
   v8h kreg[PASSES], vreg[PASSES];
@@ -830,14 +832,24 @@ template <int D, bool QO_F32>
 hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void *k, const void *v, const void *mask,
                          int kv_len, int n_heads, int n_kv_heads, float *workspace) {
   const int  group    = n_heads / n_kv_heads;
-  const int  n_splits = (kv_len + kDecSplit - 1) / kDecSplit;
+  // 64-key chunks while 128-key ones would give fewer than 128 workgroups (measured at 8 KV heads: kv = 512 8.8 -> 7.1 us;
+  // kv = 4096 and 16384 are 1 and 6 us slower with 64)
+  const bool short_kv = (long) ((kv_len + kDecSplit - 1) / kDecSplit) * n_kv_heads < 128;
+  const int  split    = short_kv ? kDecSplitShort : kDecSplit;
+  const int  n_splits = (kv_len + split - 1) / split;
   const dim3 grid((unsigned) n_splits, (unsigned) n_kv_heads);
   for (int h0 = 0; h0 < group; h0 += kDecMaxGroup) {
     const int gh = group - h0;
 #define HTPOPS_DECODE(GH)                                                                                          \
-  hipLaunchKernelGGL((flash_attn_decode_kernel<D, GH, QO_F32>), grid, dim3(kDecThreads), 0, stream, workspace, q,   \
-                     (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, kv_len, n_heads,          \
-                     n_kv_heads, h0, n_splits)
+  if (short_kv) {                                                                                                  \
+    hipLaunchKernelGGL((flash_attn_decode_kernel<D, GH, QO_F32, kDecSplitShort>), grid, dim3(kDecThreads), 0,      \
+                       stream, workspace, q, (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask,  \
+                       kv_len, n_heads, n_kv_heads, h0, n_splits);                                                 \
+  } else {                                                                                                         \
+    hipLaunchKernelGGL((flash_attn_decode_kernel<D, GH, QO_F32, kDecSplit>), grid, dim3(kDecThreads), 0, stream,   \
+                       workspace, q, (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, kv_len,  \
+                       n_heads, n_kv_heads, h0, n_splits);                                                         \
+  }
     if (gh >= 8) {
       HTPOPS_DECODE(8);
     } else if (gh > 4) {
@@ -862,7 +874,7 @@ size_t flash_attn_workspace_bytes(int qo_len, int kv_len, int n_heads, int head_
   if (qo_len != 1 || (head_dim != 64 && head_dim != 128)) {
     return 0;
   }
-  const size_t n_splits = ((size_t) kv_len + kDecSplit - 1) / kDecSplit;
+  const size_t n_splits = ((size_t) kv_len + kDecSplitShort - 1) / kDecSplitShort;  // the most there can be
   return (size_t) n_heads * n_splits * ((size_t) head_dim + 2) * sizeof(float);
 }
 

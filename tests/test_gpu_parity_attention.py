@@ -26,6 +26,9 @@ CASES = [
     (1, 300, 8, 2, 128), (1, 4096, 32, 8, 128), (1, 70, 4, 4, 64), (1, 129, 16, 1, 128), (1, 1, 4, 2, 64),
     (5, 70, 4, 2, 64), (40, 300, 4, 1, 128), (33, 517, 4, 4, 128), (64, 64, 2, 1, 64), (128, 128, 8, 2, 128),
     (100, 260, 6, 2, 128), (31, 95, 3, 1, 64), (2, 2, 2, 2, 64), (96, 200, 8, 1, 128),
+    # decode on both sides of the switch between 64- and 128-key chunks (128 workgroups of 128 keys)
+    (1, 64, 8, 8, 128), (1, 65, 8, 2, 64), (1, 2048, 32, 8, 128), (1, 1920, 32, 8, 128), (1, 1900, 16, 4, 64),
+    (1, 2100, 16, 16, 64),
     # head dims other than 64 and 128 (the reference's flash_attn_sp_hdim.c domain: any even head_dim)
     (1, 300, 8, 2, 80), (7, 133, 4, 2, 96), (33, 70, 6, 3, 40), (1, 1, 2, 1, 2), (20, 517, 4, 1, 256), (3, 64, 2, 2, 112),
     (1, 1000, 4, 4, 192), (65, 65, 2, 1, 30),
