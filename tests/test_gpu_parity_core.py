@@ -296,6 +296,22 @@ def test_small_batch_repeated_launches_are_bit_identical(ctx):
         assert np.abs(one[0] - first[r]).max() <= 2e-5 * np.abs(one).max()
 
 
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+def test_mat_mul_on_both_sides_of_every_kernel_switch(ctx, oracle, wt):
+    # which kernel a matmul takes depends on m (1 | 2..8 | 9..16 | 17..32 | 33..), on k (multiples of 32, 64, 256; the
+    # LDS panel of the few-row kernel) and on n (multiples of 16, tile counts): seeded random shapes around each switch,
+    # every one against the oracle
+    rng = wl.rng_for(68, wt)
+    ms = [1, 2, 7, 8, 9, 15, 16, 17, 31, 32, 33, 34, 63, 64, 65, 127, 128, 129, 200]
+    for m in ms:
+        for _ in range(2):
+            k = int(rng.choice([32, 64, 96, 256, 288, 512, 1024 + 64, 2048, 4096 + 256, 8192, 8960]))
+            n = int(rng.choice([1, 15, 16, 17, 48, 100, 256, 272, 1000, 1536]))
+            if m * k * n > 200e6:
+                n = 48
+            check_mat_mul(ctx, oracle, rng, m, k, n, wt)
+
+
 # --------------------------------------------------------------------------------- prefill (MFMA) path
 
 @pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
