@@ -432,6 +432,93 @@ hipError_t launch_shared_act(hipStream_t stream, const GemvGroupArgs &grp, int c
   return hipErrorInvalidValue;
 }
 
+// ---- two to four activation rows ------------------------------------------------------------------------------------
+// The same stream over the weights with M activation rows staged in LDS: a lane prepares its activation pairs of all M
+// rows once and dots every weight pair it loads against each of them (the nibble unpacking is shared), so the weights
+// are still read once and the extra rows cost vector-ALU work only. One row set per wave, 256 threads.
+template <int WT, int G, int ITERS, int M>
+__global__ __launch_bounds__(kThreads) void gemv_rows_shared_act_kernel(GemvGroupArgs grp, const uint32_t *__restrict__ act,
+                                                                        int pairs) {
+  extern __shared__ __attribute__((aligned(16))) uint32_t act_lds[];
+  constexpr int PD    = Pair<WT>::kDwords;
+  constexpr int SLOTS = kWave / G;
+  const int                    n   = grp.n[blockIdx.y];
+  float *__restrict__          out = grp.out[blockIdx.y];
+  const uint32_t *__restrict__ w   = grp.w[blockIdx.y];
+  if ((int) (blockIdx.x * (kWaves * SLOTS)) >= n) {
+    return;  // whole workgroup: this member has fewer rows than the widest one
+  }
+  const int    lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int    g = lane % G, slot = lane / G;
+  const int    row = (blockIdx.x * kWaves + wave) * SLOTS + slot;
+  const size_t row_dwords = (size_t) pairs * PD;
+
+  // the M activation rows are contiguous: requested first (they come from L2), in 16-byte pieces, the last piece slid
+  // back to the end; then the weights, which are in flight during the LDS exchange
+  constexpr int ACT_SLOTS = (M * 192 * kActPairDwords * 4 + kThreads * 16 - 1) / (kThreads * 16);
+  const int     act_bytes = M * pairs * kActPairDwords * 4;
+  uint4         areg[ACT_SLOTS];
+  int           aoff[ACT_SLOTS];
+#pragma unroll
+  for (int j = 0; j < ACT_SLOTS; ++j) {
+    const int off = (threadIdx.x + j * kThreads) * 16;
+    aoff[j]       = min(off, act_bytes - 16);
+    const u32x4_a4 v = *reinterpret_cast<const u32x4_a4 *>(reinterpret_cast<const uint8_t *>(act) + aoff[j]);
+    areg[j]       = make_uint4(v.x, v.y, v.z, v.w);
+  }
+  uint32_t  wreg[ITERS][PD];
+  const int wrow = min(row, n - 1);
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int p = min(g + i * G, pairs - 1);
+    load_dwords<PD>(wreg[i], w + (size_t) wrow * row_dwords + (size_t) p * PD);
+  }
+#pragma unroll
+  for (int j = 0; j < ACT_SLOTS; ++j) {
+    uint32_t *dst = act_lds + aoff[j] / 4;
+    dst[0] = areg[j].x, dst[1] = areg[j].y, dst[2] = areg[j].z, dst[3] = areg[j].w;
+  }
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the LDS writes have landed; vmcnt is left alone
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+
+  float acc[M];
+#pragma unroll
+  for (int mm = 0; mm < M; ++mm) {
+    acc[mm] = 0.0f;
+  }
+#pragma unroll
+  for (int i = 0; i < ITERS; ++i) {
+    const int     p    = g + i * G;
+    const bool    live = row < n && p < pairs;
+    constexpr int kScale1 = WT == kQ4_0 ? 4 : 8;  // dword holding the second block's scale (upper half)
+    wreg[i][0]       = live ? wreg[i][0] : 0u;
+    wreg[i][kScale1] = live ? wreg[i][kScale1] : 0u;
+#pragma unroll
+    for (int mm = 0; mm < M; ++mm) {
+      uint32_t a[kActPairDwords];
+      if (p < pairs) {
+#pragma unroll
+        for (int e = 0; e < kActPairDwords; ++e) {
+          a[e] = act_lds[(mm * pairs + p) * kActPairDwords + e];
+        }
+      } else {
+        zero_dwords<kActPairDwords>(a);
+      }
+      ActPair<WT> ap;
+      prepare(ap, a);
+      acc[mm] += pair_dot(wreg[i], ap);
+    }
+  }
+#pragma unroll
+  for (int mm = 0; mm < M; ++mm) {
+    const float v = group_sum_dpp<G>(acc[mm]);
+    if (g == G - 1 && row < n) {
+      out[(size_t) mm * n + row] = v;
+    }
+  }
+}
+
 // Catch-all (odd block counts, any m): one wave per weight row, 16-bit loads, scalar integer arithmetic.
 template <int WT>
 __global__ __launch_bounds__(kThreads) void gemv_blocks_generic_kernel(float *__restrict__ out,
@@ -532,6 +619,50 @@ hipError_t launch_gemv_shared(hipStream_t stream, const GemvGroupArgs &grp, int 
   return launch_shared_act<WT, 64, 3>(stream, grp, count, act, pairs, r, threads);
 }
 
+template <int WT, int G, int ITERS>
+hipError_t launch_rows_shared_act(hipStream_t stream, const GemvGroupArgs &grp, int count, const uint32_t *act, int pairs,
+                                  int m) {
+  constexpr int rows_per_group = kWaves * (kWave / G);
+  int           n_max          = 0;
+  for (int i = 0; i < count; ++i) {
+    n_max = grp.n[i] > n_max ? grp.n[i] : n_max;
+  }
+  const dim3   grid((unsigned) ((n_max + rows_per_group - 1) / rows_per_group), (unsigned) count);
+  const size_t lds = (size_t) m * pairs * kActPairDwords * 4;
+  switch (m) {
+    case 2:
+      hipLaunchKernelGGL((gemv_rows_shared_act_kernel<WT, G, ITERS, 2>), grid, dim3(kThreads), lds, stream, grp, act, pairs);
+      break;
+    case 3:
+      hipLaunchKernelGGL((gemv_rows_shared_act_kernel<WT, G, ITERS, 3>), grid, dim3(kThreads), lds, stream, grp, act, pairs);
+      break;
+    case 4:
+      hipLaunchKernelGGL((gemv_rows_shared_act_kernel<WT, G, ITERS, 4>), grid, dim3(kThreads), lds, stream, grp, act, pairs);
+      break;
+    default:
+      return hipErrorNotSupported;
+  }
+  return hipGetLastError();
+}
+
+template <int WT>
+hipError_t launch_gemv_rows_shared(hipStream_t stream, const GemvGroupArgs &grp, int count, const uint32_t *act, int pairs,
+                                   int m) {
+  if (pairs <= 16) {
+    return launch_rows_shared_act<WT, 16, 1>(stream, grp, count, act, pairs, m);
+  }
+  if (pairs <= 32) {
+    return launch_rows_shared_act<WT, 32, 1>(stream, grp, count, act, pairs, m);
+  }
+  if (pairs <= 64) {
+    return launch_rows_shared_act<WT, 64, 1>(stream, grp, count, act, pairs, m);
+  }
+  if (pairs <= 128) {
+    return launch_rows_shared_act<WT, 64, 2>(stream, grp, count, act, pairs, m);
+  }
+  return launch_rows_shared_act<WT, 64, 3>(stream, grp, count, act, pairs, m);
+}
+
 template <int WT>
 hipError_t launch_gemv_row(hipStream_t stream, float *out, const uint32_t *act, const uint32_t *w, int n, int pairs) {
   static const int forced_r = env_int("HTPOPS_GEMV_ROWS", 0);
@@ -619,6 +750,31 @@ hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *cons
   }
   return wt == kQ4_0 ? launch_gemv_shared<kQ4_0>(stream, grp, count, static_cast<const uint32_t *>(act), nblk / 2) :
                        launch_gemv_shared<kQ8_0>(stream, grp, count, static_cast<const uint32_t *>(act), nblk / 2);
+}
+
+bool gemv_rows_fits(int m, int k, WeightType wt) {
+  // measured on Llama-7B shapes: with Q8_0 weights the kernel beats the K-sliced one up to 4 rows; with Q4_0 weights
+  // (whose activation pairs cost a sum of their bytes each) it beats the repacked-weight kernel at 2 rows only
+  const int nblk = k / kQK;
+  return m >= 2 && m <= (wt == kQ4_0 ? 2 : 4) && k % (2 * kQK) == 0 && nblk / 2 <= kSharedActMaxPairs && shared_act_enabled() &&
+         env_int("HTPOPS_GEMV_ROWS_KERNEL", 1) != 0;
+}
+
+hipError_t launch_gemv_rows_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *act,
+                                           const void *const *weights, const int *ns, int m, int k, WeightType wt) {
+  if (count < 1 || count > kGemvGroupMax || !gemv_rows_fits(m, k, wt) || (reinterpret_cast<uintptr_t>(act) & 3) != 0) {
+    return hipErrorNotSupported;
+  }
+  GemvGroupArgs grp = {};
+  for (int i = 0; i < count; ++i) {
+    if ((reinterpret_cast<uintptr_t>(weights[i]) & 3) != 0) {
+      return hipErrorNotSupported;
+    }
+    grp.w[i] = static_cast<const uint32_t *>(weights[i]), grp.out[i] = outs[i], grp.n[i] = ns[i];
+  }
+  const int pairs = k / kQK / 2;
+  return wt == kQ4_0 ? launch_gemv_rows_shared<kQ4_0>(stream, grp, count, static_cast<const uint32_t *>(act), pairs, m) :
+                       launch_gemv_rows_shared<kQ8_0>(stream, grp, count, static_cast<const uint32_t *>(act), pairs, m);
 }
 
 }  // namespace htpops

@@ -489,6 +489,14 @@ int run_mat_mul(htpops_context *ctx, MatMulPlan &plan, float *dst, const void *a
     ctx->act_fragments.src = nullptr;  // these kernels put something else at the start of the workspace
   }
   if (!plan.fragments) {
+    if (htpops::gemv_rows_fits(m, k, (htpops::WeightType) wt) && aligned(act, 4) && aligned(weight, 4)) {
+      const hipError_t e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, 1, &dst, act, &weight, &n, m, k,
+                                                                   (htpops::WeightType) wt);
+      if (e == hipSuccess) {
+        return HTPOPS_OK;
+      }
+      (void) hipGetLastError();
+    }
     if (const void *lw = lane_order_weights(ctx, weight, m, k, n, wt)) {
       HTPOPS_HIP(ctx, htpops::launch_matmul_lane_order_group(ctx->stream, 1, &dst, act, &lw, &n, m, k));
       return HTPOPS_OK;
@@ -1007,6 +1015,10 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
     hipError_t e;
     if (b.m == 1) {
       e = htpops::launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k, (htpops::WeightType) b.wt);
+    } else if (htpops::gemv_rows_fits(b.m, b.k, (htpops::WeightType) b.wt)) {
+      // 2..4 rows: the decode kernel's weight stream with the rows staged in LDS, whatever n and the weight type
+      e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.m, b.k,
+                                                  (htpops::WeightType) b.wt);
     } else {
       // Members whose weights have (or get) a repacked copy go to the kernel that streams it, the others to the
       // K-sliced kernel: which kernel a matrix gets depends on that matrix alone, so a request gives the same bits

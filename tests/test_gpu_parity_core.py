@@ -296,6 +296,26 @@ def test_small_batch_repeated_launches_are_bit_identical(ctx):
         assert np.abs(one[0] - first[r]).max() <= 2e-5 * np.abs(one).max()
 
 
+@pytest.mark.parametrize("wt,m", [(wl.GGML_TYPE_Q4_0, 2), (wl.GGML_TYPE_Q8_0, 2), (wl.GGML_TYPE_Q8_0, 3), (wl.GGML_TYPE_Q8_0, 4)])
+@pytest.mark.parametrize("k,n", [(64, 1), (128, 33), (1024, 100), (4096, 4096), (11008, 272), (12288, 64), (2048 + 64, 1000)])
+def test_two_to_four_rows_on_the_decode_kernels_weight_stream(ctx, oracle, monkeypatch, wt, m, k, n):
+    # 2 rows (Q4_0) and 2..4 rows (Q8_0) run the decode kernel's stream over the weights with the rows staged in LDS.
+    # Against the oracle, against the kernels they replace (HTPOPS_GEMV_ROWS_KERNEL=0), bit for bit on a repeat, and
+    # every row against the one-row kernel (same block sums and lane mapping; the compiler is free to fuse the scale
+    # multiplications differently in the two kernels, so to rounding).
+    rng = wl.rng_for(69, wt * 1000 + m * 100 + k + n)
+    got, x, w = check_mat_mul(ctx, oracle, rng, m, k, n, wt)
+    a = oracle.quantize_q8_0(x)
+    assert np.array_equal(ctx.run_mat_mul(a, w, m, k, n, wt), got)
+    _, mag = oracle.mat_mul_q8_0_act_f64(a, w, m, k, n, wt)
+    for r in range(m):
+        one = ctx.run_mat_mul(a[r:r + 1], w, 1, k, n, wt)[0]
+        assert np.all(np.abs(one - got[r]) <= 1e-6 * mag[r]), "row %d differs from the one-row kernel" % r
+    monkeypatch.setenv("HTPOPS_GEMV_ROWS_KERNEL", "0")
+    other = ctx.run_mat_mul(a, w, m, k, n, wt)
+    assert np.all(np.abs(other - got) <= 2 * MATMUL_RTOL * mag)
+
+
 @pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
 def test_mat_mul_on_both_sides_of_every_kernel_switch(ctx, oracle, wt):
     # which kernel a matmul takes depends on m (1 | 2..8 | 9..16 | 17..32 | 33..), on k (multiples of 32, 64, 256; the
