@@ -429,11 +429,11 @@ const void *lane_order_weights(htpops_context *ctx, const void *weight, int m, i
     return nullptr;
   }
   void *fresh = nullptr;
-  if (hipMalloc(&fresh, htpops::matmul_lane_order_weight_bytes(k, n)) != hipSuccess) {
+  if (hipMalloc(&fresh, htpops::matmul_lane_order_weight_bytes(k, n, (htpops::WeightType) wt)) != hipSuccess) {
     (void) hipGetLastError();
     return nullptr;
   }
-  if (htpops::launch_q4_0_to_lane_order(ctx->stream, fresh, weight, k, n) != hipSuccess) {
+  if (htpops::launch_weights_to_lane_order(ctx->stream, fresh, weight, k, n, (htpops::WeightType) wt) != hipSuccess) {
     (void) hipGetLastError();
     (void) hipFree(fresh);
     return nullptr;
@@ -498,7 +498,8 @@ int run_mat_mul(htpops_context *ctx, MatMulPlan &plan, float *dst, const void *a
       (void) hipGetLastError();
     }
     if (const void *lw = lane_order_weights(ctx, weight, m, k, n, wt)) {
-      HTPOPS_HIP(ctx, htpops::launch_matmul_lane_order_group(ctx->stream, 1, &dst, act, &lw, &n, m, k));
+      HTPOPS_HIP(ctx, htpops::launch_matmul_lane_order_group(ctx->stream, 1, &dst, act, &lw, &n, m, k,
+                                                             (htpops::WeightType) wt));
       return HTPOPS_OK;
     }
     HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, act, weight, m, k, n, (htpops::WeightType) wt, ws,
@@ -1038,7 +1039,8 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
       }
       e = hipSuccess;
       if (count_a > 0) {
-        e = htpops::launch_matmul_lane_order_group(ctx->stream, count_a, out_a, b.act, w_a, n_a, b.m, b.k);
+        e = htpops::launch_matmul_lane_order_group(ctx->stream, count_a, out_a, b.act, w_a, n_a, b.m, b.k,
+                                                   (htpops::WeightType) b.wt);
       }
       if (e == hipSuccess && count_b > 0) {
         const size_t ws = htpops::matmul_skinny_group_workspace_bytes(count_b, n_b, b.m, b.k);

@@ -47,16 +47,17 @@ size_t     matmul_skinny_group_workspace_bytes(int count, const int *ns, int m, 
 hipError_t launch_matmul_skinny_group(hipStream_t stream, int count, float *const *outs, const void *act,
                                       const void *const *weights, const int *ns, int m, int k, WeightType wt,
                                       void *workspace, unsigned *tickets, int ticket_slots);
-// 2 <= m <= 16 rows against Q4_0 weights repacked once (launch_q4_0_to_lane_order into
+// 2 <= m <= 16 rows against Q4_0 or Q8_0 weights repacked once (launch_weights_to_lane_order into
 // matmul_lane_order_weight_bytes, same size as the weights; the caller can cache the copy) into matrix-core operand
 // order: every workgroup streams a tile of 16 rows over the whole of K, nothing is exchanged between workgroups.
 // Fits when n % 16 == 0 and k % 256 == 0 and the 8 (m <= 8) or 16 activation rows of length k fit LDS; `act` must be
 // 16-byte aligned.
 bool       matmul_lane_order_fits(int n, int m, int k, WeightType wt);
-size_t     matmul_lane_order_weight_bytes(int k, int n);
-hipError_t launch_q4_0_to_lane_order(hipStream_t stream, void *dst, const void *weight, int k, int n);
+size_t     matmul_lane_order_weight_bytes(int k, int n, WeightType wt);
+hipError_t launch_weights_to_lane_order(hipStream_t stream, void *dst, const void *weight, int k, int n, WeightType wt);
 hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *const *outs, const void *act,
-                                          const void *const *lane_order_weights, const int *ns, int m, int k);
+                                          const void *const *lane_order_weights, const int *ns, int m, int k,
+                                          WeightType wt);
 // many-row path: int8 MFMA over operands in fragment order. The weights are converted once
 // (launch_weights_to_i8_fragments into gemm_i8_weight_fragment_bytes) and can be cached by the caller; the
 // activations are converted per call into `act_fragments` (gemm_i8_act_fragment_bytes), unless the caller says that

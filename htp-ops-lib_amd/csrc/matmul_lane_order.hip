@@ -34,8 +34,9 @@ constexpr int kLoThreads  = 512;
 constexpr int kLoWaves    = kLoThreads / kWave;
 constexpr int kLoRows     = 16;                       // weight rows per tile
 constexpr int kLoMaxActRows = 16;                     // the matrix instruction's other side: 16 activation rows
-constexpr int kLoQuadBytes = 64 * 16 + kLoRows * 8;   // 1152 = 16 rows x 4 blocks x 18 B
-constexpr int kLoChunk    = 4;                        // quads a wave fetches at a time
+constexpr int kLoQuadBytes = 64 * 16 + kLoRows * 8;   // 1152 = 16 rows x 4 blocks x 18 B (Q4_0)
+constexpr int kLoQuadBytesQ8 = 64 * 32 + kLoRows * 8; // 2176 = 16 rows x 4 blocks x 34 B (Q8_0)
+constexpr int quad_bytes(int wt) { return wt == kQ4_0 ? kLoQuadBytes : kLoQuadBytesQ8; }
 constexpr size_t kLoLdsLimit = 160 * 1024;
 
 // ---- repack: one thread per (tile, quad, lane) writes its 16 nibble bytes; lanes 0..15 also write the scales ----
@@ -71,24 +72,69 @@ __global__ __launch_bounds__(256) void q4_0_to_lane_order_kernel(uint8_t *__rest
   }
 }
 
+// Q8_0: the same tile and quad, 2048 B: lane l's 32 bytes = for each of the 4 blocks its 8 int8 operand bytes, elements
+// {4 g .. 4 g + 3, 16 + 4 g .. 16 + 4 g + 3} -- the element order the Q4_0 nibbles unpack to, so that the activation
+// operand is formed the same way for both weight types; then the 128 B of scales.
+__global__ __launch_bounds__(256) void q8_0_to_lane_order_kernel(uint8_t *__restrict__ dst,
+                                                                const uint8_t *__restrict__ src, int nblk, int n) {
+  const int    nquads = nblk / 4;
+  const size_t item   = (size_t) blockIdx.x * 256 + threadIdx.x;  // (tile * nquads + quad) * 64 + lane
+  const size_t total  = (size_t) (n / kLoRows) * nquads * 64;
+  if (item >= total) {
+    return;
+  }
+  const int    lane = (int) (item & 63), nl = lane & 15, g = lane >> 4;
+  const size_t tq   = item >> 6;
+  const int    quad = (int) (tq % nquads);
+  const size_t tile = tq / nquads;
+  const uint8_t *row = src + ((size_t) (tile * kLoRows + nl) * nblk + 4 * (size_t) quad) * 34;
+  uint8_t       *out = dst + tq * kLoQuadBytesQ8;
+  uint32_t       w[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const uint8_t *q = row + j * 34 + 2;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const uint8_t *e = q + 16 * half + 4 * g;
+      w[2 * j + half] = (uint32_t) e[0] | ((uint32_t) e[1] << 8) | ((uint32_t) e[2] << 16) | ((uint32_t) e[3] << 24);
+    }
+  }
+  *reinterpret_cast<uint4 *>(out + lane * 32)      = make_uint4(w[0], w[1], w[2], w[3]);
+  *reinterpret_cast<uint4 *>(out + lane * 32 + 16) = make_uint4(w[4], w[5], w[6], w[7]);
+  if (g == 0) {
+    uint16_t s[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      s[j] = (uint16_t) (row[j * 34] | (row[j * 34 + 1] << 8));
+    }
+    *reinterpret_cast<uint2 *>(out + 2048 + nl * 8) =
+      make_uint2((uint32_t) s[0] | ((uint32_t) s[1] << 16), (uint32_t) s[2] | ((uint32_t) s[3] << 16));
+  }
+}
+
 struct LaneOrderGroupArgs {
   const uint8_t *w[kGemvGroupMax];  // repacked weights
   float         *out[kGemvGroupMax];
   int            n[kGemvGroupMax];
 };
 
+template <int WT>
 struct QuadRegs {
-  uint4 q;  // this lane's nibble bytes of the 4 blocks
-  uint2 d;  // the 4 fp16 scales of this lane's row
+  uint4 q[WT == kQ4_0 ? 1 : 2];  // this lane's nibble bytes (Q4_0) or operand bytes (Q8_0) of the 4 blocks
+  uint2 d;                       // the 4 fp16 scales of this lane's row
 };
 
 // ROWS: activation rows in the LDS panel, 8 (m <= 8: lanes 32..63 repeat rows 0..7 and their results are dropped) or 16
 // TPW:  16-row weight tiles per workgroup, 1 (8 waves per tile) or 2 (4 waves per tile). The activation panel is as
 //       many bytes as a tile's weights and every workgroup fetches it from L2, so two tiles per workgroup cut the
 //       traffic into a CU by a quarter; used when that still leaves enough workgroups.
-template <int ROWS, int TPW>
+// WT:   weight type of the repacked copy; Q8_0 quads are twice the bytes, so half as many are fetched at a time
+template <int ROWS, int TPW, int WT>
 __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrderGroupArgs grp,
                                                                        const uint8_t *__restrict__ act, int m, int k) {
+  constexpr int kLoChunk    = WT == kQ4_0 ? 4 : 2;  // quads a wave fetches at a time
+  constexpr int kQuadBytes  = quad_bytes(WT);
+  constexpr int kLoads      = WT == kQ4_0 ? 2 : 3;  // load instructions per quad
   constexpr int kLoActRows  = ROWS;
   constexpr int kLoScaleBlk = ROWS * 4;  // bytes of the scale table per block (one float per row)
   extern __shared__ __align__(16) uint8_t lo_lds[];  // activation panel, later the waves' sums
@@ -103,16 +149,21 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
   // a second tile past the end of an odd tile count repeats the last one (never stored)
   const int tile = min((int) blockIdx.x * TPW + tw, n / kLoRows - 1);
   const int nblk = k / 32, nquads = nblk / 4;
-  const uint8_t *__restrict__ wt = grp.w[blockIdx.y] + (size_t) tile * nquads * kLoQuadBytes;
+  const uint8_t *__restrict__ wt = grp.w[blockIdx.y] + (size_t) tile * nquads * kQuadBytes;
   float *__restrict__         out = grp.out[blockIdx.y];
 
-  auto fetch = [&](QuadRegs (&r)[kLoChunk], int q0) {  // quads q0, q0 + 8, ... of this wave (clamped: extra ones unused)
+  auto fetch = [&](QuadRegs<WT> (&r)[kLoChunk], int q0) {  // quads q0, q0 + WQ, ... of this wave (clamped: extra ones unused)
 #pragma unroll
     for (int c = 0; c < kLoChunk; ++c) {
       const int      q = min(q0 + c * WQ, nquads - 1);
-      const uint8_t *p = wt + (size_t) q * kLoQuadBytes;
-      r[c].q           = *reinterpret_cast<const uint4 *>(p + lane * 16);
-      r[c].d           = *reinterpret_cast<const uint2 *>(p + 1024 + nl * 8);
+      const uint8_t *p = wt + (size_t) q * kQuadBytes;
+      if (WT == kQ4_0) {
+        r[c].q[0] = *reinterpret_cast<const uint4 *>(p + lane * 16);
+      } else {
+        r[c].q[0]                = *reinterpret_cast<const uint4 *>(p + lane * 32);
+        r[c].q[WT == kQ4_0 ? 0 : 1] = *reinterpret_cast<const uint4 *>(p + lane * 32 + 16);
+      }
+      r[c].d = *reinterpret_cast<const uint2 *>(p + (kQuadBytes - 128) + nl * 8);
     }
   };
   // ---- the activation rows, as they are, by DMA: piece pc of row r goes to piece slot pc * 8 + r. Rows past m repeat
@@ -128,12 +179,12 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
     const uint32_t to  = __builtin_amdgcn_readfirstlane(lds0 + (uint32_t) i * kWave * 16);
     asm volatile("s_mov_b32 m0, %1\n s_nop 0\n global_load_lds_dwordx4 %0, off" ::"v"(p), "s"(to) : "memory");
   }
-  QuadRegs cur[kLoChunk], nxt[kLoChunk];
+  QuadRegs<WT> cur[kLoChunk], nxt[kLoChunk];
   fetch(cur, wph);  // 2 kLoChunk loads, in flight behind the DMA
   // the DMA pieces of this wave have landed once only the weight loads issued after them are outstanding
   // (s_waitcnt operand: vmcnt in bits 3:0 and 15:14, expcnt (7 = no wait) in 6:4, lgkmcnt in 11:8)
-  static_assert(2 * kLoChunk == 8, "the wait below leaves exactly the weight loads in flight");
-  __builtin_amdgcn_s_waitcnt(0x0070 | 8);
+  static_assert(kLoads * kLoChunk <= 15, "the wait below leaves exactly the weight loads in flight");
+  __builtin_amdgcn_s_waitcnt(0x0070 | (kLoads * kLoChunk));
   __builtin_amdgcn_s_barrier();  // (bare barriers: __syncthreads would also wait for the weight loads)
   // block scales of all rows as floats: [block][row]
   float *s_tab = reinterpret_cast<float *>(lo_lds + a_bytes);
@@ -176,7 +227,13 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
     for (int c = 0; c < kLoChunk; ++c) {
       const int quad = q0 + c * WQ;
       if (quad < nquads) {
-        const uint32_t wq[4] = { cur[c].q.x, cur[c].q.y, cur[c].q.z, cur[c].q.w };
+        // Q4_0: wq[j] = the nibble dword of block j; Q8_0: wq[2 j], wq[2 j + 1] = the operand dwords of block j
+        uint32_t wq[8];
+        wq[0] = cur[c].q[0].x, wq[1] = cur[c].q[0].y, wq[2] = cur[c].q[0].z, wq[3] = cur[c].q[0].w;
+        if (WT != kQ4_0) {
+          const uint4 q1 = cur[c].q[WT == kQ4_0 ? 0 : 1];
+          wq[4] = q1.x, wq[5] = q1.y, wq[6] = q1.z, wq[7] = q1.w;
+        }
         union {
           uint2    u;
           _Float16 h[4];
@@ -198,7 +255,8 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
           }
           const long   a = (long) (((uint64_t) e1 << 32) | e0);
           const float4 s = *reinterpret_cast<const float4 *>(s_lane + (size_t) it * kScaleStep + j * kLoScaleBlk);
-          const long   b = (long) (((uint64_t) hi(wq[j]) << 32) | lo(wq[j]));
+          const long   b = WT == kQ4_0 ? (long) (((uint64_t) hi(wq[j]) << 32) | lo(wq[j])) :
+                                         (long) (((uint64_t) wq[2 * j + 1] << 32) | wq[2 * j]);
           const v4i    zero = { 0, 0, 0, 0 };
           const v4i    p    = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, zero, 0, 0, 0);
           const float  dw   = (float) sc.h[j];
@@ -255,33 +313,40 @@ size_t panel_bytes(int k, int rows) {
 
 bool matmul_lane_order_fits(int n, int m, int k, WeightType wt) {
   // k % 256: activation rows (34 B per 32 elements) are whole 16-byte pieces, weight rows whole quads of blocks
-  return wt == kQ4_0 && m >= 2 && m <= kLoMaxActRows && k > 0 && k % 256 == 0 && n > 0 && n % kLoRows == 0 &&
+  return (wt == kQ4_0 || wt == kQ8_0) && m >= 2 && m <= kLoMaxActRows && k > 0 && k % 256 == 0 && n > 0 && n % kLoRows == 0 &&
          panel_bytes(k, panel_rows(m)) <= kLoLdsLimit && n / kLoRows <= 0x7fffffff;
 }
 
-size_t matmul_lane_order_weight_bytes(int k, int n) {
-  return (size_t) (n / kLoRows) * (size_t) (k / 128) * kLoQuadBytes;
+size_t matmul_lane_order_weight_bytes(int k, int n, WeightType wt) {
+  return (size_t) (n / kLoRows) * (size_t) (k / 128) * quad_bytes(wt);
 }
 
-hipError_t launch_q4_0_to_lane_order(hipStream_t stream, void *dst, const void *weight, int k, int n) {
-  if (k % 128 != 0 || n % kLoRows != 0) {
+hipError_t launch_weights_to_lane_order(hipStream_t stream, void *dst, const void *weight, int k, int n, WeightType wt) {
+  if (k % 128 != 0 || n % kLoRows != 0 || (wt != kQ4_0 && wt != kQ8_0)) {
     return hipErrorNotSupported;
   }
   const size_t items = (size_t) (n / kLoRows) * (size_t) (k / 128) * 64;
-  hipLaunchKernelGGL(q4_0_to_lane_order_kernel, dim3((unsigned) ((items + 255) / 256)), dim3(256), 0, stream,
-                     static_cast<uint8_t *>(dst), static_cast<const uint8_t *>(weight), k / 32, n);
+  const dim3   grid((unsigned) ((items + 255) / 256));
+  if (wt == kQ4_0) {
+    hipLaunchKernelGGL(q4_0_to_lane_order_kernel, grid, dim3(256), 0, stream, static_cast<uint8_t *>(dst),
+                       static_cast<const uint8_t *>(weight), k / 32, n);
+  } else {
+    hipLaunchKernelGGL(q8_0_to_lane_order_kernel, grid, dim3(256), 0, stream, static_cast<uint8_t *>(dst),
+                       static_cast<const uint8_t *>(weight), k / 32, n);
+  }
   return hipGetLastError();
 }
 
 hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *const *outs, const void *act,
-                                          const void *const *lane_order_weights, const int *ns, int m, int k) {
+                                          const void *const *lane_order_weights, const int *ns, int m, int k,
+                                          WeightType wt) {
   if (count < 1 || count > kGemvGroupMax) {
     return hipErrorNotSupported;
   }
   LaneOrderGroupArgs grp = {};
   int                n_max = 0;
   for (int i = 0; i < count; ++i) {
-    if (!matmul_lane_order_fits(ns[i], m, k, kQ4_0) || (reinterpret_cast<uintptr_t>(lane_order_weights[i]) & 15) != 0 ||
+    if (!matmul_lane_order_fits(ns[i], m, k, wt) || (reinterpret_cast<uintptr_t>(lane_order_weights[i]) & 15) != 0 ||
         (reinterpret_cast<uintptr_t>(act) & 15) != 0) {
       return hipErrorNotSupported;
     }
@@ -291,12 +356,15 @@ hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *
     n_max      = ns[i] > n_max ? ns[i] : n_max;
   }
   typedef void (*Kernel)(LaneOrderGroupArgs, const uint8_t *, int, int);
-  static const Kernel kernels[2][2] = { { matmul_lane_order_kernel<8, 1>, matmul_lane_order_kernel<8, 2> },
-                                        { matmul_lane_order_kernel<16, 1>, matmul_lane_order_kernel<16, 2> } };
+  static const Kernel kernels[2][2][2] = {
+    { { matmul_lane_order_kernel<8, 1, kQ4_0>, matmul_lane_order_kernel<8, 2, kQ4_0> },
+      { matmul_lane_order_kernel<16, 1, kQ4_0>, matmul_lane_order_kernel<16, 2, kQ4_0> } },
+    { { matmul_lane_order_kernel<8, 1, kQ8_0>, matmul_lane_order_kernel<8, 2, kQ8_0> },
+      { matmul_lane_order_kernel<16, 1, kQ8_0>, matmul_lane_order_kernel<16, 2, kQ8_0> } } };
   static bool attr_set = false;  // more than the default 64 KiB of dynamic LDS for long rows
   if (!attr_set) {
-    for (int i = 0; i < 4; ++i) {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernels[i / 2][i % 2]),
+    for (int i = 0; i < 8; ++i) {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernels[i / 4][(i / 2) % 2][i % 2]),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int) kLoLdsLimit);
       if (e != hipSuccess) {
         return e;
@@ -315,7 +383,7 @@ hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *
   const dim3   grid((unsigned) ((n_max / kLoRows + tpw - 1) / tpw), (unsigned) count);
   const int    rows = panel_rows(m);
   const size_t lds  = panel_bytes(k, rows);
-  hipLaunchKernelGGL(kernels[rows == 16][tpw - 1], grid, dim3(kLoThreads), lds, stream, grp,
+  hipLaunchKernelGGL(kernels[wt == kQ8_0][rows == 16][tpw - 1], grid, dim3(kLoThreads), lds, stream, grp,
                      static_cast<const uint8_t *>(act), m, k);
   return hipGetLastError();
 }

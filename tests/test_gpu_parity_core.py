@@ -424,29 +424,30 @@ def test_message_shares_one_activation_conversion_between_many_row_matmuls(ctx, 
             ctx.release(h)
 
 
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
 @pytest.mark.parametrize("m,k,n", [(2, 256, 16), (8, 256, 48), (3, 512, 4096), (8, 4096, 4096), (5, 11008, 272), (8, 2048 + 256, 1024),
                                    (7, 8960, 1536), (9, 256, 32), (16, 4096, 4096), (12, 2048 + 256, 1040), (13, 8192, 48),
                                    (16, 8960, 64), (11, 11008, 64)])
-def test_few_rows_over_repacked_weights(ctx, oracle, monkeypatch, m, k, n):
-    # 2..16 rows against Q4_0 weights with n % 16 == 0, k % 256 == 0 run on a copy of the weights repacked into
+def test_few_rows_over_repacked_weights(ctx, oracle, monkeypatch, wt, m, k, n):
+    # 2..16 rows against Q4_0 or Q8_0 weights with n % 16 == 0, k % 256 == 0 run on a copy of the weights repacked into
     # matrix-core operand order (9..16 rows only while 16 activation rows fit the LDS panel: k = 8960 does not,
     # nor 11008; they take the K-sliced kernel). It must meet the oracle, agree with the kernels that read the weights as they are
     # (switch HTPOPS_LANE_ORDER=0) to summation order, and repeat bit for bit.
-    rng = wl.rng_for(66, m * 17 + k + n)
-    got, x, w = check_mat_mul(ctx, oracle, rng, m, k, n, wl.GGML_TYPE_Q4_0)
+    rng = wl.rng_for(66, m * 17 + k + n + wt)
+    got, x, w = check_mat_mul(ctx, oracle, rng, m, k, n, wt)
     a = oracle.quantize_q8_0(x)
-    assert np.array_equal(ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0), got)
-    _, mag = oracle.mat_mul_q8_0_act_f64(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
+    assert np.array_equal(ctx.run_mat_mul(a, w, m, k, n, wt), got)
+    _, mag = oracle.mat_mul_q8_0_act_f64(a, w, m, k, n, wt)
     # one and two weight tiles per workgroup (the launcher picks by the number of tiles) sum the same blocks in
     # different wave order
     for tiles in ("1", "2"):
         monkeypatch.setenv("HTPOPS_LANE_ORDER_TILES", tiles)
-        forced = ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
+        forced = ctx.run_mat_mul(a, w, m, k, n, wt)
         assert np.all(np.abs(forced - got) <= 2 * MATMUL_RTOL * mag)
-        assert np.array_equal(forced, ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0))
+        assert np.array_equal(forced, ctx.run_mat_mul(a, w, m, k, n, wt))
     monkeypatch.delenv("HTPOPS_LANE_ORDER_TILES")
     monkeypatch.setenv("HTPOPS_LANE_ORDER", "0")
-    plain = ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
+    plain = ctx.run_mat_mul(a, w, m, k, n, wt)
     assert np.all(np.abs(plain - got) <= 2 * MATMUL_RTOL * mag)
 
 
