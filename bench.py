@@ -16,6 +16,7 @@ The same run also measures, and reports inside the JSON line:
   recorded_message_us_per_step   the m = 1 and m = 8 steps again, each layer's message recorded once into a HIP graph
                 and replayed (reported beside `value`, which is the ordinary message walk)
   q8_0_block    the Qwen2-1.5B-like Q8_0 block of config 4 at m = 1 and m = 128
+  decode_chain_us   config 0: RMSNorm -> Q8_0 -> GEMV (4096 x 4096) for one token, submitted as one message
   attention     config 3: decode (1 x 4096) and causal prefill (2048 x 2048), 32 query / 8 KV heads of 128, fp16
   launches      the four kernel launches of the step one by one (q+k+v, o, gate+up, down) on cold weights
   cpu_baseline  the scalar C oracle (a port of the same arithmetic) on the host cores, same layer, m = 1
@@ -262,6 +263,39 @@ def main():
         log("prefill GEMM m=512 n=%d k=%d: %.1f us  %.1f Tops (%.1f%% of 5 Pop/s)" % (n, k, us, tops, tops / 50))
         ctx.release(ha), ctx.release(ho)
 
+    # ------------------------------------------------------------------ decode chain (config 0)
+    # RMSNorm -> Q8_0 -> GEMV (4096 x 4096, Q4_0) for one token as one message: the fused norm + quantize op and the
+    # GEMV, i.e. two launches; weights rotate over the layers like the main step
+    rng0 = wl.rng_for(0, 1)
+    x0 = wl.make_activations(rng0, 1, 4096)
+    h_x0, h_q0, h_o0 = ctx.upload(x0), ctx.alloc(4096 // 32 * 34), ctx.alloc(4096 * 4)
+    h_g0 = ctx.upload(np.ones(4096, np.float32))
+    chain_msgs = [api.build_message([
+        (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(api.HTP_OPS_RMS_NORM_QUANTIZE_Q8_0,
+                                                             api.rms_norm_ex_params((h_q0, 0), (h_x0, 0), (h_g0, 0), 4096, 1, 1e-6))),
+        (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(api.HTP_OPS_MAT_MUL_Q4_0_Q8_0,
+                                                             api.mat_mul_params((h_o0, 0), (h_q0, 0), (layers[l][0], 0), 1, 4096, 4096)))])
+        for l in range(LAYERS)]
+    assert ctx.process_message(chain_msgs[0]) == 0
+    check_states(chain_msgs[0])
+    a0 = orc.quantize_q8_0(orc.rms_norm(x0, np.ones(4096, np.float32), 1e-6))
+    got0 = ctx.read(h_o0, np.float32, 4096)
+    rows0 = np.unique(np.linspace(0, 4095, 96).astype(int))
+    want0, mag0 = orc.mat_mul_q8_0_act_f64(a0, uniq[(4096, 4096)][rows0], 1, 4096, len(rows0), Q4)
+    # (the GPU's normalized row may differ from the oracle's in the last bit before quantization: a loose bound here,
+    # the bit-exact chain is in the tests)
+    assert np.all(np.abs(got0[rows0] - want0[0]) <= 2e-2 * mag0[0]), "decode chain outside tolerance"
+    for s_ in range(LAYERS):
+        ctx.enqueue_message(chain_msgs[s_ % LAYERS])
+    ctx.synchronize()
+    ctx.timer_start()
+    for s_ in range(200):
+        ctx.enqueue_message(chain_msgs[s_ % LAYERS])
+    chain_us = ctx.timer_stop_ms() * 1e3 / 200
+    log("decode chain (fused RMSNorm+Q8_0, then GEMV 4096x4096): %.2f us per token and layer slot" % chain_us)
+    for h in (h_x0, h_q0, h_o0, h_g0):
+        ctx.release(h)
+
     # ------------------------------------------------------------------ Q8_0 block (config 4), m = 1 and m = 128
     # same protocol as the headline step: one message per layer, 8 layers of distinct weights (8 x 49.7 MB) rotated
     rng4 = wl.rng_for(4, 0)
@@ -411,6 +445,7 @@ def main():
                         "GBps": round(layer_bytes[8] / ms_step8 / 1e6, 1)},
         "recorded_message_us_per_step": None if args.skip_recorded else
         {"m1": round(rec_step[1] * 1e3, 2), "m8": round(rec_step[8] * 1e3, 2)},
+        "decode_chain_us": round(chain_us, 2),
         "attention": attention,
         "q8_0_block": [q8_block[1], q8_block[128]],
         "peaks": peaks,
