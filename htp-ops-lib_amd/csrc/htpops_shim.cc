@@ -14,6 +14,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <string>
 #include <thread>
 #include <utility>
@@ -44,6 +45,11 @@ struct htpops_recorded_message {
 };
 
 struct htpops_context {
+  // Guards the buffer registry, the converted-copy caches, the workspace and the recordings: the channel's consumer
+  // thread walks messages (resolving handles, making copies) while the host thread may allocate, write or release
+  // buffers, as a host of the reference does while its consumer thread runs (reference: src/dsp/mmap_mgr.cc:15-27 maps
+  // lazily on that thread). Recursive: a message's RPCMEM_MAP request releases buffers from inside the walk.
+  std::recursive_mutex mu;
   int                 device     = HTPOPS_DEVICE_NONE;
   bool                has_device = false;
   hipStream_t         stream     = nullptr;
@@ -95,6 +101,8 @@ struct htpops_context {
 };
 
 namespace {
+
+using Lock = std::lock_guard<std::recursive_mutex>;
 
 int fail(htpops_context *ctx, int code, const char *fmt, ...) {
   char    buf[512];
@@ -412,34 +420,37 @@ constexpr int kFragKindFp6Panel  = 200;  // + ggml type: FP6 operand panels of t
 
 constexpr int kFragKindLaneOrder = 300;  // + ggml type: Q4_0 weights in matrix-core operand order (2..16 activation rows)
 
-// The repacked copy of `weight` for the few-row kernel: from the cache, or made now and cached. nullptr when this
-// matmul does not take that kernel (shape, weight type, weights in memory the context does not own and so cannot
-// watch for writes) or when the copy cannot be made; the caller then uses the kernels that read the weights as they are.
-const void *lane_order_weights(htpops_context *ctx, const void *weight, int m, int k, int n, int wt) {
-  if (htpops::env_int("HTPOPS_LANE_ORDER", 1) == 0 || !htpops::matmul_lane_order_fits(n, m, k, (htpops::WeightType) wt)) {
-    return nullptr;
+// The repacked copy of `weight` for the few-row kernel: from the cache, or made now and cached. *out stays nullptr when
+// this matmul does not take that kernel (shape, weight type, activations not 16-byte aligned for the DMA into LDS,
+// weights in memory the context does not own and so cannot watch for writes); the caller then uses the kernels that
+// read the weights as they are. A failed allocation or conversion launch is an error, not a reason to switch kernels.
+int lane_order_weights(htpops_context *ctx, const void *weight, const void *act, int m, int k, int n, int wt,
+                       const void **out) {
+  *out = nullptr;
+  if (htpops::env_int("HTPOPS_LANE_ORDER", 1) == 0 || !aligned(act, 16) ||
+      !htpops::matmul_lane_order_fits(n, m, k, (htpops::WeightType) wt)) {
+    return HTPOPS_OK;
   }
   const int kind = kFragKindLaneOrder + wt;
   for (const auto &e : ctx->frag_cache) {
     if (e.src == weight && e.kind == kind && e.k == k && e.n == n) {
-      return e.frag;
+      *out = e.frag;
+      return HTPOPS_OK;
     }
   }
   if (!in_owned_buffer(ctx, weight, weight_bytes((size_t) n, (size_t) k, wt))) {
-    return nullptr;
+    return HTPOPS_OK;
   }
   void *fresh = nullptr;
-  if (hipMalloc(&fresh, htpops::matmul_lane_order_weight_bytes(k, n, (htpops::WeightType) wt)) != hipSuccess) {
-    (void) hipGetLastError();
-    return nullptr;
-  }
-  if (htpops::launch_weights_to_lane_order(ctx->stream, fresh, weight, k, n, (htpops::WeightType) wt) != hipSuccess) {
-    (void) hipGetLastError();
+  HTPOPS_HIP(ctx, hipMalloc(&fresh, htpops::matmul_lane_order_weight_bytes(k, n, (htpops::WeightType) wt)));
+  const hipError_t e = htpops::launch_weights_to_lane_order(ctx->stream, fresh, weight, k, n, (htpops::WeightType) wt);
+  if (e != hipSuccess) {
     (void) hipFree(fresh);
-    return nullptr;
+    return hip_fail(ctx, e, "weight repack launch");
   }
   ctx->frag_cache.push_back({ weight, weight_bytes((size_t) n, (size_t) k, wt), kind, k, n, fresh });
-  return fresh;
+  *out = fresh;
+  return HTPOPS_OK;
 }
 
 struct MatMulPlan {
@@ -489,18 +500,33 @@ int run_mat_mul(htpops_context *ctx, MatMulPlan &plan, float *dst, const void *a
     ctx->act_fragments.src = nullptr;  // these kernels put something else at the start of the workspace
   }
   if (!plan.fragments) {
+    // hipErrorNotSupported from a launcher means "this kernel does not take the shape": try the next one. Any other
+    // failure is reported.
     if (htpops::gemv_rows_fits(m, k, (htpops::WeightType) wt) && aligned(act, 4) && aligned(weight, 4)) {
       const hipError_t e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, 1, &dst, act, &weight, &n, m, k,
                                                                    (htpops::WeightType) wt);
       if (e == hipSuccess) {
         return HTPOPS_OK;
       }
+      if (e != hipErrorNotSupported) {
+        return hip_fail(ctx, e, "few-row mat_mul launch");
+      }
       (void) hipGetLastError();
     }
-    if (const void *lw = lane_order_weights(ctx, weight, m, k, n, wt)) {
-      HTPOPS_HIP(ctx, htpops::launch_matmul_lane_order_group(ctx->stream, 1, &dst, act, &lw, &n, m, k,
-                                                             (htpops::WeightType) wt));
-      return HTPOPS_OK;
+    const void *lw = nullptr;
+    if (int r = lane_order_weights(ctx, weight, act, m, k, n, wt, &lw)) {
+      return r;
+    }
+    if (lw) {
+      const hipError_t e = htpops::launch_matmul_lane_order_group(ctx->stream, 1, &dst, act, &lw, &n, m, k,
+                                                                  (htpops::WeightType) wt);
+      if (e == hipSuccess) {
+        return HTPOPS_OK;
+      }
+      if (e != hipErrorNotSupported) {
+        return hip_fail(ctx, e, "repacked-weight mat_mul launch");
+      }
+      (void) hipGetLastError();
     }
     HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, act, weight, m, k, n, (htpops::WeightType) wt, ws,
                                                     ctx->tickets, kTicketSlots));
@@ -606,19 +632,31 @@ int op_mat_mul_permuted(htpops_context *ctx, float *dst, const float *act, const
       break;
     }
   }
+  // Converted copies are kept only for weights in buffers the context allocated (their contents change only through
+  // htpops_buffer_write or as an op's output, both of which drop the copy). Caller-registered memory may be rewritten
+  // behind the context's back: it is converted into the workspace on every call.
+  const size_t act_bytes  = (htpops::permuted_act_fragment_bytes(m, k) + 255) & ~(size_t) 255;
+  const size_t frag_bytes = htpops::permuted_weight_fragment_bytes(k, n);
+  const bool   cacheable  = !frag && in_owned_buffer(ctx, weight, permuted_weight_bytes((size_t) n, (size_t) k, kind));
+  if (int r = ensure_workspace(ctx, act_bytes + ((frag || cacheable) ? 0 : frag_bytes))) {
+    return r;
+  }
   if (!frag) {
-    void *fresh = nullptr;
-    HTPOPS_HIP(ctx, hipMalloc(&fresh, htpops::permuted_weight_fragment_bytes(k, n)));
+    void *fresh = static_cast<uint8_t *>(ctx->workspace) + act_bytes;
+    if (cacheable) {
+      HTPOPS_HIP(ctx, hipMalloc(&fresh, frag_bytes));
+    }
     const hipError_t e = htpops::launch_permuted_weight_to_fragments(ctx->stream, fresh, weight, k, n, kind);
     if (e != hipSuccess) {
-      (void) hipFree(fresh);
+      if (cacheable) {
+        (void) hipFree(fresh);
+      }
       return fail(ctx, HTPOPS_ERR_HIP, "weight conversion: %s", hipGetErrorString(e));
     }
-    ctx->frag_cache.push_back({ weight, permuted_weight_bytes((size_t) n, (size_t) k, kind), kind, k, n, fresh });
+    if (cacheable) {
+      ctx->frag_cache.push_back({ weight, permuted_weight_bytes((size_t) n, (size_t) k, kind), kind, k, n, fresh });
+    }
     frag = fresh;
-  }
-  if (int r = ensure_workspace(ctx, htpops::permuted_act_fragment_bytes(m, k))) {
-    return r;
   }
   HTPOPS_HIP(ctx, htpops::launch_mat_mul_fragments(ctx->stream, dst, act, frag, m, k, n, ctx->workspace));
   return HTPOPS_OK;
@@ -764,6 +802,7 @@ extern "C" int htpops_buffer_alloc(htpops_context *ctx, size_t bytes) {
   if (!ctx || bytes == 0) {
     return fail(ctx, HTPOPS_ERR_REJECTED, "buffer_alloc: zero size");
   }
+  Lock lock(ctx->mu);
   void *p = nullptr;
   if (ctx->has_device) {
     HTPOPS_HIP(ctx, hipMalloc(&p, bytes));
@@ -788,6 +827,7 @@ extern "C" int htpops_buffer_register(htpops_context *ctx, void *device_ptr, siz
   if (!ctx || !device_ptr || bytes == 0) {
     return fail(ctx, HTPOPS_ERR_REJECTED, "buffer_register: null pointer or zero size");
   }
+  Lock lock(ctx->mu);
   return new_handle(ctx, device_ptr, bytes, false);
 }
 
@@ -795,6 +835,7 @@ extern "C" int htpops_buffer_release(htpops_context *ctx, int handle) {
   if (!ctx) {
     return HTPOPS_ERR_REJECTED;
   }
+  Lock lock(ctx->mu);
   Buffer *b = lookup(ctx, handle);
   if (!b) {
     return HTPOPS_OK;  // unknown handles are ignored (reference: mmap_mgr.cc:29-37)
@@ -818,17 +859,44 @@ extern "C" int htpops_buffer_release(htpops_context *ctx, int handle) {
 }
 
 extern "C" void *htpops_buffer_device_ptr(htpops_context *ctx, int handle) {
-  Buffer *b = ctx ? lookup(ctx, handle) : nullptr;
+  if (!ctx) {
+    return nullptr;
+  }
+  Lock    lock(ctx->mu);
+  Buffer *b = lookup(ctx, handle);
   return b ? b->ptr : nullptr;
 }
 
 extern "C" size_t htpops_buffer_size(htpops_context *ctx, int handle) {
-  Buffer *b = ctx ? lookup(ctx, handle) : nullptr;
+  if (!ctx) {
+    return 0;
+  }
+  Lock    lock(ctx->mu);
+  Buffer *b = lookup(ctx, handle);
   return b ? b->size : 0;
 }
 
+// For owned weight buffers that the caller's own kernels have rewritten through htpops_buffer_device_ptr: drops the
+// converted copies made from the buffer and marks recordings that use it stale.
+extern "C" int htpops_buffer_invalidate(htpops_context *ctx, int handle) {
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  Lock    lock(ctx->mu);
+  Buffer *b = lookup(ctx, handle);
+  if (!b) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "buffer_invalidate: unknown handle %d", handle);
+  }
+  drop_fragments(ctx, b->ptr, b->size);
+  return HTPOPS_OK;
+}
+
 extern "C" int htpops_buffer_write(htpops_context *ctx, int handle, size_t offset, const void *src, size_t bytes) {
-  Buffer *b = ctx ? lookup(ctx, handle) : nullptr;
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  Lock    lock(ctx->mu);
+  Buffer *b = lookup(ctx, handle);
   if (!b || !src || offset > b->size || bytes > b->size - offset) {
     return fail(ctx, HTPOPS_ERR_REJECTED, "buffer_write: unknown handle or range outside the buffer");
   }
@@ -844,7 +912,11 @@ extern "C" int htpops_buffer_write(htpops_context *ctx, int handle, size_t offse
 }
 
 extern "C" int htpops_buffer_read(htpops_context *ctx, int handle, size_t offset, void *dst, size_t bytes) {
-  Buffer *b = ctx ? lookup(ctx, handle) : nullptr;
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  Lock    lock(ctx->mu);
+  Buffer *b = lookup(ctx, handle);
   if (!b || !dst || offset > b->size || bytes > b->size - offset) {
     return fail(ctx, HTPOPS_ERR_REJECTED, "buffer_read: unknown handle or range outside the buffer");
   }
@@ -864,6 +936,7 @@ extern "C" int htpops_execute_op(htpops_context *ctx, const struct OpComputeRequ
   if (!ctx || !req) {
     return HTPOPS_ERR_REJECTED;
   }
+  Lock lock(ctx->mu);
   switch (req->op) {
     case HTP_OPS_RMS_NORM_F32:
       {
@@ -1028,7 +1101,10 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
       const void *w_a[htpops::kGemvGroupMax], *w_b[htpops::kGemvGroupMax];
       int         n_a[htpops::kGemvGroupMax], n_b[htpops::kGemvGroupMax], count_a = 0, count_b = 0;
       for (int i = 0; i < b.count; ++i) {
-        if (const void *lw = lane_order_weights(ctx, b.w[i], b.m, b.k, b.n[i], b.wt)) {
+        const void *lw = nullptr;
+        if (int r = lane_order_weights(ctx, b.w[i], b.act, b.m, b.k, b.n[i], b.wt, &lw)) {
+          b.hdr[i]->state = r;
+        } else if (lw) {
           out_a[count_a] = b.out[i], w_a[count_a] = lw, n_a[count_a++] = b.n[i];
         } else if (b.m <= kSkinnyGroupMaxM) {
           out_b[count_b] = b.out[i], w_b[count_b] = b.w[i], n_b[count_b++] = b.n[i];
@@ -1192,6 +1268,7 @@ extern "C" int htpops_enqueue_message(htpops_context *ctx, struct MessageHeader 
   if (!ctx || !msg) {
     return HTPOPS_ERR_REJECTED;
   }
+  Lock lock(ctx->mu);
   return enqueue_message(ctx, msg, msg_bytes);
 }
 
@@ -1218,7 +1295,7 @@ extern "C" int htpops_process_message(htpops_context *ctx, struct MessageHeader 
   if (!ctx || !msg) {
     return HTPOPS_ERR_REJECTED;
   }
-  int ret = enqueue_message(ctx, msg, msg_bytes);
+  int ret = htpops_enqueue_message(ctx, msg, msg_bytes);
   if (ret != HTPOPS_OK) {
     return ret;
   }
@@ -1232,6 +1309,7 @@ extern "C" int htpops_record_message(htpops_context *ctx, struct MessageHeader *
   if (!ctx || !msg || !out) {
     return HTPOPS_ERR_REJECTED;
   }
+  Lock lock(ctx->mu);
   *out = nullptr;
   if (int r = need_device(ctx)) {
     return r;
@@ -1309,6 +1387,7 @@ extern "C" int htpops_launch_recorded_message(htpops_context *ctx, htpops_record
   if (!ctx || !rec || rec->ctx != ctx) {
     return HTPOPS_ERR_REJECTED;
   }
+  Lock lock(ctx->mu);
   if (rec->stale) {
     return fail(ctx, HTPOPS_ERR_REJECTED,
                 "launch_recorded_message: buffers were released or rewritten since the message was recorded; record it again");
@@ -1324,6 +1403,7 @@ extern "C" int htpops_release_recorded_message(htpops_context *ctx, htpops_recor
   if (!ctx || !rec || rec->ctx != ctx) {
     return HTPOPS_ERR_REJECTED;
   }
+  Lock lock(ctx->mu);
   (void) hipStreamSynchronize(ctx->stream);
   if (rec->exec) {
     (void) hipGraphExecDestroy(rec->exec);
@@ -1437,33 +1517,56 @@ extern "C" int htpops_mat_mul_permuted_w16a32(htpops_context *ctx, int output_fd
 
 extern "C" int htpops_rms_norm_f32_ex_ptr(htpops_context *ctx, float *dst, const float *src, const float *weight,
                                           float eps, int ne0, int ne1) {
-  return ctx ? op_rms_norm(ctx, dst, src, weight, eps, ne0, ne1) : HTPOPS_ERR_REJECTED;
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  Lock lock(ctx->mu);
+  return op_rms_norm(ctx, dst, src, weight, eps, ne0, ne1);
 }
 
 extern "C" int htpops_quantize_q8_0_ptr(htpops_context *ctx, void *dst, const float *src, int k, int m) {
-  return ctx ? op_quantize(ctx, dst, src, k, m) : HTPOPS_ERR_REJECTED;
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  Lock lock(ctx->mu);
+  return op_quantize(ctx, dst, src, k, m);
 }
 
 extern "C" int htpops_rms_norm_quantize_q8_0_ptr(htpops_context *ctx, void *dst, const float *src,
                                                  const float *weight, float eps, int ne0, int ne1) {
-  return ctx ? op_rms_norm_quantize(ctx, dst, src, weight, eps, ne0, ne1) : HTPOPS_ERR_REJECTED;
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  Lock lock(ctx->mu);
+  return op_rms_norm_quantize(ctx, dst, src, weight, eps, ne0, ne1);
 }
 
 extern "C" int htpops_mat_mul_q8_0_act_ptr(htpops_context *ctx, float *dst, const void *act_q8_0, const void *weight,
                                            int m, int k, int n, int weight_type) {
-  return ctx ? op_mat_mul_q8(ctx, dst, act_q8_0, weight, m, k, n, weight_type) : HTPOPS_ERR_REJECTED;
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  Lock lock(ctx->mu);
+  return op_mat_mul_q8(ctx, dst, act_q8_0, weight, m, k, n, weight_type);
 }
 
 extern "C" int htpops_mat_mul_f32_act_ptr(htpops_context *ctx, float *dst, const float *act, const void *weight, int m,
                                           int k, int n, int weight_type) {
-  return ctx ? op_mat_mul_f32(ctx, dst, act, weight, m, k, n, weight_type) : HTPOPS_ERR_REJECTED;
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  Lock lock(ctx->mu);
+  return op_mat_mul_f32(ctx, dst, act, weight, m, k, n, weight_type);
 }
 
 extern "C" int htpops_flash_attn_ptr(htpops_context *ctx, void *o, const void *q, const void *k, const void *v,
                                      const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads,
                                      int head_dim, int qo_is_f32, int causal) {
-  return ctx ? op_flash_attn(ctx, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, head_dim, qo_is_f32, causal) :
-               HTPOPS_ERR_REJECTED;
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  Lock lock(ctx->mu);
+  return op_flash_attn(ctx, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, head_dim, qo_is_f32, causal);
 }
 
 // ------------------------------------------------------------------------------------------------ measurement

@@ -49,7 +49,7 @@ GGML_TYPE_Q8_0 = 8
 EXPORTED_SYMBOLS = [
     "htpops_init_backend", "htpops_close", "htpops_last_error", "htpops_synchronize", "htpops_get_stream",
     "htpops_buffer_alloc", "htpops_buffer_register", "htpops_buffer_release", "htpops_buffer_device_ptr",
-    "htpops_buffer_size", "htpops_buffer_write", "htpops_buffer_read", "htpops_execute_op",
+    "htpops_buffer_size", "htpops_buffer_invalidate", "htpops_buffer_write", "htpops_buffer_read", "htpops_execute_op",
     "htpops_process_message", "htpops_enqueue_message", "htpops_finish_message",
     "htpops_record_message", "htpops_launch_recorded_message", "htpops_release_recorded_message", "htpops_create_channel", "htpops_destroy_channel", "htpops_rms_norm_f32",
     "htpops_mat_mul_permuted_w16a32", "htpops_rms_norm_f32_ex_ptr", "htpops_quantize_q8_0_ptr",
@@ -83,6 +83,7 @@ def load_library(path=None):
         "htpops_buffer_release": (ci, [vp, ci]),
         "htpops_buffer_device_ptr": (vp, [vp, ci]),
         "htpops_buffer_size": (sz, [vp, ci]),
+        "htpops_buffer_invalidate": (ci, [vp, ci]),
         "htpops_buffer_write": (ci, [vp, ci, sz, vp, sz]),
         "htpops_buffer_read": (ci, [vp, ci, sz, vp, sz]),
         "htpops_execute_op": (ci, [vp, vp]),
@@ -225,6 +226,9 @@ class Context:
 
     def device_ptr(self, handle):
         return self.lib.htpops_buffer_device_ptr(self._ctx, int(handle))
+
+    def invalidate(self, handle):
+        return self.lib.htpops_buffer_invalidate(self._ctx, int(handle))
 
     def write(self, handle, array, offset=0):
         a = np.ascontiguousarray(array)

@@ -3,8 +3,12 @@
  *
  * One context owns one HIP stream; ops are enqueued in order on that stream
  * (the reference executes requests strictly in order on one poller thread,
- * src/dsp/commu.c:43, :91-114). A context is not thread-safe; several
- * contexts may coexist.
+ * src/dsp/commu.c:43, :91-114). Buffer calls and op/message calls on one
+ * context may come from different threads (the channel's consumer thread
+ * runs messages while the host thread allocates, writes and releases
+ * buffers): they are serialised by a lock inside the context. Ordering of
+ * the work itself is the caller's: ops run in the order they are enqueued.
+ * Several contexts may coexist.
  *
  * Return codes: 0 success, -1 rejected request (same meaning as the
  * reference's ops: bad sizes, null/unknown buffers, misalignment), other
@@ -66,9 +70,18 @@ int htpops_buffer_register(htpops_context *ctx, void *device_ptr, size_t bytes);
  * Unknown handles are ignored and return 0, as in the reference (mmap_mgr.cc:29-37). */
 int htpops_buffer_release(htpops_context *ctx, int handle);
 
-/* Device address and size of a handle (NULL / 0 if unknown). */
+/* Device address and size of a handle (NULL / 0 if unknown). The address is for the caller's own kernels and copies.
+ * The context keeps converted copies of WEIGHTS that live in buffers it allocated (made on first use by a matmul,
+ * dropped by htpops_buffer_write and by ops that write into the buffer): a caller that rewrites such a buffer through
+ * this address must say so with htpops_buffer_invalidate before the next op reads it. Activations, KV rows and
+ * outputs need nothing; caller-registered memory is never cached. */
 void  *htpops_buffer_device_ptr(htpops_context *ctx, int handle);
 size_t htpops_buffer_size(htpops_context *ctx, int handle);
+
+/* Declares the contents of a buffer changed behind the context's back (no counterpart in the reference, whose weights
+ * are immutable once mapped, src/dsp/op_executor.cc:130): converted weight copies made from it are dropped and
+ * recorded messages that use them refuse to launch. Unknown handles return -1. */
+int htpops_buffer_invalidate(htpops_context *ctx, int handle);
 
 /* Host <-> device copies ordered on the context's stream; both return after the copy is done. */
 int htpops_buffer_write(htpops_context *ctx, int handle, size_t offset, const void *src, size_t bytes);

@@ -581,3 +581,63 @@ def test_gemm_full_prefill_shape_rows_match_the_decode_kernel(ctx, oracle):
         gemv = ctx.run_mat_mul(a[r:r + 1], w, 1, k, n, wl.GGML_TYPE_Q4_0)
         scale = np.abs(gemv).max()
         assert np.abs(gemv[0] - got[r]).max() <= 2e-5 * scale
+
+
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+@pytest.mark.parametrize("m", [1, 2, 8, 16, 40])
+def test_mat_mul_with_activations_at_a_4_byte_aligned_offset(ctx, oracle, wt, m):
+    # the request only promises 2-byte aligned activations; kernels that want 16-byte alignment (the DMA of the
+    # repacked-weight kernel) must not be picked, alone or inside a message's grouped launch
+    rng = wl.rng_for(71, wt * 100 + m)
+    k, n = 1024, 256
+    op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
+    w = wl.make_weights(rng, n, k, wt)
+    a = oracle.quantize_q8_0(wl.make_activations(rng, m, k))
+    want, mag = oracle.mat_mul_q8_0_act_f64(a, w, m, k, n, wt)
+    hw, ho, ho2 = ctx.upload(w), ctx.alloc(m * n * 4), ctx.alloc(m * n * 4)
+    ha = ctx.alloc(a.nbytes + 64)
+    try:
+        for off in (4, 8, 2):
+            ctx.write(ha, a, offset=off)
+            print("offset activations m=%d wt=%d off=%d" % (m, wt, off), flush=True)
+            assert ctx.execute(op, api.mat_mul_params((ho, 0), (ha, off), (hw, 0), m, k, n)) == 0, ctx.last_error()
+            ctx.synchronize()
+            got = ctx.read(ho, np.float32, m * n).reshape(m, n)
+            assert np.all(np.abs(got - want) <= MATMUL_RTOL * mag)
+            msg = api.build_message([(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, api.mat_mul_params((h, 0), (ha, off), (hw, 0), m, k, n)))
+                                     for h in (ho, ho2)])
+            assert ctx.process_message(msg) == 0
+            assert api.message_request_states(msg) == [0, 0], ctx.last_error()
+            for h in (ho, ho2):
+                got = ctx.read(h, np.float32, m * n).reshape(m, n)
+                assert np.all(np.abs(got - want) <= MATMUL_RTOL * mag)
+    finally:
+        for h in (hw, ho, ho2, ha):
+            ctx.release(h)
+
+
+def test_buffer_invalidate_drops_converted_weight_copies(ctx, oracle):
+    # an owned weight buffer rewritten through its device address (here by a second context that has the address
+    # registered) keeps its converted copy until the caller says so
+    rng = wl.rng_for(72, 0)
+    m, k, n = 8, 512, 64
+    w1, w2 = wl.make_q4_0_weights(rng, n, k), wl.make_q4_0_weights(rng, n, k)
+    a = oracle.quantize_q8_0(wl.make_activations(rng, m, k))
+    ha, hw, ho = ctx.upload(a), ctx.upload(w1), ctx.alloc(m * n * 4)
+    try:
+        def run():
+            assert ctx.execute(api.HTP_OPS_MAT_MUL_Q4_0_Q8_0, api.mat_mul_params((ho, 0), (ha, 0), (hw, 0), m, k, n)) == 0
+            ctx.synchronize()
+            return ctx.read(ho, np.float32, m * n).reshape(m, n)
+        first = run()
+        want2, mag2 = oracle.mat_mul_q8_0_act_f64(a, w2, m, k, n, wl.GGML_TYPE_Q4_0)
+        with api.Context(device=0) as other:
+            alias = other.register(ctx.device_ptr(hw), w2.nbytes)
+            other.write(alias, w2)
+        assert np.array_equal(run(), first)          # the repacked copy of the old weights is still in use
+        assert ctx.invalidate(hw) == 0
+        assert np.all(np.abs(run() - want2) <= MATMUL_RTOL * mag2)
+        assert ctx.invalidate(987654) == -1
+    finally:
+        for h in (ha, hw, ho):
+            ctx.release(h)

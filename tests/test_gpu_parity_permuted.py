@@ -103,3 +103,25 @@ def test_permuted_matmul_rejects_what_the_reference_rejects(ctx, bad):
         assert ctx.execute(OPS[1], api.mat_mul_params((ho, 0), (ha, 0), w, m, k, n)) == -1
     finally:
         ctx.release(ha), ctx.release(hw), ctx.release(ho)
+
+
+def test_weights_in_caller_owned_memory_are_converted_on_every_call(oracle):
+    # Memory the context did not allocate can change without the context seeing it: a second context owns the buffer
+    # here and rewrites it, the first one only has it registered. No converted copy may survive between calls.
+    rng = wl.rng_for(86, 0)
+    m, k, n = 4, 128, 64
+    x = wl.make_activations(rng, m, k)
+    raws = [wl.make_permuted_weights(rng, n, k, 2) for _ in range(3)]
+    with api.Context(device=0) as owner, api.Context(device=0) as user:
+        hw_owner = owner.upload(raws[0])
+        hw = user.register(owner.device_ptr(hw_owner), raws[0].nbytes)
+        ha, ho = user.upload(x), user.alloc(m * n * 4)
+        payload = api.mat_mul_params((ho, 0), (ha, 0), (hw, 0), m, k, n)
+        for raw in (raws[0], raws[1], raws[2], raws[0]):
+            owner.write(hw_owner, raw)
+            for _ in range(2):
+                assert user.execute(OPS[2], payload) == 0
+                user.synchronize()
+                got = user.read(ho, np.float32, m * n).reshape(m, n)
+                want = oracle.mat_mul_permuted(x, raw, m, k, n, 2)
+                assert np.mean(got == want) > 0.98 and np.allclose(got, want, rtol=2e-3, atol=1e-4)
