@@ -34,6 +34,13 @@ struct Buffer {
 constexpr int kMaxHandles  = 1 << 20;
 constexpr int kTicketSlots = 1 << 16;
 
+// Device memory of the entry point that allocates nothing (htpops_flash_attn_noalloc_ptr): the split-KV partials of
+// decode attention. Every GPU the library runs on holds its own copy of this array from the moment the code object is
+// loaded until the process ends. The name is only a host-side stand-in for the symbol: host code uses the address
+// that hipGetSymbolAddress returned for the context's device (htpops_context::scratch_ptr), never the name.
+constexpr size_t kNoAllocScratchBytes = (size_t) 8 << 20;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
 }  // namespace
 
 struct htpops_recorded_message {
@@ -92,6 +99,9 @@ struct htpops_context {
   uint64_t                                   memory_generation = 0;
 
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+
+  // this device's copy of the file-scope `scratch` array (hipGetSymbolAddress at init, with the device current)
+  void *scratch_ptr = nullptr;
 
   // mailbox channel
   std::thread           poller;
@@ -663,7 +673,8 @@ int op_mat_mul_permuted(htpops_context *ctx, float *dst, const float *act, const
 }
 
 int op_flash_attn(htpops_context *ctx, void *o, const void *q, const void *k, const void *v, const void *mask,
-                  int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim, int qo_is_f32, int causal) {
+                  int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim, int qo_is_f32, int causal,
+                  bool no_alloc = false) {
   if (!o || !q || !k || !v || qo_len <= 0 || kv_len <= 0 || n_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0) {
     return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn: null buffer or non-positive size");
   }
@@ -683,12 +694,35 @@ int op_flash_attn(htpops_context *ctx, void *o, const void *q, const void *k, co
   if (int r = need_device(ctx)) {
     return r;
   }
-  if (int r = ensure_workspace(ctx, htpops::flash_attn_workspace_bytes(qo_len, kv_len, n_heads, head_dim))) {
-    return r;
+  const size_t ws_bytes = htpops::flash_attn_workspace_bytes(qo_len, kv_len, n_heads, head_dim);
+  const size_t o_bytes  = (size_t) qo_len * n_heads * head_dim * (qo_is_f32 ? 4 : 2);
+  void        *ws       = nullptr;
+  if (no_alloc) {
+    // nothing may be allocated or freed here: the partials go to this device's static scratch array, and an output
+    // that would overwrite weights with a converted copy (whose release is a hipFree) is refused instead
+    if (ws_bytes > kNoAllocScratchBytes) {
+      return fail(ctx, HTPOPS_ERR_REJECTED,
+                  "flash_attn (no allocation): %zu bytes of split-KV partials exceed the %zu-byte static scratch "
+                  "(n_heads * ceil(kv_len / 64) * (head_dim + 2) * 4 must fit)", ws_bytes, kNoAllocScratchBytes);
+    }
+    for (const auto &e : ctx->frag_cache) {
+      if (ranges_overlap(o, o_bytes, e.src, e.src_bytes)) {
+        return fail(ctx, HTPOPS_ERR_REJECTED, "flash_attn (no allocation): the output overlaps cached weights");
+      }
+    }
+    if (ctx->act_fragments.src && ranges_overlap(o, o_bytes, ctx->act_fragments.src, ctx->act_fragments.src_bytes)) {
+      ctx->act_fragments.src = nullptr;
+    }
+    ws = ctx->scratch_ptr;
+  } else {
+    if (int r = ensure_workspace(ctx, ws_bytes)) {
+      return r;
+    }
+    note_device_write(ctx, o, o_bytes);
+    ws = ctx->workspace;
   }
-  note_device_write(ctx, o, (size_t) qo_len * n_heads * head_dim * (qo_is_f32 ? 4 : 2));
   HTPOPS_HIP(ctx, htpops::launch_flash_attn(ctx->stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads,
-                                            head_dim, qo_is_f32 != 0, causal != 0, ctx->workspace));
+                                            head_dim, qo_is_f32 != 0, causal != 0, ws));
   return HTPOPS_OK;
 }
 
@@ -721,6 +755,16 @@ extern "C" int htpops_init_backend(htpops_context **out_ctx, int device) {
         hipEventCreate(&ctx->ev_start) != hipSuccess || hipEventCreate(&ctx->ev_stop) != hipSuccess ||
         hipMalloc(reinterpret_cast<void **>(&ctx->tickets), kTicketSlots * sizeof(unsigned)) != hipSuccess ||
         hipMemset(ctx->tickets, 0, kTicketSlots * sizeof(unsigned)) != hipSuccess) {
+      delete ctx;
+      return HTPOPS_ERR_HIP;
+    }
+    // each GPU holds its own copy of the scratch array at its own address: ask for this device's, once, here
+    if (hipGetSymbolAddress(&ctx->scratch_ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ctx->scratch_ptr) {
+      (void) hipGetLastError();
+      (void) hipFree(ctx->tickets);
+      (void) hipEventDestroy(ctx->ev_start);
+      (void) hipEventDestroy(ctx->ev_stop);
+      (void) hipStreamDestroy(ctx->stream);
       delete ctx;
       return HTPOPS_ERR_HIP;
     }
@@ -1567,6 +1611,17 @@ extern "C" int htpops_flash_attn_ptr(htpops_context *ctx, void *o, const void *q
   }
   Lock lock(ctx->mu);
   return op_flash_attn(ctx, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, head_dim, qo_is_f32, causal);
+}
+
+extern "C" int htpops_flash_attn_noalloc_ptr(htpops_context *ctx, void *o, const void *q, const void *k, const void *v,
+                                             const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads,
+                                             int head_dim, int qo_is_f32, int causal) {
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  Lock lock(ctx->mu);
+  return op_flash_attn(ctx, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, head_dim, qo_is_f32, causal,
+                       /*no_alloc=*/true);
 }
 
 // ------------------------------------------------------------------------------------------------ measurement

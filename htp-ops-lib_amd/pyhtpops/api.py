@@ -54,7 +54,7 @@ EXPORTED_SYMBOLS = [
     "htpops_record_message", "htpops_launch_recorded_message", "htpops_release_recorded_message", "htpops_create_channel", "htpops_destroy_channel", "htpops_rms_norm_f32",
     "htpops_mat_mul_permuted_w16a32", "htpops_rms_norm_f32_ex_ptr", "htpops_quantize_q8_0_ptr",
     "htpops_rms_norm_quantize_q8_0_ptr", "htpops_mat_mul_q8_0_act_ptr", "htpops_mat_mul_f32_act_ptr",
-    "htpops_flash_attn_ptr", "htpops_timer_start", "htpops_timer_stop", "htpops_timer_elapsed_ms",
+    "htpops_flash_attn_ptr", "htpops_flash_attn_noalloc_ptr", "htpops_timer_start", "htpops_timer_stop", "htpops_timer_elapsed_ms",
     "htpops_measure_mfma_peak", "htpops_measure_copy_bandwidth",
 ]
 
@@ -103,6 +103,7 @@ def load_library(path=None):
         "htpops_mat_mul_q8_0_act_ptr": (ci, [vp, vp, vp, vp, ci, ci, ci, ci]),
         "htpops_mat_mul_f32_act_ptr": (ci, [vp, vp, vp, vp, ci, ci, ci, ci]),
         "htpops_flash_attn_ptr": (ci, [vp] * 6 + [ci] * 7),
+        "htpops_flash_attn_noalloc_ptr": (ci, [vp] * 6 + [ci] * 7),
         "htpops_timer_start": (ci, [vp]),
         "htpops_timer_stop": (ci, [vp]),
         "htpops_timer_elapsed_ms": (ci, [vp, ctypes.POINTER(ctypes.c_float)]),

@@ -179,6 +179,18 @@ int htpops_flash_attn_ptr(htpops_context *ctx, void *o, const void *q, const voi
                           const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
                           int qo_is_f32, int causal);
 
+/* htpops_flash_attn_ptr for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. Same arguments, same kernels, same
+ * results bit for bit; the split-KV partials of decode attention (qo_len == 1) go to a static 8 MiB device array
+ * inside the library instead of the context's grown-on-demand workspace, and the call performs no hipMalloc / hipFree
+ * of any kind. Limit: n_heads * ceil(kv_len / 64) * (head_dim + 2) * 4 bytes <= 8 MiB (e.g. 32 heads of 128 up to
+ * kv_len 32256); larger requests, and outputs that overlap weights the context holds a converted copy of, return -1
+ * with a message. All contexts on one GPU share the array, and it keeps the last call's contents: calls that overlap
+ * in time on one GPU (two contexts, i.e. two streams) race; calls on one context are ordered by its stream. */
+int htpops_flash_attn_noalloc_ptr(htpops_context *ctx, void *o, const void *q, const void *k, const void *v,
+                                  const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
+                                  int qo_is_f32, int causal);
+
 /* ---- measurement helpers (bench harness; no counterpart in the reference) ---- */
 
 /* Records an event on the context's stream / returns elapsed milliseconds between the two most
