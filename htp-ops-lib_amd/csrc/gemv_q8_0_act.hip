@@ -21,8 +21,6 @@
 
 #include <stdlib.h>
 
-#include <type_traits>
-
 namespace htpops {
 
 namespace {
@@ -166,64 +164,89 @@ __device__ __forceinline__ float pair_dot(const uint32_t (&w)[17], const ActPair
   return t;
 }
 
-// ITERS > 0: every lane handles exactly ITERS pairs per row (pairs <= G * ITERS), all loads up front.
-template <int WT, int G, int ITERS, int R>
-__global__ __launch_bounds__(kThreads) void gemv_pairs_kernel(float *__restrict__ out,
-                                                              const uint32_t *__restrict__ act,
-                                                              const uint32_t *__restrict__ w, int n, int pairs) {
-  constexpr int PD    = Pair<WT>::kDwords;
-  constexpr int SLOTS = kWave / G;
-  const int     lane  = threadIdx.x & (kWave - 1);
-  const int     wave  = threadIdx.x / kWave;
-  const int     g     = lane % G;
-  const int     slot  = lane / G;
-  const int     row0  = (blockIdx.x * kWaves + wave) * (SLOTS * R);
-  if (row0 >= n) {
-    return;
-  }
-  const size_t row_dwords = (size_t) pairs * PD;
+// ---- activation pairs prepared once per workgroup ------------------------------------------------------------------
+// The decode kernel keeps the PREPARED form of the activation row in LDS as a table of kEntries words per pair, entry e
+// of pair p at tab[e * TS + p] (consecutive lanes read consecutive words: no bank conflicts): the masked dwords that
+// meet the weight dwords, the two scales as floats and, for Q4_0 weights, 8 x the two block sums. One thread prepares
+// one pair; every wave of the workgroup then reads operands from the table right where it uses them, so the sums and
+// masks are computed once per workgroup instead of once per wave and no wave holds a prepared pair in registers.
+template <int WT>
+struct Prepared;
+template <>
+struct Prepared<kQ4_0> {
+  static constexpr int kEntries = 22;  // lo[9], hi[9], d0, d1, off0, off1
+};
+template <>
+struct Prepared<kQ8_0> {
+  static constexpr int kEntries = 19;  // a[17] (scale bytes zeroed), d0, d1
+};
 
-  uint32_t wreg[R][ITERS][PD];
+template <int TS>
+__device__ __forceinline__ void store_prepared(uint32_t *tab, int p, const ActPair<kQ4_0> &ap) {
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int row = row0 + r * SLOTS + slot;
-#pragma unroll
-    for (int i = 0; i < ITERS; ++i) {
-      const int p = g + i * G;
-      if (row < n && p < pairs) {
-        load_dwords<PD>(wreg[r][i], w + (size_t) row * row_dwords + (size_t) p * PD);
-      } else {
-        zero_dwords<PD>(wreg[r][i]);  // zero scales: the pair contributes exactly 0
-      }
-    }
+  for (int i = 0; i < 9; ++i) {
+    tab[i * TS + p]       = ap.lo[i];
+    tab[(9 + i) * TS + p] = ap.hi[i];
   }
+  tab[18 * TS + p] = __float_as_uint(ap.d0);
+  tab[19 * TS + p] = __float_as_uint(ap.d1);
+  tab[20 * TS + p] = (uint32_t) ap.off0;
+  tab[21 * TS + p] = (uint32_t) ap.off1;
+}
 
-  ActPair<WT> ap[ITERS];
+template <int TS>
+__device__ __forceinline__ void store_prepared(uint32_t *tab, int p, const ActPair<kQ8_0> &ap) {
+  tab[p] = ap.a[0] & 0xffff0000u;
 #pragma unroll
-  for (int i = 0; i < ITERS; ++i) {
-    const int p = g + i * G;
-    uint32_t  a[kActPairDwords];
-    if (p < pairs) {
-      load_dwords<kActPairDwords>(a, act + (size_t) p * kActPairDwords);
-    } else {
-      zero_dwords<kActPairDwords>(a);
-    }
-    prepare(ap[i], a);
+  for (int i = 1; i < 8; ++i) {
+    tab[i * TS + p] = ap.a[i];
   }
+  tab[8 * TS + p] = ap.a[8] & 0x0000ffffu;
+#pragma unroll
+  for (int i = 9; i < 17; ++i) {
+    tab[i * TS + p] = ap.a[i];
+  }
+  tab[17 * TS + p] = __float_as_uint(ap.d0);
+  tab[18 * TS + p] = __float_as_uint(ap.d1);
+}
 
+// the same arithmetic as pair_dot, operands from the table
+template <int TS>
+__device__ __forceinline__ float pair_dot_prepared(const uint32_t (&w)[9], const uint32_t *tab, int p, Prepared<kQ4_0>) {
+  int s0 = -(int) tab[20 * TS + p], s1 = -(int) tab[21 * TS + p];
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    float acc = 0.0f;
-#pragma unroll
-    for (int i = 0; i < ITERS; ++i) {
-      acc += pair_dot(wreg[r][i], ap[i]);
-    }
-    acc           = group_sum<G>(acc);
-    const int row = row0 + r * SLOTS + slot;
-    if (g == 0 && row < n) {
-      out[row] = acc;
-    }
+  for (int i = 0; i < 5; ++i) {
+    s0 = dot4_i8(w[i] & 0x0f0f0f0fu, tab[i * TS + p], s0);
+    s0 = dot4_i8((w[i] >> 4) & 0x0f0f0f0fu, tab[(9 + i) * TS + p], s0);
   }
+#pragma unroll
+  for (int i = 5; i < 9; ++i) {
+    s1 = dot4_i8(w[i] & 0x0f0f0f0fu, tab[i * TS + p], s1);
+    s1 = dot4_i8((w[i] >> 4) & 0x0f0f0f0fu, tab[(9 + i) * TS + p], s1);
+  }
+  const float dw0 = half_bits_to_float(w[0]);
+  const float dw1 = half_bits_to_float(w[4] >> 16);
+  float       t   = ((float) s0 * dw0) * __uint_as_float(tab[18 * TS + p]);
+  t += ((float) s1 * dw1) * __uint_as_float(tab[19 * TS + p]);
+  return t;
+}
+
+template <int TS>
+__device__ __forceinline__ float pair_dot_prepared(const uint32_t (&w)[17], const uint32_t *tab, int p, Prepared<kQ8_0>) {
+  int s0 = 0, s1 = 0;
+#pragma unroll
+  for (int i = 0; i < 9; ++i) {
+    s0 = dot4_i8(w[i], tab[i * TS + p], s0);
+  }
+#pragma unroll
+  for (int i = 9; i < 17; ++i) {
+    s1 = dot4_i8(w[i], tab[i * TS + p], s1);
+  }
+  const float dw0 = half_bits_to_float(w[0]);
+  const float dw1 = half_bits_to_float(w[8] >> 16);
+  float       t   = ((float) s0 * dw0) * __uint_as_float(tab[17 * TS + p]);
+  t += ((float) s1 * dw1) * __uint_as_float(tab[18 * TS + p]);
+  return t;
 }
 
 // Any number of pairs per row: lanes loop over the row, activations are re-read (L2) for every row set.
@@ -291,55 +314,78 @@ __device__ __forceinline__ float group_sum_dpp(float v) {
   return v;
 }
 
-// ---- shared-activation variant --------------------------------------------------------------------------------
-// Same arithmetic and lane mapping as gemv_pairs_kernel, but the activation row is staged in LDS once per
-// workgroup instead of being fetched by every wave: the texture path then carries (almost) only weight bytes.
-// Weight loads are issued first, the cooperative activation copy second, so the weights are in flight while the
-// workgroup synchronises. Partial sums are reduced with DPP row operations instead of LDS permutes.
+// ---- the decode kernel -------------------------------------------------------------------------------------------
+// The activation row is staged in LDS once per workgroup instead of being fetched by every wave: the texture path then
+// carries (almost) only weight bytes. Weight loads are issued right behind the activation loads, so the weights are in
+// flight while the workgroup synchronises. Partial sums are reduced with DPP row operations instead of LDS permutes.
 //
-// One launch can serve several weight matrices that share the activation row (the q/k/v or gate/up projections of a
-// decoder layer): blockIdx.y picks the member, whose weight pointer, output pointer and row count come from the
-// argument table.
-struct GemvGroupArgs {
-  const uint32_t *w[kGemvGroupMax];
-  float          *out[kGemvGroupMax];
-  int             n[kGemvGroupMax];
+// One launch serves up to kGemvGroupMax matrix-vector products ("members"), each with its own weight matrix, output,
+// row count, row length and ACTIVATION ROW: a workgroup finds its member from a table of first-workgroup indices
+// (blockIdx.x is one-dimensional over all members) and then runs the row-set body compiled for that member's row
+// length. The caller guarantees that no member reads what another member writes; members that share an activation
+// row (q/k/v, gate/up of a decoder layer) are simply members with equal `act`.
+struct GemvMember {
+  const uint32_t *w;
+  const uint32_t *act;
+  float          *out;
+  int             n;       // weight rows
+  int             pairs;   // block pairs per row (k / 64)
+  int             block0;  // first workgroup of this member
+  int             shape;   // kShape* below: lanes per row and pairs per lane
+  int             r;       // row sets per wave (1 or 2)
 };
 
-template <int WT, int G, int ITERS, int R, int THREADS>
-__global__ __launch_bounds__(THREADS) void gemv_shared_act_kernel(GemvGroupArgs grp, const uint32_t *__restrict__ act,
-                                                                  int pairs) {
-  extern __shared__ __attribute__((aligned(16))) uint32_t act_lds[];
-  constexpr int PD    = Pair<WT>::kDwords;
-  constexpr int SLOTS = kWave / G;
-  constexpr int WAVES = THREADS / kWave;
-  const int                       n   = grp.n[blockIdx.y];
-  float *__restrict__             out = grp.out[blockIdx.y];
-  const uint32_t *__restrict__    w   = grp.w[blockIdx.y];
-  if ((int) (blockIdx.x * (WAVES * SLOTS * R)) >= n) {
-    return;  // whole workgroup: this member has fewer rows than the widest one
-  }
-  const int     lane  = threadIdx.x & (kWave - 1);
-  const int     wave  = threadIdx.x / kWave;
-  const int     g     = lane % G;
-  const int     slot  = lane / G;
-  const int     row0  = (blockIdx.x * WAVES + wave) * (SLOTS * R);
-  const size_t  row_dwords = (size_t) pairs * PD;
+struct GemvMembers {
+  GemvMember m[kGemvGroupMax];
+  int        count;
+};
 
-  // The activation row is requested FIRST and the weights right behind it: loads retire in order, so the (L2
-  // resident, quickly served) activations never wait behind the HBM stream, while the weights are already in
-  // flight during the workgroup's LDS exchange. A row is at most 192 pairs = 13056 bytes: ACT_SLOTS 16-byte
-  // pieces per thread cover it; pieces at or across the end of the row are slid back to end - 16.
-  constexpr int ACT_SLOTS = (192 * kActPairDwords * 4 + THREADS * 16 - 1) / (THREADS * 16);
-  const int     act_bytes = pairs * kActPairDwords * 4;
-  uint4         areg[ACT_SLOTS];
-  int           aoff[ACT_SLOTS];
-#pragma unroll
-  for (int j = 0; j < ACT_SLOTS; ++j) {
-    const int off = (threadIdx.x + j * THREADS) * 16;
-    aoff[j]       = min(off, act_bytes - 16);
-    const u32x4_a4 v = *reinterpret_cast<const u32x4_a4 *>(reinterpret_cast<const uint8_t *>(act) + aoff[j]);
-    areg[j]       = make_uint4(v.x, v.y, v.z, v.w);
+// lanes per row x pairs per lane x waves per row
+enum { kShapeG16 = 0, kShapeG32 = 1, kShapeG64 = 2, kShapeG64x2 = 3, kShapeG64x2S2 = 4 };
+
+constexpr int kSharedActMaxPairs = 192;  // longest activation row the kernel stages (k = 12288)
+constexpr int kRedDwords         = 16;   // LDS words in front of the staged row: partial sums of rows split over waves
+
+// One workgroup of WAVES waves. SEG = 1: wave `wave` computes rows row0 .. row0 + SLOTS * R - 1, SLOTS = 64 / G rows at
+// a time. SEG = 2 (G = 64, R = 1): a row is split into two halves taken by two neighbouring waves, whose partial sums
+// meet in LDS and are added in a fixed order (first half + second half) -- measured on MI355X, a wave that requests
+// more than about 4.6 KB of the stream at once (three pairs per lane, the k = 11008 rows on one wave) streams 10-25 %
+// slower than two waves with half of it each.
+template <int WT, int G, int ITERS, int R, int SEG, int WAVES>
+__device__ __forceinline__ void gemv_row_sets(const GemvMember &mem, int wg, uint32_t *lds) {
+  static_assert(SEG == 1 || (G == kWave && R == 1 && WAVES % SEG == 0), "split rows: one row per wave pair");
+  constexpr int PD      = Pair<WT>::kDwords;
+  constexpr int SLOTS   = kWave / G;
+  constexpr int THREADS = WAVES * kWave;
+  constexpr int TS      = G * ITERS * SEG < kSharedActMaxPairs ? G * ITERS * SEG : kSharedActMaxPairs;  // pairs in the table
+  static_assert(TS <= THREADS, "one thread prepares one activation pair");
+  uint32_t *tab = lds + kRedDwords;
+  const int                    n     = mem.n;
+  const int                    pairs = mem.pairs;
+  float *__restrict__          out   = mem.out;
+  const uint32_t *__restrict__ w     = mem.w;
+  const uint32_t *__restrict__ act   = mem.act;
+  const int    lane = threadIdx.x & (kWave - 1);
+  const int    wave = threadIdx.x / kWave;
+  const int    g    = lane % G;
+  const int    slot = lane / G;
+  const int    seg  = SEG == 1 ? 0 : wave % SEG;
+  const int    row0 = SEG == 1 ? (wg * WAVES + wave) * (SLOTS * R) : wg * (WAVES / SEG) + wave / SEG;
+  const int    seg_pairs = SEG == 1 ? pairs : (pairs + SEG - 1) / SEG;
+  const int    p_begin   = seg * seg_pairs;
+  const int    p_end     = min(pairs, p_begin + seg_pairs);  // may be <= p_begin for a very short row: no live pair
+  const size_t row_dwords = (size_t) pairs * PD;
+
+  // The activation pair this thread prepares is requested FIRST and the weights right behind it: loads retire in
+  // order, so the (L2 resident, quickly served) activations never wait behind the HBM stream, while the weights are
+  // already in flight during the workgroup's LDS exchange. Only waves that have a pair to prepare issue these loads
+  // (a wave-uniform branch): measured, the address processing of five more load instructions in every wave costs
+  // about 4 % of a decoder layer's stream. Threads beyond the row inside such a wave re-read its last pair.
+  uint32_t   araw[kActPairDwords];
+  const bool stager = wave * kWave < pairs;
+  if (stager) {
+    const int my_pair = min((int) threadIdx.x, pairs - 1);
+    load_dwords<kActPairDwords>(araw, act + (size_t) my_pair * kActPairDwords);
   }
 
   // Branch-free weight loads (so that the compiler can count them and wait per use): lanes without work read a
@@ -350,37 +396,21 @@ __global__ __launch_bounds__(THREADS) void gemv_shared_act_kernel(GemvGroupArgs 
     const int row = min(row0 + r * SLOTS + slot, n - 1);
 #pragma unroll
     for (int i = 0; i < ITERS; ++i) {
-      const int p = min(g + i * G, pairs - 1);
+      const int p = min(p_begin + g + i * G, pairs - 1);
       load_dwords<PD>(wreg[r][i], w + (size_t) row * row_dwords + (size_t) p * PD);
     }
   }
 
-  // every thread stores its pieces, without a branch: pieces clamped to the end of the row rewrite the same
-  // bytes with the same values, which is harmless and keeps the loads above where they were issued
-#pragma unroll
-  for (int j = 0; j < ACT_SLOTS; ++j) {
-    uint32_t *dst = act_lds + aoff[j] / 4;  // only dword aligned when the piece was slid back
-    dst[0] = areg[j].x, dst[1] = areg[j].y, dst[2] = areg[j].z, dst[3] = areg[j].w;
+  if (stager) {
+    ActPair<WT> ap;
+    prepare(ap, araw);
+    if ((int) threadIdx.x < pairs) {
+      store_prepared<TS>(tab, (int) threadIdx.x, ap);
+    }
   }
   __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the LDS writes have landed; vmcnt is left alone
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
-
-  ActPair<WT> ap[ITERS];
-#pragma unroll
-  for (int i = 0; i < ITERS; ++i) {
-    const int p = g + i * G;
-    uint32_t  a[kActPairDwords];
-    if (p < pairs) {
-#pragma unroll
-      for (int e = 0; e < kActPairDwords; ++e) {
-        a[e] = act_lds[p * kActPairDwords + e];
-      }
-    } else {
-      zero_dwords<kActPairDwords>(a);
-    }
-    prepare(ap[i], a);
-  }
 
 #pragma unroll
   for (int r = 0; r < R; ++r) {
@@ -388,49 +418,158 @@ __global__ __launch_bounds__(THREADS) void gemv_shared_act_kernel(GemvGroupArgs 
     float     acc = 0.0f;
 #pragma unroll
     for (int i = 0; i < ITERS; ++i) {
-      const bool live = row < n && g + i * G < pairs;
+      const int  p    = p_begin + g + i * G;
+      const bool live = row < n && p < p_end;
       constexpr int kScale1 = WT == kQ4_0 ? 4 : 8;  // dword holding the second block's scale (upper half)
       wreg[r][i][0]         = live ? wreg[r][i][0] : 0u;
       wreg[r][i][kScale1]   = live ? wreg[r][i][kScale1] : 0u;
-      acc += pair_dot(wreg[r][i], ap[i]);
+      acc += pair_dot_prepared<TS>(wreg[r][i], tab, min(p, pairs - 1), Prepared<WT>());
     }
     acc = group_sum_dpp<G>(acc);
-    if (g == G - 1 && row < n) {
-      out[row] = acc;
+    if (SEG == 1) {
+      if (g == G - 1 && row < n) {
+        out[row] = acc;
+      }
+    } else {
+      float *red = reinterpret_cast<float *>(lds);
+      if (lane == kWave - 1) {
+        red[wave] = acc;
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      if (lane == kWave - 1 && seg == 0 && row < n) {
+        float total = acc;
+#pragma unroll
+        for (int sg = 1; sg < SEG; ++sg) {
+          total += red[wave + sg];
+        }
+        out[row] = total;
+      }
     }
   }
 }
 
-template <int WT, int G, int ITERS, int R, int THREADS>
-hipError_t launch_shared_act_instance(hipStream_t stream, const GemvGroupArgs &grp, int count, const uint32_t *act,
-                                      int pairs) {
-  constexpr int rows_per_group = (THREADS / kWave) * (kWave / G) * R;
-  int           n_max          = 0;
-  for (int i = 0; i < count; ++i) {
-    n_max = grp.n[i] > n_max ? grp.n[i] : n_max;
+// LONG = false: every member has at most 64 pairs per row (k <= 4096); the kernel then holds only the one-pair bodies
+// and keeps their small register footprint. LONG = true adds the bodies for longer rows.
+// The first workgroup of members 1..7 travels as plain leading arguments (INT_MAX for members that do not exist), the
+// first words of the argument block: a wave knows its member after one scalar load and fetches that member's record with
+// a second one, instead of walking the table in memory.
+template <int WT, bool LONG, int THREADS>
+__global__ __launch_bounds__(THREADS) void gemv_members_kernel(int b1, int b2, int b3, int b4, int b5, int b6, int b7,
+                                                               GemvMembers grp) {
+  static_assert(kGemvGroupMax == 8, "one leading argument per member after the first");
+  extern __shared__ __attribute__((aligned(16))) uint32_t gemv_lds[];
+  constexpr int W   = THREADS / kWave;
+  const int     bid = (int) blockIdx.x;
+  const int     mi  = bid >= b7 ? 7 : bid >= b6 ? 6 : bid >= b5 ? 5 : bid >= b4 ? 4 : bid >= b3 ? 3 : bid >= b2 ? 2 : bid >= b1 ? 1 : 0;
+  const GemvMember &mem = grp.m[mi];
+  const int         wg  = (int) blockIdx.x - mem.block0;
+  const int         sel = mem.shape * 2 + (mem.r - 1);
+  switch (sel) {
+    case kShapeG16 * 2 + 0: gemv_row_sets<WT, 16, 1, 1, 1, W>(mem, wg, gemv_lds); break;
+    case kShapeG16 * 2 + 1: gemv_row_sets<WT, 16, 1, 2, 1, W>(mem, wg, gemv_lds); break;
+    case kShapeG32 * 2 + 0: gemv_row_sets<WT, 32, 1, 1, 1, W>(mem, wg, gemv_lds); break;
+    case kShapeG32 * 2 + 1: gemv_row_sets<WT, 32, 1, 2, 1, W>(mem, wg, gemv_lds); break;
+    case kShapeG64 * 2 + 0: gemv_row_sets<WT, 64, 1, 1, 1, W>(mem, wg, gemv_lds); break;
+    case kShapeG64 * 2 + 1: gemv_row_sets<WT, 64, 1, 2, 1, W>(mem, wg, gemv_lds); break;
+    default:
+      if (LONG) {
+        switch (sel) {
+          case kShapeG64x2 * 2 + 0: gemv_row_sets<WT, 64, 2, 1, 1, W>(mem, wg, gemv_lds); break;
+          case kShapeG64x2S2 * 2 + 0: gemv_row_sets<WT, 64, 2, 1, 2, W>(mem, wg, gemv_lds); break;
+          default: break;
+        }
+      }
+      break;
   }
-  const dim3 grid((unsigned) ((n_max + rows_per_group - 1) / rows_per_group), (unsigned) count);
-  hipLaunchKernelGGL((gemv_shared_act_kernel<WT, G, ITERS, R, THREADS>), grid, dim3(THREADS),
-                     (size_t) pairs * kActPairDwords * 4, stream, grp, act, pairs);
+}
+
+// Fills shape, r and block0 of every member and launches.
+template <int WT>
+hipError_t launch_gemv_members(hipStream_t stream, GemvMembers &grp) {
+  static const int forced_r       = env_int("HTPOPS_GEMV_ROWS", 0);
+  static const int forced_threads = env_int("HTPOPS_GEMV_THREADS", 0);
+  // measured on MI355X: short-lived waves (one row set each) stream best; only very wide launches of short rows
+  // (gate + up of a 7B layer: 22016 rows of 64 pairs) gain from two rows per lane group
+  long total_short_rows = 0;
+  for (int i = 0; i < grp.count; ++i) {
+    if (grp.m[i].pairs <= 64) {
+      total_short_rows += grp.m[i].n;
+    }
+  }
+  // Workgroups of 512 threads stage the activation row half as often per weight byte (measured on a 7B layer's seven
+  // projections in one launch: 20.3 us against 20.9 us); launches too small to give every compute unit a few of them
+  // keep 256 threads.
+  auto place = [&](int threads, bool commit) {
+    const int waves  = threads / kWave;
+    int       blocks = 0;
+    for (int i = 0; i < grp.count; ++i) {
+      GemvMember &mem            = grp.m[i];
+      const int   lanes_per_row  = mem.shape == kShapeG16 ? 16 : mem.shape == kShapeG32 ? 32 : 64;
+      const int   rows_per_group = mem.shape == kShapeG64x2S2 ? waves / 2 : waves * (kWave / lanes_per_row) * mem.r;
+      if (commit) {
+        mem.block0 = blocks;
+      }
+      blocks += (mem.n + rows_per_group - 1) / rows_per_group;
+    }
+    return blocks;
+  };
+  int  max_pairs = 0;
+  bool any_long  = false;
+  for (int i = 0; i < grp.count; ++i) {
+    GemvMember &mem = grp.m[i];
+    const int   p   = mem.pairs;
+    if (p < 1 || p > kSharedActMaxPairs || mem.n < 1) {
+      return hipErrorNotSupported;
+    }
+    mem.shape = p <= 16 ? kShapeG16 : p <= 32 ? kShapeG32 : p <= 64 ? kShapeG64 : p <= 128 ? kShapeG64x2 : kShapeG64x2S2;
+    mem.r     = (p <= 64 && total_short_rows >= 16384) ? 2 : 1;
+    if (forced_r == 1 || forced_r == 2) {
+      mem.r = forced_r;
+    }
+    if (p > 64) {
+      mem.r = 1;
+    }
+    max_pairs = p > max_pairs ? p : max_pairs;
+    any_long  = any_long || p > 64;
+  }
+  int threads = place(512, false) >= 1024 ? 512 : kThreads;
+  if (forced_threads == 256 || forced_threads == 512) {
+    threads = forced_threads;
+  }
+  const int blocks = place(threads, true);
+  // the table stride of the widest body among the members (see TS in gemv_row_sets)
+  const int    table_pairs = max_pairs <= 16 ? 16 : max_pairs <= 32 ? 32 : max_pairs <= 64 ? 64 : max_pairs <= 128 ? 128 : kSharedActMaxPairs;
+  const size_t lds = (size_t) (kRedDwords + table_pairs * Prepared<WT>::kEntries) * 4;
+  const dim3   grid((unsigned) blocks);
+  int b[kGemvGroupMax];
+  for (int i = 1; i < kGemvGroupMax; ++i) {
+    b[i] = i < grp.count ? grp.m[i].block0 : 0x7fffffff;
+  }
+#define HTPOPS_GEMV_LAUNCH(LONG, T) \
+  hipLaunchKernelGGL((gemv_members_kernel<WT, LONG, T>), grid, dim3(T), lds, stream, b[1], b[2], b[3], b[4], b[5], b[6], b[7], grp)
+  if (threads == 512) {
+    if (any_long) {
+      HTPOPS_GEMV_LAUNCH(true, 512);
+    } else {
+      HTPOPS_GEMV_LAUNCH(false, 512);
+    }
+  } else if (any_long) {
+    HTPOPS_GEMV_LAUNCH(true, kThreads);
+  } else {
+    HTPOPS_GEMV_LAUNCH(false, kThreads);
+  }
+#undef HTPOPS_GEMV_LAUNCH
   return hipGetLastError();
 }
 
-template <int WT, int G, int ITERS>
-hipError_t launch_shared_act(hipStream_t stream, const GemvGroupArgs &grp, int count, const uint32_t *act, int pairs,
-                             int r, int threads) {
-#define HTPOPS_CASE(R, T)                                                                         \
-  if (r == R && threads == T) {                                                                   \
-    return launch_shared_act_instance<WT, G, ITERS, R, T>(stream, grp, count, act, pairs);       \
-  }
-  HTPOPS_CASE(1, 256)
-  HTPOPS_CASE(2, 256)
-  HTPOPS_CASE(1, 512)
-  HTPOPS_CASE(2, 512)
-  HTPOPS_CASE(4, 256)
-  HTPOPS_CASE(1, 1024)
-#undef HTPOPS_CASE
-  return hipErrorInvalidValue;
-}
+// the argument table of the two-to-four-row kernel below: members share the activation rows, blockIdx.y picks one
+struct GemvGroupArgs {
+  const uint32_t *w[kGemvGroupMax];
+  float          *out[kGemvGroupMax];
+  int             n[kGemvGroupMax];
+};
 
 // ---- two to four activation rows ------------------------------------------------------------------------------------
 // The same stream over the weights with M activation rows staged in LDS: a lane prepares its activation pairs of all M
@@ -561,65 +700,6 @@ __global__ __launch_bounds__(kThreads) void gemv_blocks_generic_kernel(float *__
 }
 
 template <int WT, int G, int ITERS>
-hipError_t launch_pairs(hipStream_t stream, float *out, const uint32_t *act, const uint32_t *w, int n, int pairs,
-                        int rows_per_slot) {
-  constexpr int SLOTS = kWave / G;
-  auto          grid  = [&](int r) { return dim3((unsigned) ((n + kWaves * SLOTS * r - 1) / (kWaves * SLOTS * r))); };
-  switch (rows_per_slot) {
-    case 1:
-      hipLaunchKernelGGL((gemv_pairs_kernel<WT, G, ITERS, 1>), grid(1), dim3(kThreads), 0, stream, out, act, w, n, pairs);
-      break;
-    case 2:
-      hipLaunchKernelGGL((gemv_pairs_kernel<WT, G, ITERS, 2>), grid(2), dim3(kThreads), 0, stream, out, act, w, n, pairs);
-      break;
-    default:
-      hipLaunchKernelGGL((gemv_pairs_kernel<WT, G, ITERS, 4>), grid(4), dim3(kThreads), 0, stream, out, act, w, n, pairs);
-      break;
-  }
-  return hipGetLastError();
-}
-
-constexpr int kSharedActMaxPairs = 192;  // longest activation row the shared-activation kernel stages (k = 12288)
-
-bool shared_act_enabled() {
-  static const int use_shared = env_int("HTPOPS_GEMV_SHARED", 1);
-  return use_shared != 0;
-}
-
-// the default kernel for `count` weight matrices that share one activation row of `pairs` <= kSharedActMaxPairs
-template <int WT>
-hipError_t launch_gemv_shared(hipStream_t stream, const GemvGroupArgs &grp, int count, const uint32_t *act, int pairs) {
-  static const int forced_r       = env_int("HTPOPS_GEMV_ROWS", 0);
-  static const int forced_threads = env_int("HTPOPS_GEMV_THREADS", 0);
-  // measured on MI355X: short-lived waves (one row set each) in 256-thread groups stream best; only very wide
-  // launches of short rows (gate + up of a 7B layer: 22016 rows of 64 pairs) gain from two rows per lane group
-  int total_rows = 0;
-  for (int i = 0; i < count; ++i) {
-    total_rows += grp.n[i];
-  }
-  int r = (pairs <= 64 && total_rows >= 16384) ? 2 : 1, threads = 256;
-  if (forced_r) {
-    r = forced_r;
-  }
-  if (forced_threads) {
-    threads = forced_threads;
-  }
-  if (pairs <= 16) {
-    return launch_shared_act<WT, 16, 1>(stream, grp, count, act, pairs, r, threads);
-  }
-  if (pairs <= 32) {
-    return launch_shared_act<WT, 32, 1>(stream, grp, count, act, pairs, r, threads);
-  }
-  if (pairs <= 64) {
-    return launch_shared_act<WT, 64, 1>(stream, grp, count, act, pairs, r, threads);
-  }
-  if (pairs <= 128) {
-    return launch_shared_act<WT, 64, 2>(stream, grp, count, act, pairs, r, threads);
-  }
-  return launch_shared_act<WT, 64, 3>(stream, grp, count, act, pairs, r, threads);
-}
-
-template <int WT, int G, int ITERS>
 hipError_t launch_rows_shared_act(hipStream_t stream, const GemvGroupArgs &grp, int count, const uint32_t *act, int pairs,
                                   int m) {
   constexpr int rows_per_group = kWaves * (kWave / G);
@@ -665,38 +745,11 @@ hipError_t launch_gemv_rows_shared(hipStream_t stream, const GemvGroupArgs &grp,
 
 template <int WT>
 hipError_t launch_gemv_row(hipStream_t stream, float *out, const uint32_t *act, const uint32_t *w, int n, int pairs) {
-  static const int forced_r = env_int("HTPOPS_GEMV_ROWS", 0);
-  constexpr int    PD       = Pair<WT>::kDwords;
-  if (shared_act_enabled() && pairs <= kSharedActMaxPairs) {
-    GemvGroupArgs grp = {};
-    grp.w[0] = w, grp.out[0] = out, grp.n[0] = n;
-    return launch_gemv_shared<WT>(stream, grp, 1, act, pairs);
-  }
-  // rows in flight per lane group: fewer for long rows (register budget), more for short ones
-  auto pick_r = [&](int regs_per_row, int slots) {
-    if (forced_r == 1 || forced_r == 2 || forced_r == 4) {
-      return forced_r;
-    }
-    int r = 4;
-    while (r > 1 && (regs_per_row * r > 72 || (long long) n / (slots * r) < 2048)) {
-      r >>= 1;
-    }
-    return r;
-  };
-  if (pairs <= 16) {
-    return launch_pairs<WT, 16, 1>(stream, out, act, w, n, pairs, pick_r(PD, 4));
-  }
-  if (pairs <= 32) {
-    return launch_pairs<WT, 32, 1>(stream, out, act, w, n, pairs, pick_r(PD, 2));
-  }
-  if (pairs <= 64) {
-    return launch_pairs<WT, 64, 1>(stream, out, act, w, n, pairs, pick_r(PD, 1));
-  }
-  if (pairs <= 128) {
-    return launch_pairs<WT, 64, 2>(stream, out, act, w, n, pairs, pick_r(2 * PD, 1));
-  }
-  if (pairs <= 192) {
-    return launch_pairs<WT, 64, 3>(stream, out, act, w, n, pairs, pick_r(3 * PD, 1));
+  if (pairs <= kSharedActMaxPairs) {
+    GemvMembers grp = {};
+    grp.count       = 1;
+    grp.m[0].w = w, grp.m[0].act = act, grp.m[0].out = out, grp.m[0].n = n, grp.m[0].pairs = pairs;
+    return launch_gemv_members<WT>(stream, grp);
   }
   hipLaunchKernelGGL((gemv_pairs_loop_kernel<WT, 2>), dim3((unsigned) ((n + kWaves * 2 - 1) / (kWaves * 2))),
                      dim3(kThreads), 0, stream, out, act, w, n, pairs);
@@ -734,29 +787,30 @@ hipError_t launch_gemv_q8_0_act(hipStream_t stream, float *out, const void *act,
   return hipSuccess;
 }
 
-hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *act,
-                                      const void *const *weights, const int *ns, int k, WeightType wt) {
-  const int nblk = k / kQK;
-  if (count < 1 || count > kGemvGroupMax || nblk % 2 != 0 || nblk / 2 > kSharedActMaxPairs || !shared_act_enabled() ||
-      (reinterpret_cast<uintptr_t>(act) & 3) != 0) {
+hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *const *acts,
+                                      const void *const *weights, const int *ns, const int *ks, WeightType wt) {
+  if (count < 1 || count > kGemvGroupMax) {
     return hipErrorNotSupported;
   }
-  GemvGroupArgs grp = {};
+  GemvMembers grp = {};
+  grp.count       = count;
   for (int i = 0; i < count; ++i) {
-    if ((reinterpret_cast<uintptr_t>(weights[i]) & 3) != 0) {
+    const int nblk = ks[i] / kQK;
+    if (ks[i] % (2 * kQK) != 0 || nblk / 2 > kSharedActMaxPairs ||
+        ((reinterpret_cast<uintptr_t>(weights[i]) | reinterpret_cast<uintptr_t>(acts[i])) & 3) != 0) {
       return hipErrorNotSupported;
     }
-    grp.w[i] = static_cast<const uint32_t *>(weights[i]), grp.out[i] = outs[i], grp.n[i] = ns[i];
+    grp.m[i].w = static_cast<const uint32_t *>(weights[i]), grp.m[i].act = static_cast<const uint32_t *>(acts[i]);
+    grp.m[i].out = outs[i], grp.m[i].n = ns[i], grp.m[i].pairs = nblk / 2;
   }
-  return wt == kQ4_0 ? launch_gemv_shared<kQ4_0>(stream, grp, count, static_cast<const uint32_t *>(act), nblk / 2) :
-                       launch_gemv_shared<kQ8_0>(stream, grp, count, static_cast<const uint32_t *>(act), nblk / 2);
+  return wt == kQ4_0 ? launch_gemv_members<kQ4_0>(stream, grp) : launch_gemv_members<kQ8_0>(stream, grp);
 }
 
 bool gemv_rows_fits(int m, int k, WeightType wt) {
   // measured on Llama-7B shapes: with Q8_0 weights the kernel beats the K-sliced one up to 4 rows; with Q4_0 weights
   // (whose activation pairs cost a sum of their bytes each) it beats the repacked-weight kernel at 2 rows only
   const int nblk = k / kQK;
-  return m >= 2 && m <= (wt == kQ4_0 ? 2 : 4) && k % (2 * kQK) == 0 && nblk / 2 <= kSharedActMaxPairs && shared_act_enabled() &&
+  return m >= 2 && m <= (wt == kQ4_0 ? 2 : 4) && k % (2 * kQK) == 0 && nblk / 2 <= kSharedActMaxPairs &&
          env_int("HTPOPS_GEMV_ROWS_KERNEL", 1) != 0;
 }
 

@@ -89,6 +89,8 @@ struct htpops_context {
     int         m = 0, k = 0;
   } act_fragments;
   bool in_message = false;
+  // how many separately launched units (grouped launches and single ops) the most recent message walk issued
+  int  message_submissions = 0;
 
   // Recorded messages hold device addresses. Each keeps the buffer ranges its requests resolved to (collected through
   // `collect_ranges` while it is recorded) and is marked stale when one of them is released, when a converted copy of
@@ -1108,34 +1110,43 @@ extern "C" int htpops_execute_op(htpops_context *ctx, const struct OpComputeRequ
 
 namespace {
 
-// Consecutive matmul requests of a message with 1 to 8 activation rows that read the SAME activation buffer (q/k/v or
-// gate/up of a decoder layer) are collected and run as one kernel launch: the result of every request is what its own launch would have
-// produced (same kernel, same arithmetic), the requests just stop paying a launch and a ramp-up each. A request
-// joins the open batch only if its output cannot feed or clobber anything the batch reads or writes.
+// Consecutive matmul requests of a message are collected and run as one kernel launch when that cannot change any
+// result: the result of every request is what its own launch would have produced (same kernel, same arithmetic), the
+// requests just stop paying a launch and a ramp-up each. The reference runs requests strictly in order
+// (src/dsp/commu.c:91-114); a request therefore joins the open batch only if it neither reads (activations, weights)
+// nor overwrites anything an earlier member of the batch writes, and writes nothing an earlier member reads.
+//  * one activation row (decode): members may read different activation buffers and have different k -- a whole
+//    hazard-free run of matrix-vector products (the seven projections of a layer whose inputs are all ready) is one
+//    launch; where a real data dependency exists (o after attention after q/k/v) the run is split there;
+//  * 2..16 rows: members must read the SAME activation rows (q/k/v or gate/up), which the few-row kernels stage once.
 struct GemvBatch {
-  int                   wt = 0, k = 0, m = 0, count = 0;
-  const void           *act = nullptr;
+  int                   wt = 0, m = 0, count = 0;
   struct RequestHeader *hdr[htpops::kGemvGroupMax];
   float                *out[htpops::kGemvGroupMax];
   const void           *w[htpops::kGemvGroupMax];
+  const void           *act[htpops::kGemvGroupMax];
   int                   n[htpops::kGemvGroupMax];
+  int                   k[htpops::kGemvGroupMax];
 };
 
 void flush_batch(htpops_context *ctx, GemvBatch &b) {
   if (b.count == 0) {
     return;
   }
+  ++ctx->message_submissions;
   int ret = HTPOPS_OK;
   if (b.count > 1) {
     for (int i = 0; i < b.count; ++i) {
       note_device_write(ctx, b.out[i], (size_t) b.m * b.n[i] * 4);
     }
+    const int        k0 = b.k[0];
+    const void      *a0 = b.act[0];
     hipError_t e;
     if (b.m == 1) {
       e = htpops::launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k, (htpops::WeightType) b.wt);
-    } else if (htpops::gemv_rows_fits(b.m, b.k, (htpops::WeightType) b.wt)) {
+    } else if (htpops::gemv_rows_fits(b.m, k0, (htpops::WeightType) b.wt)) {
       // 2..4 rows: the decode kernel's weight stream with the rows staged in LDS, whatever n and the weight type
-      e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.m, b.k,
+      e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, b.count, b.out, a0, b.w, b.n, b.m, k0,
                                                   (htpops::WeightType) b.wt);
     } else {
       // Members whose weights have (or get) a repacked copy go to the kernel that streams it, the others to the
@@ -1146,7 +1157,7 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
       int         n_a[htpops::kGemvGroupMax], n_b[htpops::kGemvGroupMax], count_a = 0, count_b = 0;
       for (int i = 0; i < b.count; ++i) {
         const void *lw = nullptr;
-        if (int r = lane_order_weights(ctx, b.w[i], b.act, b.m, b.k, b.n[i], b.wt, &lw)) {
+        if (int r = lane_order_weights(ctx, b.w[i], a0, b.m, k0, b.n[i], b.wt, &lw)) {
           b.hdr[i]->state = r;
         } else if (lw) {
           out_a[count_a] = b.out[i], w_a[count_a] = lw, n_a[count_a++] = b.n[i];
@@ -1154,20 +1165,20 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
           out_b[count_b] = b.out[i], w_b[count_b] = b.w[i], n_b[count_b++] = b.n[i];
         } else {
           // more rows than the K-sliced group launch takes: on its own
-          b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act, b.w[i], b.m, b.k, b.n[i], b.wt);
+          b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], a0, b.w[i], b.m, k0, b.n[i], b.wt);
         }
       }
       e = hipSuccess;
       if (count_a > 0) {
-        e = htpops::launch_matmul_lane_order_group(ctx->stream, count_a, out_a, b.act, w_a, n_a, b.m, b.k,
+        e = htpops::launch_matmul_lane_order_group(ctx->stream, count_a, out_a, a0, w_a, n_a, b.m, k0,
                                                    (htpops::WeightType) b.wt);
       }
       if (e == hipSuccess && count_b > 0) {
-        const size_t ws = htpops::matmul_skinny_group_workspace_bytes(count_b, n_b, b.m, b.k);
+        const size_t ws = htpops::matmul_skinny_group_workspace_bytes(count_b, n_b, b.m, k0);
         if (int r = ensure_workspace(ctx, ws)) {
           ret = r;
         } else {
-          e = htpops::launch_matmul_skinny_group(ctx->stream, count_b, out_b, b.act, w_b, n_b, b.m, b.k,
+          e = htpops::launch_matmul_skinny_group(ctx->stream, count_b, out_b, a0, w_b, n_b, b.m, k0,
                                                  (htpops::WeightType) b.wt, ctx->workspace, ctx->tickets, kTicketSlots);
         }
       }
@@ -1175,13 +1186,13 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
     if (e == hipErrorNotSupported) {
       (void) hipGetLastError();
       for (int i = 0; i < b.count; ++i) {
-        b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act, b.w[i], b.m, b.k, b.n[i], b.wt);
+        b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act[i], b.w[i], b.m, b.k[i], b.n[i], b.wt);
       }
     } else if (e != hipSuccess) {
       ret = fail(ctx, HTPOPS_ERR_HIP, "grouped mat_mul launch: %s", hipGetErrorString(e));
     }
   } else {
-    ret = op_mat_mul_q8(ctx, b.out[0], b.act, b.w[0], b.m, b.k, b.n[0], b.wt);
+    ret = op_mat_mul_q8(ctx, b.out[0], b.act[0], b.w[0], b.m, b.k[0], b.n[0], b.wt);
   }
   if (ret != HTPOPS_OK) {
     for (int i = 0; i < b.count; ++i) {
@@ -1212,17 +1223,22 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
       ranges_overlap(out, out_bytes, act, act_bytes) || ranges_overlap(out, out_bytes, w, w_bytes)) {
     return false;  // the ordinary path reports what is wrong, or handles the aliasing in order
   }
-  bool join = b.count > 0 && b.count < htpops::kGemvGroupMax && b.wt == wt && b.k == p->k && b.m == p->m && b.act == act;
+  bool join = b.count > 0 && b.count < htpops::kGemvGroupMax && b.wt == wt && b.m == p->m &&
+              (p->m == 1 || (b.k[0] == p->k && b.act[0] == act));
   for (int i = 0; join && i < b.count; ++i) {
-    const size_t wi = weight_bytes((size_t) b.n[i], (size_t) b.k, b.wt), oi = (size_t) b.m * b.n[i] * 4;
-    join = !ranges_overlap(out, out_bytes, b.out[i], oi) && !ranges_overlap(out, out_bytes, b.w[i], wi) &&
-           !ranges_overlap(b.out[i], oi, w, w_bytes);
+    const size_t wi = weight_bytes((size_t) b.n[i], (size_t) b.k[i], b.wt), oi = (size_t) b.m * b.n[i] * 4;
+    const size_t ai = q8_0_bytes((size_t) b.m, (size_t) b.k[i]);
+    join = !ranges_overlap(out, out_bytes, b.out[i], oi) &&   // two writers of the same bytes must stay ordered
+           !ranges_overlap(out, out_bytes, b.w[i], wi) &&     // must not clobber what a member still reads
+           !ranges_overlap(out, out_bytes, b.act[i], ai) &&
+           !ranges_overlap(b.out[i], oi, w, w_bytes) &&       // must not read what a member is about to write
+           !ranges_overlap(b.out[i], oi, act, act_bytes);
   }
   if (!join) {
     flush_batch(ctx, b);
-    b.wt = wt, b.k = p->k, b.m = p->m, b.act = act;
+    b.wt = wt, b.m = p->m;
   }
-  b.hdr[b.count] = hdr, b.out[b.count] = out, b.w[b.count] = w, b.n[b.count] = p->n;
+  b.hdr[b.count] = hdr, b.out[b.count] = out, b.w[b.count] = w, b.act[b.count] = act, b.n[b.count] = p->n, b.k[b.count] = p->k;
   ++b.count;
   hdr->state = HTPOPS_OK;
   return true;
@@ -1259,8 +1275,9 @@ int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_b
   }
   const int n_reqs = msg->n_reqs;
   GemvBatch batch;
-  ctx->act_fragments.src = nullptr;
-  ctx->in_message        = true;
+  ctx->act_fragments.src   = nullptr;
+  ctx->in_message          = true;
+  ctx->message_submissions = 0;
   for (int i = 0; i < n_reqs; ++i) {
     struct RequestHeader *hdr  = message_header_get_request_ptr(msg, i);
     const size_t          size = message_header_get_request_size(msg, i);
@@ -1275,6 +1292,7 @@ int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_b
             size >= sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest) + sizeof(MatMulParams);
           if (!(matmul_payload && try_batch(ctx, req, hdr, batch))) {
             flush_batch(ctx, batch);
+            ++ctx->message_submissions;
             hdr->state = htpops_execute_op(ctx, req);
           }
         }
@@ -1344,6 +1362,14 @@ extern "C" int htpops_process_message(htpops_context *ctx, struct MessageHeader 
     return ret;
   }
   return htpops_finish_message(ctx, msg);
+}
+
+extern "C" int htpops_last_message_submissions(htpops_context *ctx) {
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  Lock lock(ctx->mu);
+  return ctx->message_submissions;
 }
 
 // ------------------------------------------------------------------------------------------------ recorded messages

@@ -24,11 +24,13 @@ hipError_t launch_rms_norm_quantize_q8_0(hipStream_t stream, void *dst, const fl
 // decode path: one pass over the weight bytes per activation row
 hipError_t launch_gemv_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
                                 int n, WeightType wt);
-// several weight matrices against ONE shared activation row (m = 1) in a single launch; hipErrorNotSupported when
-// the shapes do not fit the fast kernel (the caller then launches them one by one)
+// several matrix-vector products (m = 1) in a single launch, each with its own weight matrix, activation row, row
+// length k and output; the caller guarantees that no member reads what another writes. hipErrorNotSupported when a
+// member does not fit the fast kernel (k % 64, k <= 12288, 4-byte aligned buffers): the caller then launches them one
+// by one.
 constexpr int kGemvGroupMax = 8;
-hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *act,
-                                      const void *const *weights, const int *ns, int k, WeightType wt);
+hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *const *acts,
+                                      const void *const *weights, const int *ns, const int *ks, WeightType wt);
 // 2 <= m <= 4 activation rows against several weight matrices in one launch: the decode kernel's stream over the
 // weights with the m rows staged in LDS (k % 64 == 0, k <= 12288, 4-byte aligned buffers; else hipErrorNotSupported)
 bool       gemv_rows_fits(int m, int k, WeightType wt);  // whether the launch below is the kernel of choice

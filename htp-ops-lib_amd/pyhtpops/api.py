@@ -50,7 +50,7 @@ EXPORTED_SYMBOLS = [
     "htpops_init_backend", "htpops_close", "htpops_last_error", "htpops_synchronize", "htpops_get_stream",
     "htpops_buffer_alloc", "htpops_buffer_register", "htpops_buffer_release", "htpops_buffer_device_ptr",
     "htpops_buffer_size", "htpops_buffer_invalidate", "htpops_buffer_write", "htpops_buffer_read", "htpops_execute_op",
-    "htpops_process_message", "htpops_enqueue_message", "htpops_finish_message",
+    "htpops_process_message", "htpops_enqueue_message", "htpops_finish_message", "htpops_last_message_submissions",
     "htpops_record_message", "htpops_launch_recorded_message", "htpops_release_recorded_message", "htpops_create_channel", "htpops_destroy_channel", "htpops_rms_norm_f32",
     "htpops_mat_mul_permuted_w16a32", "htpops_rms_norm_f32_ex_ptr", "htpops_quantize_q8_0_ptr",
     "htpops_rms_norm_quantize_q8_0_ptr", "htpops_mat_mul_q8_0_act_ptr", "htpops_mat_mul_f32_act_ptr",
@@ -90,6 +90,7 @@ def load_library(path=None):
         "htpops_process_message": (ci, [vp, vp, sz]),
         "htpops_enqueue_message": (ci, [vp, vp, sz]),
         "htpops_finish_message": (ci, [vp, vp]),
+        "htpops_last_message_submissions": (ci, [vp]),
         "htpops_record_message": (ci, [vp, vp, sz, ctypes.POINTER(vp)]),
         "htpops_launch_recorded_message": (ci, [vp, vp]),
         "htpops_release_recorded_message": (ci, [vp, vp]),
@@ -268,6 +269,9 @@ class Context:
     def finish_message(self, msg):
         buf = (ctypes.c_char * len(msg)).from_buffer(msg)
         return self.lib.htpops_finish_message(self._ctx, ctypes.cast(buf, ctypes.c_void_p))
+
+    def last_message_submissions(self):
+        return self.lib.htpops_last_message_submissions(self._ctx)
 
     def record_message(self, msg):
         """htpops_record_message: runs `msg` once and returns (code, recording); the recording is None on failure."""

@@ -109,6 +109,12 @@ int htpops_process_message(htpops_context *ctx, struct MessageHeader *msg, size_
 int htpops_enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes);
 int htpops_finish_message(htpops_context *ctx, struct MessageHeader *msg);
 
+/* How many separately launched units the most recent walk of a message on this context issued: compute requests that
+ * were grouped into one kernel launch count once (diagnostic; the reference runs one op per request,
+ * src/dsp/commu.c:91-100). Grouping never changes a result: a request joins a group only if it neither reads nor
+ * overwrites what an earlier member writes and writes nothing an earlier member reads. */
+int htpops_last_message_submissions(htpops_context *ctx);
+
 /* A message recorded once and replayed many times: the kernel launches of a whole message (a decoder block that is
  * submitted again for every token, reference: src/dsp/commu.c:91-114 walks it anew each time) are captured into one
  * HIP graph and re-enqueued on the context's stream with a single call.

@@ -641,3 +641,96 @@ def test_buffer_invalidate_drops_converted_weight_copies(ctx, oracle):
     finally:
         for h in (ha, hw, ho):
             ctx.release(h)
+
+
+def _mm(op, ho, ha, hw, m, k, n, out_off=0, act_off=0):
+    return (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, api.mat_mul_params((ho, out_off), (ha, act_off), (hw, 0), m, k, n)))
+
+
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+def test_message_groups_independent_gemvs_of_different_activations(ctx, oracle, wt):
+    # one-row matmuls whose inputs and outputs are all independent run as ONE launch even when they read different
+    # activation buffers and have different k (the reference runs them one after the other, commu.c:91-114; with no
+    # data dependency between them the order cannot be observed). Every request must equal its own launch bit for bit.
+    rng = wl.rng_for(73, wt)
+    op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
+    shapes = [(256, 1536), (272, 1536), (100, 4096), (1536, 8960), (33, 64), (640, 11008), (7, 2048)]   # (n, k)
+    ws = [wl.make_weights(rng, n, k, wt) for n, k in shapes]
+    acts = [oracle.quantize_q8_0(wl.make_activations(rng, 1, k)) for _, k in shapes]
+    acts[1] = acts[0]  # two members share an activation row
+    has = [ctx.upload(a) for a in acts]
+    ctx.release(has[1])
+    has[1] = has[0]
+    hws = [ctx.upload(w) for w in ws]
+    hos = [ctx.alloc(n * 4) for n, _ in shapes]
+    try:
+        msg = api.build_message([_mm(op, ho, ha, hw, 1, k, n) for ho, ha, hw, (n, k) in zip(hos, has, hws, shapes)])
+        for _ in range(2):
+            for ho, (n, _) in zip(hos, shapes):
+                ctx.write(ho, np.full(n, np.nan, np.float32))
+            assert ctx.process_message(msg) == 0
+            assert api.message_request_states(msg) == [0] * len(shapes), ctx.last_error()
+            assert ctx.last_message_submissions() == 1
+            for ho, a, w, (n, k) in zip(hos, acts, ws, shapes):
+                got = ctx.read(ho, np.float32, n)
+                assert np.array_equal(got, ctx.run_mat_mul(a, w, 1, k, n, wt)[0]), "a request differs from its own launch"
+                want, mag = oracle.mat_mul_q8_0_act_f64(a, w, 1, k, n, wt)
+                assert np.all(np.abs(got - want[0]) <= MATMUL_RTOL * mag[0])
+    finally:
+        for h in set(has) | set(hws) | set(hos):
+            ctx.release(h)
+
+
+def test_message_keeps_dependent_gemvs_in_order(ctx, oracle):
+    # Requests with a data dependency must not share a launch. (1) read-after-write: request 1's fp32 output bytes are
+    # request 2's Q8_0 activation row (unit scales and small integers make those bytes finite Q8_0 blocks);
+    # (2) write-after-read: request 3 reads activation A, request 4 writes its output over A;
+    # (3) write-after-write: requests 5 and 6 write the same output, the later one wins.
+    wt, op = wl.GGML_TYPE_Q8_0, api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
+    rng = wl.rng_for(74, 0)
+    one = np.array([1.0], np.float16).view(np.uint8)
+    k1, n1 = 256, 272                      # 272 floats = 1088 bytes = 32 Q8_0 blocks -> k2 = 1024
+    k2, n2 = 1024, 96
+    w1 = wl.make_q8_0_weights(rng, n1, k1).reshape(n1, k1 // 32, 34)
+    w1[:, :, 0:2] = one
+    w1[:, :, 2:] = rng.integers(-3, 4, (n1, k1 // 32, 32), dtype=np.int8).view(np.uint8)
+    w1 = w1.reshape(n1, -1)
+    a1 = np.empty((1, k1 // 32, 34), np.uint8)
+    a1[:, :, 0:2] = one
+    a1[:, :, 2:] = rng.integers(-3, 4, (1, k1 // 32, 32), dtype=np.int8).view(np.uint8)
+    a1 = a1.reshape(1, -1)
+    w2 = wl.make_q8_0_weights(rng, n2, k2)
+    stale = oracle.quantize_q8_0(wl.make_activations(rng, 1, k2))       # what the buffer holds before request 1 runs
+    a3 = oracle.quantize_q8_0(wl.make_activations(rng, 1, k2))
+    w4 = wl.make_q8_0_weights(rng, 272, k1)                              # 272 floats overwrite the 1088 bytes of a3
+    h = {name: ctx.upload(x) for name, x in dict(w1=w1, a1=a1, w2=w2, mid=stale, a3=a3, w4=w4).items()}
+    h.update(o2=ctx.alloc(n2 * 4), o3=ctx.alloc(n2 * 4), o5=ctx.alloc(n2 * 4))
+    try:
+        msg = api.build_message([
+            _mm(op, h["mid"], h["a1"], h["w1"], 1, k1, n1),       # 1
+            _mm(op, h["o2"], h["mid"], h["w2"], 1, k2, n2),       # 2 reads what 1 writes
+            _mm(op, h["o3"], h["a3"], h["w2"], 1, k2, n2),        # 3
+            _mm(op, h["a3"], h["a1"], h["w4"], 1, k1, 272),       # 4 overwrites what 3 reads
+            _mm(op, h["o5"], h["a3"], h["w2"], 1, k2, n2),        # 5 reads what 4 wrote
+            _mm(op, h["o5"], h["a1"], h["w1"], 1, k1, n2),        # 6 overwrites 5's output
+        ])
+        for _ in range(3):
+            ctx.write(h["mid"], stale), ctx.write(h["a3"], a3)
+            assert ctx.process_message(msg) == 0
+            assert api.message_request_states(msg) == [0] * 6, ctx.last_error()
+            assert ctx.last_message_submissions() >= 4
+            out1 = ctx.read(h["mid"], np.float32, n1)
+            _, q1 = wl.q8_0_split(a1, k1)
+            _, qw1 = wl.q8_0_split(w1, k1)
+            assert np.array_equal(out1, (q1.astype(np.int64) @ qw1.astype(np.int64).T)[0].astype(np.float32))
+            act2 = out1.view(np.uint8).reshape(1, -1)
+            assert np.array_equal(ctx.read(h["o2"], np.float32, n2), ctx.run_mat_mul(act2, w2, 1, k2, n2, wt)[0])
+            want2, mag2 = oracle.mat_mul_q8_0_act_f64(act2, w2, 1, k2, n2, wt)
+            assert np.all(np.isfinite(want2)) and np.all(np.abs(ctx.read(h["o2"], np.float32, n2) - want2[0]) <= MATMUL_RTOL * mag2[0])
+            assert np.array_equal(ctx.read(h["o3"], np.float32, n2), ctx.run_mat_mul(a3, w2, 1, k2, n2, wt)[0])
+            out4 = ctx.read(h["a3"], np.float32, 272)
+            assert np.array_equal(out4, ctx.run_mat_mul(a1, w4, 1, k1, 272, wt)[0])
+            assert np.array_equal(ctx.read(h["o5"], np.float32, n2), out1[:n2])
+    finally:
+        for v in h.values():
+            ctx.release(v)
