@@ -1,0 +1,507 @@
+// Prefill-sized Q4_0 x Q8_0 matmul on gfx950: out fp32 [m][n] = act block_q8_0 [m][k/32] x W (Q4_0 rows), exact block
+// sums on the FP6 matrix instruction, operands staged in LDS by DMA.
+//
+// Replaces the many-row case of hmx_mat_mul_permuted_qk_0_d16a32 (reference: src/dsp/ops/mat_mul.c:875-1153), whose
+// pipeline stages a weight chunk in on-chip memory, converts it there and feeds the matrix unit while the next chunk is
+// on its way (:964-999, :1006-1139), with the activations re-tiled once per call (:89-128).
+//
+// Arithmetic per 32 x 32 x 32 block ("unit"): ggml's integer block dot, exact.
+//     S = act_int8 x (q - 8)    ONE v_mfma_scale_f32_32x32x64_f8f6f4 on FP6 (E2M3) operands: an int8 activation is
+//                               a = 16 hi + lo with hi in [-8, 7], lo in [0, 15]; hi, lo and q - 8 are integers of
+//                               magnitude <= 15, which E2M3 holds exactly as t / 8 (code = sign bit | magnitude).
+//                               The instruction's K = 64 is spent as [hi (32) | lo (32)] against [w (32) | w (32)];
+//                               its per-32 power-of-two block scales supply the 16 of the hi half and undo the 1/8s.
+//                               S leaves the matrix core as fp32, so no int -> float conversion is needed.
+//     C = d_act (x) d_w         one v_mfma_f32_32x32x8_f16 with the fp16 scales in K slots 0 / 1: the exact fp32
+//                               product of every (row, column) scale pair
+//     acc = fma(S, C, acc)      the only vector-ALU work: one fma per block sum (half of what int8 MFMA + convert +
+//                               fma issues, and the vector ALU is what bounds this arithmetic)
+// Both operands are kept in the byte order the matrix core wants ("tiles"), so that the kernel's memory side is DMA
+// straight into LDS and ds_read into operand registers, with no data shuffling and no vector-ALU work:
+//   weights      converted once per weight buffer (1 byte per weight incl. scales) and cached by the caller
+//   activations  converted per call from block_q8_0 rows; shared by the matmuls of a message that read the same rows
+// A workgroup owns 128 x 64 outputs over all of K (no exchange between workgroups, results independent of the grid):
+// 8 waves, one 32 x 32 accumulator tile each, few registers per wave, several waves per SIMD -- while one accumulates,
+// another one's matrix instructions run. K advances in steps of two blocks through a ring of three LDS stages filled
+// two steps ahead. With KS = 2 a second group of 8 waves takes the other half of K (shapes with too few tiles to fill
+// the device) and the two partial tiles are added through LDS in a fixed order.
+#include "device_utils.h"
+#include "kernels.h"
+
+#include <algorithm>
+#include <type_traits>
+
+namespace htpops {
+
+namespace {
+
+typedef int      v4i __attribute__((ext_vector_type(4)));
+typedef int      v2i __attribute__((ext_vector_type(2)));
+typedef int      v8i __attribute__((ext_vector_type(8)));
+typedef float    v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+constexpr int kBM = 128, kBN = 64;  // outputs per workgroup
+constexpr int kGroupWaves = 4;      // each wave: 64 x 32 outputs (two accumulator tiles)
+constexpr int kNA = 3;              // LDS stages
+constexpr int kMinTiles = 192;      // output tiles from which the kernel is used
+
+// ---- tiles ----------------------------------------------------------------------------------------------------------
+// The 32 FP6 codes of one row (column) of a block are 24 bytes, element e at bits [6 e, 6 e + 6). A step = a block
+// pair; its two code strings travel as three 16-byte pieces per lane ("planes"):
+//   plane 0 = [lane][block 0 bytes 0..15], plane 1 = [lane][block 0 bytes 16..23] then [lane][block 1 bytes 16..23],
+//   plane 2 = [lane][block 1 bytes 0..15]
+// so that each block's operand registers are filled by one 16-byte and one 8-byte LDS read.
+//   activation tile (32 rows, step): 3 planes x 64 lanes x 16 bytes; lane (c, h): row c, h = 0 the hi parts, h = 1 the lo
+//                                    parts. Row scales apart: one dword per row and step (even block | odd block << 16).
+//   weight tile (64 columns, step):  3 planes x 64 columns x 16 bytes, then the scales as operand dwords of the scale
+//                                    product: [block][column tile of 32][64 lanes], lane l < 32: the column's fp16
+//                                    scale in the half-word of its block (K slot 0 or 1), lanes 32..63: 0.
+constexpr int kATile  = 3 * 1024;
+constexpr int kWTile  = 4 * 1024;
+constexpr int kOffA   = 0;
+constexpr int kOffW   = kOffA + (kBM / 32) * kATile;
+constexpr int kOffSa  = kOffW + kWTile;
+constexpr int kStage  = kOffSa + (kBM / 32) * 256;
+constexpr int kRing   = kNA * kStage;
+constexpr int kDmaPerStep = (kBM / 32) * 3 + 4 + (kBM / 32);  // 12 activation planes, 4 weight KiB, 4 scale rows
+
+__device__ __forceinline__ uint32_t fp6_code(int t) {  // integer |t| <= 15 as E2M3 value t / 8
+  const uint32_t mag = (uint32_t) (t < 0 ? -t : t);
+  return (t < 0 ? 32u : 0u) | mag;
+}
+
+__device__ __forceinline__ void pack_fp6(uint32_t w[6], const int t[32]) {
+#pragma unroll
+  for (int i = 0; i < 6; ++i) {
+    w[i] = 0;
+  }
+#pragma unroll
+  for (int e = 0; e < 32; ++e) {
+    const uint32_t code = fp6_code(t[e]);
+    const int      bit  = 6 * e;
+    w[bit / 32] |= code << (bit % 32);
+    if (bit % 32 > 26) {
+      w[bit / 32 + 1] |= code >> (32 - bit % 32);
+    }
+  }
+}
+
+__device__ __forceinline__ void store_planes(uint8_t *tile, int lane, const uint32_t (&b0)[6], const uint32_t (&b1)[6]) {
+  uint4 *p = reinterpret_cast<uint4 *>(tile) + lane;
+  p[0]   = make_uint4(b0[0], b0[1], b0[2], b0[3]);
+  p[128] = make_uint4(b1[0], b1[1], b1[2], b1[3]);
+  uint2 *q = reinterpret_cast<uint2 *>(tile + 1024) + lane;
+  q[0]  = make_uint2(b0[4], b0[5]);
+  q[64] = make_uint2(b1[4], b1[5]);
+}
+
+// one thread per (column tile, step, column)
+__global__ __launch_bounds__(256) void q4_0_to_fp6_tiles_kernel(uint8_t *__restrict__ tiles, const uint32_t *__restrict__ w,
+                                                                int n, int pairs, size_t total) {
+  const size_t t = (size_t) blockIdx.x * 256 + threadIdx.x;
+  if (t >= total) {
+    return;
+  }
+  const int    c = (int) (t & 63);
+  const size_t rec = t >> 6;  // tile * pairs + step
+  const int    step = (int) (rec % (size_t) pairs), tile = (int) (rec / (size_t) pairs);
+  const int    col = tile * kBN + c;
+  uint32_t     o0[6] = { 0, 0, 0, 0, 0, 0 }, o1[6] = { 0, 0, 0, 0, 0, 0 };
+  uint32_t     d0 = 0, d1 = 0;
+  if (col < n) {
+    const uint32_t *src = w + ((size_t) col * pairs + step) * 9;  // [d0:2][16 nibble bytes][d1:2][16 nibble bytes]
+    uint32_t        r[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) {
+      r[i] = src[i];
+    }
+    d0 = r[0] & 0xffffu;
+    d1 = r[4] & 0xffff0000u;
+    uint32_t q0[4], q1[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      q0[i] = __builtin_amdgcn_alignbyte(r[i + 1], r[i], 2);
+      q1[i] = r[5 + i];
+    }
+    int v0[32], v1[32];
+    // byte j: low nibble = element j, high nibble = element j + 16 (reference: mat_mul.c:266-271)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const uint32_t b0 = (q0[j / 4] >> (8 * (j % 4))) & 0xffu, b1 = (q1[j / 4] >> (8 * (j % 4))) & 0xffu;
+      v0[j] = (int) (b0 & 15) - 8, v0[j + 16] = (int) (b0 >> 4) - 8;
+      v1[j] = (int) (b1 & 15) - 8, v1[j + 16] = (int) (b1 >> 4) - 8;
+    }
+    pack_fp6(o0, v0);
+    pack_fp6(o1, v1);
+  }
+  uint8_t *tile_base = tiles + rec * kWTile;
+  store_planes(tile_base, c, o0, o1);
+  uint32_t *sc = reinterpret_cast<uint32_t *>(tile_base + 3 * 1024);
+  const int nt = c >> 5, l = c & 31;
+  sc[(0 * 2 + nt) * 64 + l]      = d0;
+  sc[(0 * 2 + nt) * 64 + 32 + l] = 0u;
+  sc[(1 * 2 + nt) * 64 + l]      = d1;
+  sc[(1 * 2 + nt) * 64 + 32 + l] = 0u;
+}
+
+// one thread per (row of the padded row count, step)
+__global__ __launch_bounds__(256) void q8_0_to_fp6_tiles_kernel(uint8_t *__restrict__ tiles, uint32_t *__restrict__ scales,
+                                                                const uint32_t *__restrict__ act, int m, int pairs,
+                                                                int rows_padded) {
+  const size_t t = (size_t) blockIdx.x * 256 + threadIdx.x;
+  const int    r = (int) (t % (size_t) rows_padded), step = (int) (t / (size_t) rows_padded);
+  if (step >= pairs) {
+    return;
+  }
+  uint32_t a[17];
+  if (r < m) {
+    const uint32_t *src = act + ((size_t) r * pairs + step) * 17;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const u32x4_a4 v = *reinterpret_cast<const u32x4_a4 *>(src + 4 * i);
+      a[4 * i] = v.x, a[4 * i + 1] = v.y, a[4 * i + 2] = v.z, a[4 * i + 3] = v.w;
+    }
+    a[16] = src[16];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 17; ++i) {
+      a[i] = 0u;
+    }
+  }
+  // block 0: quants at bytes 2 .. 33; block 1: quants at bytes 36 .. 67
+  uint32_t q[2][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    q[0][i] = __builtin_amdgcn_alignbyte(a[i + 1], a[i], 2);
+    q[1][i] = a[9 + i];
+  }
+  uint32_t oh[2][6], ol[2][6];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    int hi[32], lo[32];
+#pragma unroll
+    for (int e = 0; e < 32; ++e) {
+      const int v = (int) (int8_t) ((q[b][e / 4] >> (8 * (e % 4))) & 0xffu);
+      lo[e] = v & 15;               // a = 16 hi + lo, hi = floor(a / 16)
+      hi[e] = (v - lo[e]) / 16;
+    }
+    pack_fp6(oh[b], hi);
+    pack_fp6(ol[b], lo);
+  }
+  uint8_t *tile = tiles + ((size_t) (r / 32) * pairs + step) * kATile;
+  store_planes(tile, r % 32, oh[0], oh[1]);
+  store_planes(tile, 32 + r % 32, ol[0], ol[1]);
+  scales[((size_t) (r / 32) * pairs + step) * 32 + (r % 32)] = (a[0] & 0xffffu) | (a[8] & 0xffff0000u);
+}
+
+// ---- the matmul -----------------------------------------------------------------------------------------------------
+template <int KS>
+__global__ __launch_bounds__(kGroupWaves * kWave * KS) void gemm_fp6_lds_kernel(float *__restrict__ out,
+                                                                                const uint8_t *__restrict__ a_tiles,
+                                                                                const uint32_t *__restrict__ a_scales,
+                                                                                const uint8_t *__restrict__ w_tiles, int m, int n,
+                                                                                int pairs, int tiles_m, int tiles_n) {
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kg = wave / kGroupWaves, u = wave % kGroupWaves;  // K group, wave of the group
+  const int wm = u >> 1, nt = u & 1;                          // rows 64 wm .. 64 wm + 63, columns 32 nt .. 32 nt + 31
+
+  // Workgroups are handed to the 8 XCDs round-robin, and each XCD has its own L2: the row blocks of one column tile
+  // (which read the same weights) are consecutive workgroups of ONE XCD.
+  const int xcd = blockIdx.x % 8, j = blockIdx.x / 8;
+  const int tile_n = (j / tiles_m) * 8 + xcd, tile_m = j % tiles_m;
+  if (tile_n >= tiles_n) {
+    return;  // whole workgroup
+  }
+
+  // steps of this K group: [s0, s0 + steps); every group runs `iters` iterations (barriers), some of them empty
+  const int iters = (pairs + KS - 1) / KS;
+  const int s0    = kg * iters;
+  const int steps = min(iters, pairs - s0);
+  auto step_of = [&](int x) { return s0 + max(0, min(x, steps - 1)); };  // (DMA for steps past the end re-reads the last one)
+
+  uint8_t       *ring  = lds + kg * kRing;
+  const uint32_t ring0 = (uint32_t) (uintptr_t) ring;
+
+  // ---- DMA: everything this kernel reads from memory goes straight into LDS (written out as instructions: the
+  // compiler would make every LDS read after a DMA it knows of wait for ALL DMA in flight). The kDmaPerStep = 20
+  // transfers of a step are dealt to the 4 waves of a K group, 5 each: wave u issues activation planes u, u + 4 and
+  // u + 8 (of 12: row tile p / 3, plane p % 3), weight KiB u and the scales of row tile u. Addresses are a scalar base
+  // (tile and step) plus a per-lane offset that never changes, so a transfer costs no vector ALU work. ----
+  auto dma16 = [&](const uint8_t *base, uint32_t lane_off, uint32_t dst) {
+    asm volatile("s_mov_b32 m0, %2\n s_nop 0\n global_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(dst) : "memory");
+  };
+  auto dma4 = [&](const void *base, uint32_t lane_off, uint32_t dst) {
+    asm volatile("s_mov_b32 m0, %2\n s_nop 0\n global_load_lds_dword %0, %1" ::"v"(lane_off), "s"(base), "s"(dst) : "memory");
+  };
+  const int last_mt = (m + 31) / 32 - 1;
+  auto      row_tile = [&](int i) { return (size_t) min(tile_m * (kBM / 32) + i, last_mt); };
+  const uint8_t *src_a[3];
+  uint32_t       dst_a[3];
+#pragma unroll
+  for (int i = 0; i < 3; ++i) {
+    const int p = u + 4 * i;
+    src_a[i] = a_tiles + row_tile(p / 3) * pairs * kATile + (p % 3) * 1024;
+    dst_a[i] = ring0 + kOffA + (p / 3) * kATile + (p % 3) * 1024;
+  }
+  const uint8_t  *src_w  = w_tiles + (size_t) tile_n * pairs * kWTile + u * 1024;
+  const uint32_t  dst_w  = ring0 + kOffW + u * 1024;
+  const uint32_t *src_s  = a_scales + row_tile(u) * pairs * 32;
+  const uint32_t  dst_s  = ring0 + kOffSa + u * 256;
+  const uint32_t  lane16 = lane * 16, lane4 = (lane & 31) * 4;
+  auto issue_group = [&](int x, int stage) {  // the transfers of step x into `stage`
+    const size_t   s  = (size_t) step_of(x);
+    const uint32_t so = (uint32_t) stage * kStage;
+    dma4(src_s + s * 32, lane4, dst_s + so);
+    dma16(src_w + s * kWTile, lane16, dst_w + so);
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      dma16(src_a[i] + s * kATile, lane16, dst_a[i] + so);
+    }
+  };
+  static_assert(kDmaPerStep == 5 * kGroupWaves, "five transfers per wave and step");
+
+  static_assert(kNA == 3, "the loop below is unrolled over the three stages");
+  issue_group(0, 0);
+  issue_group(1, 1);
+
+  const v16f zero_f = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+  v16f       acc0 = zero_f, acc1 = zero_f;  // rows 64 wm .. + 31 and 64 wm + 32 .. + 63
+  // block scales of the FP6 instruction (E8M0 bytes): activations 2^3 (lo half) or 2^7 (hi half: x 16), weights 2^3
+  const int scale_a = (lane >> 5) ? 127 + 3 : 127 + 7, scale_b = 127 + 3;
+  const uint32_t a_rd  = ring0 + kOffA + (2 * wm) * kATile + lane * 16;
+  const uint32_t a_rd8 = ring0 + kOffA + (2 * wm) * kATile + 1024 + lane * 8;  // plane 1: [block 0 tails: 64 x 8][block 1 tails]
+  const uint32_t w_rd  = ring0 + kOffW + (nt * 32 + (lane & 31)) * 16;
+  const uint32_t w_rd8 = ring0 + kOffW + 1024 + (nt * 32 + (lane & 31)) * 8;
+  const uint32_t sb_rd = ring0 + kOffW + 3 * 1024 + nt * 256 + lane * 4;
+  const uint32_t sa_rd = ring0 + kOffSa + (2 * wm) * 256 + lane * 4;
+
+  typedef __attribute__((address_space(3))) const uint8_t *lds_ptr;
+  auto lds_v4i = [](uint32_t addr, int off) {
+    return *reinterpret_cast<__attribute__((address_space(3))) const v4i *>((lds_ptr) (uintptr_t) addr + off);
+  };
+  auto lds_u32 = [](uint32_t addr, int off) {
+    return *reinterpret_cast<__attribute__((address_space(3))) const uint32_t *>((lds_ptr) (uintptr_t) addr + off);
+  };
+  auto operand = [](v4i lo, v2i hi) {  // (elements 6 and 7 of an FP6 operand are not read by the instruction)
+    v8i f;
+    f[0] = lo[0], f[1] = lo[1], f[2] = lo[2], f[3] = lo[3], f[4] = hi[0], f[5] = hi[1];
+    return f;
+  };
+  auto fma_half = [](v16f &acc, const v16f &s, const v16f &c, int half) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      acc[half * 8 + i] = __builtin_fmaf(s[half * 8 + i], c[half * 8 + i], acc[half * 8 + i]);
+    }
+  };
+
+  // Block sums / scale products in flight: x belongs to the upper row tile (acc0), y to the lower one (acc1).
+  v16f sx = zero_f, cx = zero_f, sy = zero_f, cy = zero_f;
+  // One step out of stage ST (a compile-time constant: every LDS offset is an immediate). A wave's four units of a
+  // step -- (row tile, block) = (0, 0), (1, 0), (0, 1), (1, 1) -- are software-pipelined: behind every matrix instruction
+  // come eight fmas of the unit before, so that the matrix core and the vector ALU both stay busy from within one
+  // wave. The last unit's fmas are deferred past the next barrier, behind the first matrix instructions of the next
+  // step. The 8-byte tails are read with written-out instructions so that each lands in the two registers behind its
+  // operand's first four.
+  auto step = [&](auto stage_tag, int t) {
+    constexpr int ST = decltype(stage_tag)::value;
+    constexpr int so = ST * kStage;
+    // step t is complete in LDS: this wave's transfers of it have landed (the next step's five may stay in flight;
+    // s_waitcnt operand: vmcnt in bits 3:0 and 15:14, expcnt 7 = no wait in 6:4, lgkmcnt(0) in 11:8), then everybody's
+    __builtin_amdgcn_s_waitcnt(0x0070 | 5);
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    v2i a00hi, a01hi, a10hi, a11hi, b0hi, b1hi;  // a<row tile><block>
+    asm volatile(
+        "ds_read_b64 %0, %6 offset:%c8\n ds_read_b64 %1, %6 offset:%c9\n ds_read_b64 %2, %6 offset:%c10\n"
+        " ds_read_b64 %3, %6 offset:%c11\n ds_read_b64 %4, %7 offset:%c12\n ds_read_b64 %5, %7 offset:%c13"
+        : "=&v"(a00hi), "=&v"(a01hi), "=&v"(a10hi), "=&v"(a11hi), "=&v"(b0hi), "=&v"(b1hi)
+        : "v"(a_rd8), "v"(w_rd8), "i"(so), "i"(so + 512), "i"(so + kATile), "i"(so + kATile + 512), "i"(so), "i"(so + 512)
+        : "memory");
+    const v4i      a00lo = lds_v4i(a_rd, so), a01lo = lds_v4i(a_rd, so + 2048);
+    const v4i      a10lo = lds_v4i(a_rd, so + kATile), a11lo = lds_v4i(a_rd, so + kATile + 2048);
+    const v4i      b0lo = lds_v4i(w_rd, so), b1lo = lds_v4i(w_rd, so + 2048);
+    const uint32_t sb0 = lds_u32(sb_rd, so), sb1 = lds_u32(sb_rd, so + 512);
+    uint32_t       sa0 = lds_u32(sa_rd, so), sa1 = lds_u32(sa_rd, so + 256);
+    // everybody has left step t - 1: its stage takes step t + 2
+    issue_group(t + 2, (ST + 2) % kNA);
+    if (KS > 1) {
+      sa0 = t < steps ? sa0 : 0u;  // an iteration past this K group's last step adds zeros
+      sa1 = t < steps ? sa1 : 0u;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a00hi), "+v"(a01hi), "+v"(a10hi), "+v"(a11hi), "+v"(b0hi), "+v"(b1hi)::"memory");
+    const v8i fa00 = operand(a00lo, a00hi), fa01 = operand(a01lo, a01hi), fa10 = operand(a10lo, a10hi), fa11 = operand(a11lo, a11hi);
+    const v8i fb0 = operand(b0lo, b0hi), fb1 = operand(b1lo, b1hi);
+    const v4h sa0_op = __builtin_bit_cast(v4h, make_uint2(sa0, 0u)), sa1_op = __builtin_bit_cast(v4h, make_uint2(sa1, 0u));
+    const v4h sb0_op = __builtin_bit_cast(v4h, make_uint2(sb0, 0u)), sb1_op = __builtin_bit_cast(v4h, make_uint2(sb1, 0u));
+#define HTPOPS_FP6_SUMS(fa, fb) __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa, fb, zero_f, 2, 2, 0, scale_a, 0, scale_b)
+#define HTPOPS_SCALE_PRODUCTS(sa, sb) __builtin_amdgcn_mfma_f32_32x32x8f16(sa, sb, zero_f, 0, 0, 0)
+#define HTPOPS_FENCE __builtin_amdgcn_sched_barrier(0)
+    HTPOPS_FENCE;
+    sx = HTPOPS_FP6_SUMS(fa00, fb0);            HTPOPS_FENCE;
+    fma_half(acc1, sy, cy, 0);                  HTPOPS_FENCE;  // unit (1, 1) of the step before (zeros at the start)
+    cx = HTPOPS_SCALE_PRODUCTS(sa0_op, sb0_op); HTPOPS_FENCE;
+    fma_half(acc1, sy, cy, 1);                  HTPOPS_FENCE;
+    sy = HTPOPS_FP6_SUMS(fa10, fb0);            HTPOPS_FENCE;
+    fma_half(acc0, sx, cx, 0);                  HTPOPS_FENCE;
+    cy = HTPOPS_SCALE_PRODUCTS(sa1_op, sb0_op); HTPOPS_FENCE;
+    fma_half(acc0, sx, cx, 1);                  HTPOPS_FENCE;
+    sx = HTPOPS_FP6_SUMS(fa01, fb1);            HTPOPS_FENCE;
+    fma_half(acc1, sy, cy, 0);                  HTPOPS_FENCE;
+    cx = HTPOPS_SCALE_PRODUCTS(sa0_op, sb1_op); HTPOPS_FENCE;
+    fma_half(acc1, sy, cy, 1);                  HTPOPS_FENCE;
+    sy = HTPOPS_FP6_SUMS(fa11, fb1);            HTPOPS_FENCE;
+    fma_half(acc0, sx, cx, 0);                  HTPOPS_FENCE;
+    cy = HTPOPS_SCALE_PRODUCTS(sa1_op, sb1_op); HTPOPS_FENCE;
+    fma_half(acc0, sx, cx, 1);                  HTPOPS_FENCE;
+#undef HTPOPS_FP6_SUMS
+#undef HTPOPS_SCALE_PRODUCTS
+#undef HTPOPS_FENCE
+  };
+  for (int t = 0; t < iters; t += 3) {
+    step(std::integral_constant<int, 0>(), t);
+    if (t + 1 < iters) {
+      step(std::integral_constant<int, 1>(), t + 1);
+    }
+    if (t + 2 < iters) {
+      step(std::integral_constant<int, 2>(), t + 2);
+    }
+  }
+  fma_half(acc1, sy, cy, 0);  // the last step's unit (1, 1)
+  fma_half(acc1, sy, cy, 1);
+
+  // -- the K groups meet: group g > 0 leaves its tiles in LDS, group 0 adds them in order --
+  __builtin_amdgcn_s_waitcnt(0x0070);  // (transfers of steps past the end must have landed before LDS is reused or released)
+  if (KS > 1) {
+    __builtin_amdgcn_s_barrier();
+    float *red = reinterpret_cast<float *>(lds);
+    if (kg > 0) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        red[(((kg - 1) * kGroupWaves + u) * 32 + i) * 64 + lane]      = acc0[i];
+        red[(((kg - 1) * kGroupWaves + u) * 32 + 16 + i) * 64 + lane] = acc1[i];
+      }
+    }
+    __syncthreads();
+    if (kg > 0) {
+      return;
+    }
+#pragma unroll
+    for (int g = 1; g < KS; ++g) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        acc0[i] += red[(((g - 1) * kGroupWaves + u) * 32 + i) * 64 + lane];
+        acc1[i] += red[(((g - 1) * kGroupWaves + u) * 32 + 16 + i) * 64 + lane];
+      }
+    }
+  }
+
+  const int col = tile_n * kBN + nt * 32 + (lane & 31);
+  if (col < n) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = tile_m * kBM + wm * 64 + (i / 4) * 8 + (lane >> 5) * 4 + (i & 3);
+      if (row < m) {
+        out[(size_t) row * n + col] = acc0[i];
+      }
+      if (row + 32 < m) {
+        out[(size_t) (row + 32) * n + col] = acc1[i];
+      }
+    }
+  }
+}
+
+template <int KS>
+hipError_t launch_instance(hipStream_t stream, float *out, const uint8_t *a_tiles, const uint32_t *a_scales,
+                           const uint8_t *w_tiles, int m, int n, int pairs) {
+  const int    tiles_m = (m + kBM - 1) / kBM, tiles_n = (n + kBN - 1) / kBN;
+  const size_t lds     = (size_t) KS * kRing;
+  const dim3   grid((unsigned) (((tiles_n + 7) / 8) * 8 * tiles_m));
+  auto         kernel  = gemm_fp6_lds_kernel<KS>;
+  static bool  raised  = false;
+  if (!raised) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) {
+      return e;
+    }
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(kGroupWaves * kWave * KS), lds, stream, out, a_tiles, a_scales, w_tiles, m, n, pairs,
+                     tiles_m, tiles_n);
+  return hipGetLastError();
+}
+
+}  // namespace
+
+bool gemm_fp6_lds_fits(int m, int k, int n) {
+  return m >= 1 && n >= 1 && k >= 64 && k % 64 == 0;
+}
+
+bool gemm_fp6_lds_fills_device(int m, int n) {
+  // Below this the kernel's workgroups (one per tile, K split over at most three wave groups inside it) leave compute
+  // units idle, and the fragment kernel, which splits K over workgroups, is faster.
+  return (long) ((m + kBM - 1) / kBM) * ((n + kBN - 1) / kBN) >= kMinTiles;
+}
+
+size_t gemm_fp6_lds_weight_tile_bytes(int k, int n) {
+  return (size_t) ((n + kBN - 1) / kBN) * (size_t) (k / 64) * kWTile;
+}
+
+size_t gemm_fp6_lds_act_tile_bytes(int m, int k) {
+  const size_t m_tiles = ((size_t) m + 31) / 32, pairs = (size_t) k / 64;
+  return m_tiles * pairs * kATile + m_tiles * pairs * 128;
+}
+
+hipError_t launch_q4_0_to_fp6_tiles(hipStream_t stream, void *dst, const void *weight, int k, int n) {
+  if (k % 64 != 0 || n <= 0 || (reinterpret_cast<uintptr_t>(weight) & 3) != 0) {
+    return hipErrorNotSupported;
+  }
+  const int    pairs = k / 64;
+  const size_t total = (size_t) ((n + kBN - 1) / kBN) * pairs * 64;
+  hipLaunchKernelGGL(q4_0_to_fp6_tiles_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, stream,
+                     static_cast<uint8_t *>(dst), static_cast<const uint32_t *>(weight), n, pairs, total);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm_fp6_lds(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_tiles, int m, int k,
+                               int n, void *act_tiles, bool act_tiles_ready) {
+  if (!gemm_fp6_lds_fits(m, k, n) || (reinterpret_cast<uintptr_t>(act_q8_0) & 3) != 0) {
+    return hipErrorNotSupported;
+  }
+  const int pairs   = k / 64;
+  const int m_tiles = (m + 31) / 32;
+  uint8_t  *tiles   = static_cast<uint8_t *>(act_tiles);
+  uint32_t *scales  = reinterpret_cast<uint32_t *>(tiles + (size_t) m_tiles * pairs * kATile);
+  if (!act_tiles_ready) {
+    const size_t threads = (size_t) m_tiles * 32 * pairs;
+    hipLaunchKernelGGL(q8_0_to_fp6_tiles_kernel, dim3((unsigned) ((threads + 255) / 256)), dim3(256), 0, stream, tiles, scales,
+                       static_cast<const uint32_t *>(act_q8_0), m, pairs, m_tiles * 32);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+      return e;
+    }
+  }
+  // A K group is 4 waves and one LDS ring, and a compute unit holds three rings: one group per workgroup when the
+  // tiles alone give every compute unit three workgroups, otherwise up to three groups per workgroup, each with its
+  // share of K, so that the same tiles put more waves on a compute unit.
+  static const int forced_ks = env_int("HTPOPS_GEMM_KGROUPS", 0);
+  const long       out_tiles = (long) ((m + kBM - 1) / kBM) * ((n + kBN - 1) / kBN);
+  int              ks        = out_tiles >= 640 ? 1 : out_tiles >= 384 ? 2 : 3;
+  ks                         = std::max(1, std::min(ks, pairs / 4));
+  if (forced_ks >= 1 && forced_ks <= 3) {
+    ks = forced_ks;
+  }
+  const uint8_t *wt = static_cast<const uint8_t *>(weight_tiles);
+  switch (ks) {
+    case 1:
+      return launch_instance<1>(stream, out, tiles, scales, wt, m, n, pairs);
+    case 2:
+      return launch_instance<2>(stream, out, tiles, scales, wt, m, n, pairs);
+    default:
+      return launch_instance<3>(stream, out, tiles, scales, wt, m, n, pairs);
+  }
+}
+
+}  // namespace htpops

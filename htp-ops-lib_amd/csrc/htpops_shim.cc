@@ -87,6 +87,7 @@ struct htpops_context {
     const void *src       = nullptr;
     size_t      src_bytes = 0;
     int         m = 0, k = 0;
+    int         kind = 0;  // which kernel family's layout (PlanKind)
   } act_fragments;
   bool in_message = false;
   // how many separately launched units (grouped launches and single ops) the most recent message walk issued
@@ -427,9 +428,6 @@ bool ranges_overlap(const void *a, size_t a_bytes, const void *b, size_t b_bytes
 
 constexpr int kFragKindRowLayout = 100;  // + ggml type, to keep apart from the tile-permuted kinds 1..4
 
-// How one quantized matmul will run and how much of the context's workspace it needs.
-constexpr int kFragKindFp6Panel  = 200;  // + ggml type: FP6 operand panels of the many-row Q4_0 matmul
-
 constexpr int kFragKindLaneOrder = 300;  // + ggml type: Q4_0 weights in matrix-core operand order (2..16 activation rows)
 
 // The repacked copy of `weight` for the few-row kernel: from the cache, or made now and cached. *out stays nullptr when
@@ -465,93 +463,120 @@ int lane_order_weights(htpops_context *ctx, const void *weight, const void *act,
   return HTPOPS_OK;
 }
 
+constexpr int kFragKindFp6Tiles = 400;  // + ggml type: FP6 operand tiles of the many-row Q4_0 matmul (LDS kernel)
+
+// Which kernel family a quantized matmul takes and how much of the context's workspace it needs.
+enum PlanKind {
+  kPlanFewRows,    // m below the many-row threshold: the weight-streaming kernels
+  kPlanLdsFp6,     // many rows, Q4_0, k % 64 == 0, enough output tiles, weights the context may keep a converted copy of
+  kPlanFragments,  // every other many-row matmul: int8 fragments (converted weights)
+};
+
 struct MatMulPlan {
-  bool        fragments = false;  // many rows: matrix-core kernels over converted operands
-  bool        fp6       = false;  // Q4_0 weights: FP6 panels; otherwise int8 fragments
+  PlanKind    kind      = kPlanFewRows;
   const void *cached    = nullptr;
   bool        cacheable = false;
-  size_t      act_bytes = 0, weight_bytes = 0;  // fragment sizes
+  int         frag_kind = 0;
+  size_t      act_bytes = 0, weight_bytes = 0;  // converted operand sizes
   size_t      ws_bytes  = 0;
 };
 
-MatMulPlan plan_mat_mul(htpops_context *ctx, const void *weight, int m, int k, int n, int wt) {
+// `act_aligned`: the Q8_0 activations start on a 4-byte boundary (the re-tiling pass of the FP6 kernel reads dwords)
+MatMulPlan plan_mat_mul(htpops_context *ctx, const void *weight, bool act_aligned, int m, int k, int n, int wt) {
   static const int frag_min_m = htpops::env_int("HTPOPS_GEMM_FRAG_MIN_M", 33);
   MatMulPlan       p;
-  if (m >= frag_min_m && k % 32 == 0) {
-    // Q4_0 weights have two many-row kernels. The FP6 one issues half the vector instructions per block but pays an
-    // exchange through memory for every output tile that several workgroups share; measured, it wins once the
-    // tiles fill the device at least once (HTPOPS_GEMM_FP6: 0 never, 1 always, unset by shape).
-    const int use_fp6 = htpops::env_int("HTPOPS_GEMM_FP6", -1);  // read per call: tests switch kernels
-    p.fragments    = true;
-    p.fp6          = wt == htpops::kQ4_0 && (use_fp6 < 0 ? htpops::gemm_fp6_fills_device(m, n) : use_fp6 != 0);
-    p.act_bytes    = ((p.fp6 ? htpops::gemm_fp6_act_panel_bytes(m, k) : htpops::gemm_i8_act_fragment_bytes(m, k)) + 255) & ~(size_t) 255;
-    p.weight_bytes = p.fp6 ? htpops::gemm_fp6_weight_panel_bytes(k, n) : htpops::gemm_i8_weight_fragment_bytes(k, n);
-    const int kind = (p.fp6 ? kFragKindFp6Panel : kFragKindRowLayout) + wt;
+  if (m < frag_min_m || k % 32 != 0) {
+    p.ws_bytes = htpops::mat_mul_workspace_bytes(m, k, n);
+    return p;
+  }
+  auto lookup_copy = [&](int frag_kind) {
+    p.frag_kind = frag_kind;
+    p.cached    = nullptr;
     for (const auto &e : ctx->frag_cache) {
-      if (e.src == weight && e.kind == kind && e.k == k && e.n == n) {
+      if (e.src == weight && e.kind == frag_kind && e.k == k && e.n == n) {
         p.cached = e.frag;
-        break;
+        return;
       }
     }
-    if (!p.cached) {
-      p.cacheable = in_owned_buffer(ctx, weight, weight_bytes((size_t) n, (size_t) k, wt));
+    p.cacheable = in_owned_buffer(ctx, weight, weight_bytes((size_t) n, (size_t) k, wt));
+  };
+  // Q4_0 weights in a buffer of the context's own, on a shape whose output tiles fill the device: the FP6 kernel over
+  // a converted copy kept with the buffer (half the vector-ALU work per block sum of the int8 path). Caller-owned
+  // memory may change behind the context's back, so nothing converted from it is kept, and the FP6 conversion is too
+  // slow to redo per call.
+  const int use_fp6 = htpops::env_int("HTPOPS_GEMM_FP6", -1);  // read per call: tests switch kernels
+  if (wt == htpops::kQ4_0 && use_fp6 != 0 && htpops::gemm_fp6_lds_fits(m, k, n) && aligned(weight, 4) && act_aligned &&
+      (use_fp6 > 0 || htpops::gemm_fp6_lds_fills_device(m, n))) {
+    lookup_copy(kFragKindFp6Tiles + wt);
+    if (p.cached || p.cacheable) {
+      p.kind         = kPlanLdsFp6;
+      p.act_bytes    = (htpops::gemm_fp6_lds_act_tile_bytes(m, k) + 255) & ~(size_t) 255;
+      p.weight_bytes = htpops::gemm_fp6_lds_weight_tile_bytes(k, n);
+      p.ws_bytes     = p.act_bytes;
+      return p;
     }
-    p.weight_bytes = (p.weight_bytes + 255) & ~(size_t) 255;
-    p.ws_bytes = p.act_bytes + ((p.cached || p.cacheable) ? 0 : p.weight_bytes) + (p.fp6 ? htpops::gemm_fp6_workspace_bytes() : 0);
-  } else {
-    p.ws_bytes = htpops::mat_mul_workspace_bytes(m, k, n);
   }
+  p.kind         = kPlanFragments;
+  p.act_bytes    = (htpops::gemm_i8_act_fragment_bytes(m, k) + 255) & ~(size_t) 255;
+  p.weight_bytes = (htpops::gemm_i8_weight_fragment_bytes(k, n) + 255) & ~(size_t) 255;
+  lookup_copy(kFragKindRowLayout + wt);
+  p.ws_bytes = p.act_bytes + ((p.cached || p.cacheable) ? 0 : p.weight_bytes);
   return p;
+}
+
+int run_few_rows(htpops_context *ctx, float *dst, const void *act, const void *weight, int m, int k, int n, int wt,
+                 uint8_t *ws) {
+  // hipErrorNotSupported from a launcher means "this kernel does not take the shape": try the next one. Any other
+  // failure is reported.
+  if (htpops::gemv_rows_fits(m, k, (htpops::WeightType) wt) && aligned(act, 4) && aligned(weight, 4)) {
+    const hipError_t e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, 1, &dst, act, &weight, &n, m, k,
+                                                                 (htpops::WeightType) wt);
+    if (e == hipSuccess) {
+      return HTPOPS_OK;
+    }
+    if (e != hipErrorNotSupported) {
+      return hip_fail(ctx, e, "few-row mat_mul launch");
+    }
+    (void) hipGetLastError();
+  }
+  const void *lw = nullptr;
+  if (int r = lane_order_weights(ctx, weight, act, m, k, n, wt, &lw)) {
+    return r;
+  }
+  if (lw) {
+    const hipError_t e = htpops::launch_matmul_lane_order_group(ctx->stream, 1, &dst, act, &lw, &n, m, k,
+                                                                (htpops::WeightType) wt);
+    if (e == hipSuccess) {
+      return HTPOPS_OK;
+    }
+    if (e != hipErrorNotSupported) {
+      return hip_fail(ctx, e, "repacked-weight mat_mul launch");
+    }
+    (void) hipGetLastError();
+  }
+  HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, act, weight, m, k, n, (htpops::WeightType) wt, ws,
+                                                  ctx->tickets, kTicketSlots));
+  return HTPOPS_OK;
 }
 
 // `ws` is this matmul's share of the workspace (plan.ws_bytes, already ensured by the caller)
 int run_mat_mul(htpops_context *ctx, MatMulPlan &plan, float *dst, const void *act, const void *weight, int m, int k,
                 int n, int wt, uint8_t *ws) {
   note_device_write(ctx, dst, (size_t) m * n * 4);
-  if (!plan.fragments || plan.fp6) {
+  if (plan.kind == kPlanFewRows) {
     ctx->act_fragments.src = nullptr;  // these kernels put something else at the start of the workspace
+    return run_few_rows(ctx, dst, act, weight, m, k, n, wt, ws);
   }
-  if (!plan.fragments) {
-    // hipErrorNotSupported from a launcher means "this kernel does not take the shape": try the next one. Any other
-    // failure is reported.
-    if (htpops::gemv_rows_fits(m, k, (htpops::WeightType) wt) && aligned(act, 4) && aligned(weight, 4)) {
-      const hipError_t e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, 1, &dst, act, &weight, &n, m, k,
-                                                                   (htpops::WeightType) wt);
-      if (e == hipSuccess) {
-        return HTPOPS_OK;
-      }
-      if (e != hipErrorNotSupported) {
-        return hip_fail(ctx, e, "few-row mat_mul launch");
-      }
-      (void) hipGetLastError();
-    }
-    const void *lw = nullptr;
-    if (int r = lane_order_weights(ctx, weight, act, m, k, n, wt, &lw)) {
-      return r;
-    }
-    if (lw) {
-      const hipError_t e = htpops::launch_matmul_lane_order_group(ctx->stream, 1, &dst, act, &lw, &n, m, k,
-                                                                  (htpops::WeightType) wt);
-      if (e == hipSuccess) {
-        return HTPOPS_OK;
-      }
-      if (e != hipErrorNotSupported) {
-        return hip_fail(ctx, e, "repacked-weight mat_mul launch");
-      }
-      (void) hipGetLastError();
-    }
-    HTPOPS_HIP(ctx, htpops::launch_mat_mul_q8_0_act(ctx->stream, dst, act, weight, m, k, n, (htpops::WeightType) wt, ws,
-                                                    ctx->tickets, kTicketSlots));
-    return HTPOPS_OK;
-  }
+  // the converted copy of the weights, for the kernels that want one
   const void *frags = plan.cached;
   if (!frags) {
     void *fresh = ws + plan.act_bytes;
     if (plan.cacheable) {
       HTPOPS_HIP(ctx, hipMalloc(&fresh, plan.weight_bytes));
     }
-    const hipError_t e = plan.fp6 ? htpops::launch_q4_0_to_fp6_panel(ctx->stream, fresh, weight, k, n)
-                                  : htpops::launch_weights_to_i8_fragments(ctx->stream, fresh, weight, k, n, (htpops::WeightType) wt);
+    const hipError_t e = plan.kind == kPlanLdsFp6 ?
+                             htpops::launch_q4_0_to_fp6_tiles(ctx->stream, fresh, weight, k, n) :
+                             htpops::launch_weights_to_i8_fragments(ctx->stream, fresh, weight, k, n, (htpops::WeightType) wt);
     if (e != hipSuccess) {
       if (plan.cacheable) {
         (void) hipFree(fresh);
@@ -559,26 +584,26 @@ int run_mat_mul(htpops_context *ctx, MatMulPlan &plan, float *dst, const void *a
       return fail(ctx, HTPOPS_ERR_HIP, "weight conversion: %s", hipGetErrorString(e));
     }
     if (plan.cacheable) {
-      ctx->frag_cache.push_back({ weight, weight_bytes((size_t) n, (size_t) k, wt),
-                                  (plan.fp6 ? kFragKindFp6Panel : kFragKindRowLayout) + wt, k, n, fresh });
+      ctx->frag_cache.push_back({ weight, weight_bytes((size_t) n, (size_t) k, wt), plan.frag_kind, k, n, fresh });
     }
     frags = fresh;
   }
-  if (plan.fp6) {
-    uint8_t *partials = ws + plan.act_bytes + ((plan.cached || plan.cacheable) ? 0 : plan.weight_bytes);
-    HTPOPS_HIP(ctx, htpops::launch_gemm_fp6_panels(ctx->stream, dst, act, frags, m, k, n, ws, partials, ctx->tickets, kTicketSlots));
-    return HTPOPS_OK;
-  }
-  // note_device_write above has already cleared the record if this matmul writes into its own activations
+  // The converted activations at the start of the workspace are shared by the requests of a message that read the same
+  // rows with the same kernel family (note_device_write above has already cleared the record if this matmul writes
+  // into its own activations).
   auto      &af    = ctx->act_fragments;
-  const bool ready = af.src == act && af.m == m && af.k == k && ws == ctx->workspace;
+  const bool ready = af.src == act && af.m == m && af.k == k && af.kind == (int) plan.kind && ws == ctx->workspace;
   const bool keep  = ready || (ctx->in_message && ws == ctx->workspace &&
                                in_owned_buffer(ctx, act, q8_0_bytes((size_t) m, (size_t) k)) &&
                                !ranges_overlap(dst, (size_t) m * n * 4, act, q8_0_bytes((size_t) m, (size_t) k)));
   af.src = nullptr;
-  HTPOPS_HIP(ctx, htpops::launch_gemm_i8_fragments(ctx->stream, dst, act, frags, m, k, n, ws, ready));
+  if (plan.kind == kPlanLdsFp6) {
+    HTPOPS_HIP(ctx, htpops::launch_gemm_fp6_lds(ctx->stream, dst, act, frags, m, k, n, ws, ready));
+  } else {
+    HTPOPS_HIP(ctx, htpops::launch_gemm_i8_fragments(ctx->stream, dst, act, frags, m, k, n, ws, ready));
+  }
   if (keep) {
-    af.src = act, af.src_bytes = q8_0_bytes((size_t) m, (size_t) k), af.m = m, af.k = k;
+    af.src = act, af.src_bytes = q8_0_bytes((size_t) m, (size_t) k), af.m = m, af.k = k, af.kind = (int) plan.kind;
   }
   return HTPOPS_OK;
 }
@@ -591,7 +616,7 @@ int op_mat_mul_q8(htpops_context *ctx, float *dst, const void *act, const void *
   if (int r = need_device(ctx)) {
     return r;
   }
-  MatMulPlan plan = plan_mat_mul(ctx, weight, m, k, n, weight_type);
+  MatMulPlan plan = plan_mat_mul(ctx, weight, aligned(act, 4), m, k, n, weight_type);
   if (int r = ensure_workspace(ctx, plan.ws_bytes, /*keep_act_fragments=*/true)) {
     return r;
   }
@@ -611,7 +636,7 @@ int op_mat_mul_f32(htpops_context *ctx, float *dst, const float *act, const void
   }
   // workspace: [quantized activations][what the matmul itself needs]
   const size_t q_bytes = (q8_0_bytes((size_t) m, (size_t) k) + 255) & ~(size_t) 255;
-  MatMulPlan   plan    = plan_mat_mul(ctx, weight, m, k, n, weight_type);
+  MatMulPlan   plan    = plan_mat_mul(ctx, weight, true, m, k, n, weight_type);
   if (int r = ensure_workspace(ctx, q_bytes + plan.ws_bytes)) {
     return r;
   }

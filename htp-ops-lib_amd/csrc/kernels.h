@@ -60,6 +60,17 @@ hipError_t launch_weights_to_lane_order(hipStream_t stream, void *dst, const voi
 hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *const *outs, const void *act,
                                           const void *const *lane_order_weights, const int *ns, int m, int k,
                                           WeightType wt);
+// many-row path for Q4_0 weights, k % 64 == 0: FP6 scaled MFMA (exact: int8 = 16 hi + lo, all parts |t| <= 15) over operand
+// tiles staged in LDS by DMA. The weight tiles (gemm_fp6_lds_weight_tile_bytes, 1 byte per weight) are converted once
+// (launch_q4_0_to_fp6_tiles) and can be cached by the caller; the activation tiles (gemm_fp6_lds_act_tile_bytes) are
+// written per call unless `act_tiles_ready`. Buffers 4-byte aligned, else hipErrorNotSupported.
+bool       gemm_fp6_lds_fits(int m, int k, int n);
+bool       gemm_fp6_lds_fills_device(int m, int n);  // enough 128 x 64 output tiles to keep every compute unit busy
+size_t     gemm_fp6_lds_weight_tile_bytes(int k, int n);
+size_t     gemm_fp6_lds_act_tile_bytes(int m, int k);
+hipError_t launch_q4_0_to_fp6_tiles(hipStream_t stream, void *dst, const void *weight, int k, int n);
+hipError_t launch_gemm_fp6_lds(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_tiles, int m, int k,
+                               int n, void *act_tiles, bool act_tiles_ready);
 // many-row path: int8 MFMA over operands in fragment order. The weights are converted once
 // (launch_weights_to_i8_fragments into gemm_i8_weight_fragment_bytes) and can be cached by the caller; the
 // activations are converted per call into `act_fragments` (gemm_i8_act_fragment_bytes), unless the caller says that
@@ -70,18 +81,6 @@ hipError_t launch_weights_to_i8_fragments(hipStream_t stream, void *dst, const v
                                           WeightType wt);
 hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_fragments,
                                     int m, int k, int n, void *act_fragments, bool act_fragments_ready);
-// many-row path for Q4_0 weights: FP6 scaled MFMA over operand panels (exact: int8 = 16 hi + lo, all parts |t| <= 15).
-// The weight panel (gemm_fp6_weight_panel_bytes) is converted once and can be cached by the caller; the activation
-// panel (gemm_fp6_act_panel_bytes) is scratch written per call.
-size_t     gemm_fp6_weight_panel_bytes(int k, int n);
-size_t     gemm_fp6_act_panel_bytes(int m, int k);
-hipError_t launch_q4_0_to_fp6_panel(hipStream_t stream, void *dst, const void *weight, int k, int n);
-// `workspace` (gemm_fp6_workspace_bytes) holds the partial tiles of K ranges shared between workgroups, `tickets` is
-// an array of `ticket_slots` zeroed counters that the kernel leaves zeroed.
-size_t     gemm_fp6_workspace_bytes();
-bool       gemm_fp6_fills_device(int m, int n);  // at least one 128 x 256 output tile per compute unit
-hipError_t launch_gemm_fp6_panels(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_panel, int m,
-                                  int k, int n, void *act_panel, void *workspace, unsigned *tickets, int ticket_slots);
 // picks between the one-row and the small-batch kernel by m (any m; many rows are better served by the fragment path)
 size_t     mat_mul_workspace_bytes(int m, int k, int n);
 hipError_t launch_mat_mul_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
