@@ -2,25 +2,30 @@
 """Benchmark of the op backend's hot path on one MI355X.
 
 A step is one Llama-7B decoder layer's seven Q4_0 x Q8_0 matrix-vector products at m = 1 (q/k/v/o 4096x4096,
-gate/up 11008x4096, down 4096x11008), submitted as ONE mailbox message (seven OP_COMPUTE requests) and executed
-back-to-back on the context's stream; requests that read the same activation buffer (q/k/v, gate/up) share a launch. Weights of LAYERS distinct layers are resident in HBM and steps rotate
-through them (LAYERS x 113.8 MB > the 256 MB memory-side cache), so every step streams its weights from HBM.
+gate/up 11008x4096, down 4096x11008), submitted as ONE mailbox message (seven OP_COMPUTE requests). The seven
+requests write seven different outputs and read nothing another one writes, so the message becomes ONE kernel launch
+that streams all seven weight matrices. Weights of LAYERS distinct layers are resident in HBM and steps rotate through
+them (LAYERS x 113.8 MB > the 256 MB memory-side cache), so every step streams its weights from HBM.
 `value` is algorithmic bytes per step / time per step (weights once, Q8_0 activations once, fp32 outputs once).
 
 The same run also measures, and reports inside the JSON line:
-  roofline      the launch that takes the largest share of the step (gate + up, 2 x 11008 x 4096 in one launch):
-                algorithmic bytes per launch / average launch duration from HIP events on the launching stream,
-                against 8 TB/s
-  prefill_gemm  m = 512 Q4_0 GEMM, both shapes of config 2, in int8 Tera-ops/s (2 m n k per launch)
+  roofline      that one launch: algorithmic bytes per launch / average launch duration from HIP events on the
+                launching stream, against 8 TB/s; `traffic` is the HBM-side byte count of the same launch from hardware
+                counters, profiled offline (counters cannot be read from inside a run) and kept beside the package
+  step_us       the step time again over 20 blocks of steps: median, 10th and 90th percentile
+  launches      q+k+v, o, gate+up and down as launches of their own (cold weights), each with its share of HBM peak
+  prefill_gemm  m = 512 Q4_0 GEMM, both shapes of config 2, in int8 Tera-ops/s (2 m n k per launch); the per-call
+                re-tiling of the activations and the one-time conversion of a weight buffer are reported separately
   small_batch   the same layer at m = 8
   recorded_message_us_per_step   the m = 1 and m = 8 steps again, each layer's message recorded once into a HIP graph
                 and replayed (reported beside `value`, which is the ordinary message walk)
   q8_0_block    the Qwen2-1.5B-like Q8_0 block of config 4 at m = 1 and m = 128
   decode_chain_us   config 0: RMSNorm -> Q8_0 -> GEMV (4096 x 4096) for one token, submitted as one message
-  attention     config 3: decode (1 x 4096) and causal prefill (2048 x 2048), 32 query / 8 KV heads of 128, fp16
-  launches      the four kernel launches of the step one by one (q+k+v, o, gate+up, down) on cold weights
-  cpu_baseline  the scalar C oracle (a port of the same arithmetic) on the host cores, same layer, m = 1
-  peaks         MFMA-only loops and a plain copy kernel measured on this device
+  elementwise   RMSNorm, the Q8_0 quantizer and the fused RMSNorm + quantizer over m x 4096 at m = 1 / 128 / 512
+  attention     config 3: decode (1 x 4096, 1 x 16384) and causal prefill (2048 x 2048), 32 query / 8 KV heads of 128, fp16
+  cpu_baseline  the scalar C oracle (a port of the same arithmetic) on the host cores: the headline layer, and under
+                `others` the prefill GEMM, the Q8_0 block, attention and RMSNorm on bounded samples
+  peaks         MFMA-only loops, a plain copy kernel and a pure one-pass read of the step's bytes, measured on this device
 Every GPU result used for timing is first checked against the oracle on a sample of rows.
 
 usage: python bench.py [--gpus 1] [--steps K] [--warmup W]
@@ -59,13 +64,31 @@ def measured_traffic(launch):
         return None
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def percentiles(xs):
+    xs = np.asarray(xs, np.float64)
+    return {"median": round(float(np.median(xs)), 3), "p10": round(float(np.percentile(xs, 10)), 3),
+            "p90": round(float(np.percentile(xs, 90)), 3), "blocks": int(xs.size)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=400)
-    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=400)
     ap.add_argument("--skip-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--skip-recorded", action="store_true", help="skip the replays of recorded messages (HIP graphs)")
+    ap.add_argument("--only-step", action="store_true", help="the headline step only (profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (every box of this pool has one); --gpus %d is not "
@@ -87,9 +110,9 @@ def main():
     for _, n, k in shapes:
         if (n, k) not in uniq:
             uniq[(n, k)] = wl.make_q4_0_weights(rng, n, k)
-    # The data flow of a decoder layer decides which requests may share a launch: q/k/v read the normed hidden
-    # state, o reads the attention output, gate/up read the second normed hidden state, down reads the gated product.
-    # Four distinct activation buffers reproduce that (requests on different buffers are never batched together).
+    # The data flow of a decoder layer: q/k/v read the normed hidden state, o reads the attention output, gate/up
+    # read the second normed hidden state, down reads the gated product. Four distinct activation buffers reproduce
+    # that.
     ACT_OF = {"q": 0, "k": 0, "v": 0, "o": 1, "gate": 2, "up": 2, "down": 3}
     ACT_K = {0: 4096, 1: 4096, 2: 4096, 3: 11008}
     act_q, h_act = {}, {}
@@ -124,6 +147,7 @@ def main():
         msg = layer_message(0, m)
         assert ctx.process_message(msg) == 0
         check_states(msg)
+        submissions = ctx.last_message_submissions()
         worst = 0.0
         for i, (name, n, k) in enumerate(shapes):
             got = ctx.read(h_out[m][i], np.float32, m * n).reshape(m, n)
@@ -132,9 +156,10 @@ def main():
             err = np.abs(got[:, rows] - want) / mag
             worst = max(worst, float(err.max()))
             assert np.all(err <= 1e-5), "matmul %d outside 1e-5 relative: %g" % (i, err.max())
-        return worst
+        return worst, submissions
 
-    log("parity m=1: worst |err|/sum|terms| = %.2e; m=8: %.2e" % (check_layer(1), check_layer(8)))
+    (worst1, subs1), (worst8, subs8) = check_layer(1), check_layer(8)
+    log("parity m=1: worst |err|/sum|terms| = %.2e (%d launch per message); m=8: %.2e (%d launches)" % (worst1, subs1, worst8, subs8))
 
     layer_bytes = {m: sum(wl.matmul_algorithmic_bytes(m, k, n, Q4) for _, n, k in shapes) for m in (1, 8)}
 
@@ -179,29 +204,41 @@ def main():
         return ev_ms / steps
 
     ms_step, wall_step = time_layers(1, args.steps, args.warmup)
-    rec_step = {1: None if args.skip_recorded else time_recorded_layers(1, args.steps, args.warmup)}
     value = layer_bytes[1] / (ms_step * 1e-3) / 1e9
-    log("layer m=1: %.2f us/step (events) %.2f us/step (wall)  %.0f GB/s" % (ms_step * 1e3, wall_step * 1e3, value))
+    log("layer m=1: %.2f us/step (events) %.2f us/step (wall)  %.0f GB/s (%.1f%% of 8 TB/s)" % (
+        ms_step * 1e3, wall_step * 1e3, value, value / 80))
+    if args.only_step:
+        ctx.close()
+        print(json.dumps({"metric": "layer step only", "value": round(value, 1), "unit": "GB/s", "ms_per_step": round(ms_step, 6)}))
+        return
+    block_us = [time_layers(1, 40, LAYERS)[0] * 1e3 for _ in range(20)]
+    step_stats = percentiles(block_us)
+    log("layer m=1 over 20 blocks of 40 steps: median %.2f us  p10 %.2f  p90 %.2f" % (
+        step_stats["median"], step_stats["p10"], step_stats["p90"]))
+    rec_step = {1: None if args.skip_recorded else time_recorded_layers(1, args.steps, args.warmup)}
     if rec_step[1] is not None:
         log("layer m=1 as recorded messages: %.2f us/step" % (rec_step[1] * 1e3))
 
-    # ------------------------------------------------------------------ the step's four launches, one by one
+    # ------------------------------------------------------------------ parts of the step as launches of their own
     def time_single(n, k, m, wt, handles, h_a, h_o, reps, op):
         reqs = [(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, api.mat_mul_params((h_o, 0), (h_a, 0), (h, 0), m, k, n)))
                 for h in handles]
         msg = api.build_message(reqs)
         for _ in range(3):
-            ctx.process_message(msg)
+            ctx.enqueue_message(msg)
+        ctx.synchronize()
         ctx.timer_start()
         for _ in range(reps):
-            ctx.process_message(msg)
+            ctx.enqueue_message(msg)  # (no host wait between messages: the stream stays busy)
         ms = ctx.timer_stop_ms()
+        ctx.finish_message(msg)
         check_states(msg)
         return ms * 1e3 / (reps * len(handles))  # us per launch
 
     def time_launch(names, reps=40):
-        """One message = this launch (the requests `names` of a layer, which share an activation buffer) for every
-        resident layer in turn: LAYERS back-to-back launches on cold weights; HIP events on the launching stream."""
+        """One message = this launch (the requests `names` of a layer) for every resident layer in turn: the requests of
+        different layers write the same outputs, so each layer's group is a launch of its own, LAYERS back-to-back
+        launches on cold weights; HIP events on the launching stream."""
         reqs = []
         for l in range(LAYERS):
             for i, (name, n, k) in enumerate(shapes):
@@ -219,6 +256,7 @@ def main():
         ms = ctx.timer_stop_ms()
         ctx.finish_message(msg)
         check_states(msg)
+        assert ctx.last_message_submissions() == LAYERS, "expected one launch per layer"
         us = ms * 1e3 / (reps * LAYERS)
         nbytes = sum(wl.matmul_algorithmic_bytes(1, k, n, Q4) for name, n, k in shapes if name in names)
         return {"launch": "+".join(names), "us_per_launch": round(us, 3), "bytes_per_launch": nbytes,
@@ -228,29 +266,40 @@ def main():
     for r in launches:
         log("launch %-8s %.2f us  %.0f GB/s (%.1f%% of 8 TB/s)" % (r["launch"], r["us_per_launch"], r["GBps"],
                                                                   r["frac_of_hbm_peak"] * 100))
-    dominant = max(launches, key=lambda r: r["us_per_launch"])  # gate+up: the largest share of the step
     # the same weights again and again: served by the 256 MB memory-side cache, not by HBM
     us_hot = time_single(11008, 4096, 1, Q4, [layers[0][4]] * 16, h_act[(1, 2)], h_out[1][4], 30, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)
     log("gate GEMV 11008x4096 on cache-resident weights: %.2f us" % us_hot)
 
     # ------------------------------------------------------------------ m = 8
     # (every layer is touched before the clock starts: the first few-row use of a weight buffer repacks it once)
-    ms_step8, _ = time_layers(8, max(20, args.steps // 4), LAYERS)
+    ms_step8, _ = time_layers(8, max(20, min(args.steps // 4, 200)), LAYERS)
     log("layer m=8: %.2f us/step  %.0f GB/s" % (ms_step8 * 1e3, layer_bytes[8] / ms_step8 / 1e6))
-    rec_step[8] = None if args.skip_recorded else time_recorded_layers(8, max(20, args.steps // 4), LAYERS)
+    rec_step[8] = None if args.skip_recorded else time_recorded_layers(8, max(20, min(args.steps // 4, 200)), LAYERS)
     if rec_step[8] is not None:
         log("layer m=8 as recorded messages: %.2f us/step" % (rec_step[8] * 1e3))
 
     # ------------------------------------------------------------------ prefill GEMM (config 2)
     prefill = []
     rng2 = wl.rng_for(2, 0)
+    prefill_inputs = {}
     for (n, k) in ((11008, 4096), (4096, 11008)):
         m = 512
         x = wl.make_activations(rng2, m, k)
         aq = ctx.run_quantize_q8_0(x)
+        prefill_inputs[(n, k)] = aq
         ha, ho = ctx.upload(aq), ctx.alloc(m * n * 4)
+        # one-time cost of a weight buffer's first many-row use (converted copy made and kept with the buffer)
+        h_fresh = ctx.upload(uniq[(n, k)])
+        one = api.build_message([(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
+            api.HTP_OPS_MAT_MUL_Q4_0_Q8_0, api.mat_mul_params((ho, 0), (ha, 0), (h_fresh, 0), m, k, n)))])
+        ctx.synchronize()
+        ctx.timer_start()
+        ctx.process_message(one)
+        first_us = ctx.timer_stop_ms() * 1e3
+        ctx.release(h_fresh)
         hw = layers[0][4] if (n, k) == (11008, 4096) else layers[0][6]
-        us = time_single(n, k, m, Q4, [hw] * 8, ha, ho, 5, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)  # 8 launches back to back per message
+        us = time_single(n, k, m, Q4, [hw] * 8, ha, ho, 5, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)  # 8 launches per message share the re-tiled activations
+        us_alone = time_single(n, k, m, Q4, [hw], ha, ho, 20, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)  # re-tiling + one launch
         got = ctx.read(ho, np.float32, m * n).reshape(m, n)
         rows_m = [0, 257, 511]
         cols = np.unique(np.linspace(0, n - 1, 64).astype(int))
@@ -259,8 +308,13 @@ def main():
         tops = 2.0 * m * n * k / us / 1e6
         prefill.append({"m": m, "n": n, "k": k, "us": round(us, 2), "tera_ops": round(tops, 1),
                         "frac_of_int8_nominal": round(tops / INT8_PEAK_TOPS, 4),
+                        "us_with_activation_retiling": round(us_alone, 2),
+                        "activation_retiling_us": round(max(0.0, us_alone - us) * 8 / 7, 2),
+                        "first_use_us_incl_weight_conversion": round(first_us, 1),
+                        "converted_weight_copy_bytes": n * k,
                         "algorithmic_bytes": wl.matmul_algorithmic_bytes(m, k, n, Q4)})
-        log("prefill GEMM m=512 n=%d k=%d: %.1f us  %.1f Tops (%.1f%% of 5 Pop/s)" % (n, k, us, tops, tops / 50))
+        log("prefill GEMM m=512 n=%d k=%d: %.1f us  %.1f Tops (%.1f%% of 5 Pop/s); alone with re-tiling %.1f us; first use %.0f us" % (
+            n, k, us, tops, tops / 50, us_alone, first_us))
         ctx.release(ha), ctx.release(ho)
 
     # ------------------------------------------------------------------ decode chain (config 0)
@@ -296,6 +350,46 @@ def main():
     for h in (h_x0, h_q0, h_o0, h_g0):
         ctx.release(h)
 
+    # ------------------------------------------------------------------ RMSNorm and the Q8_0 quantizer, m x 4096
+    elementwise = []
+    rng5 = wl.rng_for(0, 2)
+    ne0 = 4096
+    for m in (1, 128, 512):
+        x = wl.make_activations(rng5, m, ne0)
+        g = (1.0 + 0.1 * rng5.standard_normal(ne0)).astype(np.float32)
+        hx, hg = ctx.upload(x), ctx.upload(g)
+        hy, hq = ctx.alloc(x.nbytes), ctx.alloc(m * (ne0 // 32) * 34)
+        ops = {
+            "rms_norm": (api.HTP_OPS_RMS_NORM_F32_EX, api.rms_norm_ex_params((hy, 0), (hx, 0), (hg, 0), ne0, m, 1e-6),
+                         2 * x.nbytes + g.nbytes),
+            "quantize_q8_0": (api.HTP_OPS_QUANTIZE_Q8_0, api.rms_norm_params((hq, 0), (hx, 0), ne0, m),
+                              x.nbytes + m * (ne0 // 32) * 34),
+            "rms_norm_quantize_q8_0": (api.HTP_OPS_RMS_NORM_QUANTIZE_Q8_0,
+                                       api.rms_norm_ex_params((hq, 0), (hx, 0), (hg, 0), ne0, m, 1e-6),
+                                       x.nbytes + g.nbytes + m * (ne0 // 32) * 34),
+        }
+        row = {"m": m, "ne0": ne0}
+        for name, (op, body, nbytes) in ops.items():
+            msg = api.build_message([(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, body))] * 50)
+            ctx.process_message(msg)
+            check_states(msg)
+            ctx.timer_start()
+            for _ in range(4):
+                ctx.enqueue_message(msg)
+            us = ctx.timer_stop_ms() * 1e3 / 200
+            ctx.finish_message(msg)
+            row[name] = {"us": round(us, 3), "GBps": round(nbytes / us / 1e3, 1), "bytes": nbytes}
+        # parity of what was timed: quantizer bit-exact, norm within 2e-3
+        assert np.array_equal(ctx.run_quantize_q8_0(x), orc.quantize_q8_0(x)), "Q8_0 quantizer is not bit-exact"
+        got_n = ctx.read(hy, np.float32, m * ne0).reshape(m, ne0)
+        assert np.allclose(got_n, orc.rms_norm(x, g, 1e-6), rtol=2e-3, atol=2e-3), "RMSNorm outside 2e-3"
+        elementwise.append(row)
+        log("m=%d x 4096: rms_norm %.2f us (%.0f GB/s)  quantize %.2f us (%.0f GB/s)  fused %.2f us (%.0f GB/s)" % (
+            m, row["rms_norm"]["us"], row["rms_norm"]["GBps"], row["quantize_q8_0"]["us"], row["quantize_q8_0"]["GBps"],
+            row["rms_norm_quantize_q8_0"]["us"], row["rms_norm_quantize_q8_0"]["GBps"]))
+        for h in (hx, hg, hy, hq):
+            ctx.release(h)
+
     # ------------------------------------------------------------------ Q8_0 block (config 4), m = 1 and m = 128
     # same protocol as the headline step: one message per layer, 8 layers of distinct weights (8 x 49.7 MB) rotated
     rng4 = wl.rng_for(4, 0)
@@ -306,8 +400,11 @@ def main():
             uniq8[(n, k)] = wl.make_q8_0_weights(rng4, n, k)
     layers8 = [[ctx.upload(uniq8[(n, k)]) for _, n, k in shapes8] for _ in range(LAYERS)]
     q8_block = {}
+    act8_m1 = None
     for m8, steps8 in ((1, 200), (128, 40)):
         act8 = {g: ctx.run_quantize_q8_0(wl.make_activations(rng4, m8, k)) for g, k in {0: 1536, 1: 1536, 2: 1536, 3: 8960}.items()}
+        if m8 == 1:
+            act8_m1 = act8
         h_act8 = {g: ctx.upload(a) for g, a in act8.items()}
         h_out8 = [ctx.alloc(m8 * n * 4) for _, n, _ in shapes8]
         msgs8 = [api.build_message([(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
@@ -316,6 +413,7 @@ def main():
             for i, (name, n, k) in enumerate(shapes8)]) for l in range(LAYERS)]
         assert ctx.process_message(msgs8[0]) == 0
         check_states(msgs8[0])
+        subs = ctx.last_message_submissions()
         for i, (name, n, k) in enumerate(shapes8):
             got = ctx.read(h_out8[i], np.float32, m8 * n).reshape(m8, n)
             rows = np.unique(np.linspace(0, n - 1, 64).astype(int))
@@ -335,9 +433,9 @@ def main():
         q8_bytes = sum(wl.matmul_algorithmic_bytes(m8, k, n, Q8) for _, n, k in shapes8)
         q8_ops = sum(2.0 * m8 * k * n for _, n, k in shapes8)
         q8_block[m8] = {"m": m8, "us_per_step": round(q8_us, 2), "GBps": round(q8_bytes / q8_us / 1e3, 1),
-                        "tera_ops": round(q8_ops / q8_us / 1e6, 2)}
-        log("Q8_0 block m=%d: %.1f us/step (7 matmuls), %.0f GB/s, %.1f Tops" % (m8, q8_us, q8_bytes / q8_us / 1e3,
-                                                                               q8_ops / q8_us / 1e6))
+                        "tera_ops": round(q8_ops / q8_us / 1e6, 2), "launches_per_message": subs}
+        log("Q8_0 block m=%d: %.1f us/step (7 matmuls, %d launches), %.0f GB/s, %.1f Tops" % (
+            m8, q8_us, subs, q8_bytes / q8_us / 1e3, q8_ops / q8_us / 1e6))
         for h in h_out8 + list(h_act8.values()):
             ctx.release(h)
     for h in [h for l in layers8 for h in l]:
@@ -347,8 +445,10 @@ def main():
     rng3 = wl.rng_for(3, 0)
     nh, nkv, hd = 32, 8, 128
     attention = []
-    for qo, kv, copies, reps in ((1, 4096, 24, 10), (2048, 2048, 1, 10)):
+    attn_inputs = {}
+    for qo, kv, copies, reps in ((1, 4096, 24, 10), (1, 16384, 8, 10), (2048, 2048, 1, 10)):
         q, kk, vv = wl.make_attention_inputs(rng3, qo, kv, nh, nkv, hd)
+        attn_inputs[(qo, kv)] = (q, kk, vv)
         hq, ho = ctx.upload(q), ctx.alloc(q.nbytes)
         hks, hvs = [ctx.upload(kk) for _ in range(copies)], [ctx.upload(vv) for _ in range(copies)]  # 24 x 16.8 MB: cold
         reqs = [(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
@@ -374,6 +474,7 @@ def main():
         kv_bytes = 2 * kv * nkv * hd * 2
         flops = 4.0 * nh * qo * kv * hd * (0.5 if qo > 1 else 1.0)  # causal: half of the score matrix
         attention.append({"qo_len": qo, "kv_len": kv, "us": round(us, 2), "kv_GBps": round(kv_bytes / us / 1e3, 1),
+                          "frac_of_hbm_peak": round(kv_bytes / us / 1e3 / HBM_PEAK_GBPS, 4),
                           "tera_flops_causal": round(flops / us / 1e6, 2), "max_abs_err_vs_f64": worst})
         log("attention qo=%d kv=%d: %.2f us  KV %.0f GB/s  %.1f TFLOP/s  (max |err| %.1e)" % (
             qo, kv, us, kv_bytes / us / 1e3, flops / us / 1e6, worst))
@@ -381,11 +482,18 @@ def main():
             ctx.release(h)
 
     # ------------------------------------------------------------------ device ceilings
+    read_layer_us = ctx.measure_read_us(layer_bytes[1] // 16 * 16, LAYERS, 10)
+    read_down_us = ctx.measure_read_us(wl.matmul_algorithmic_bytes(1, 11008, 4096, Q4) // 16 * 16, 24, 10)
     peaks = {
         "mfma_i8_32x32x32_tera_ops": round(ctx.measure_mfma_peak(0, 20000), 1),
         "mfma_i8_16x16x64_tera_ops": round(ctx.measure_mfma_peak(1, 20000), 1),
         "mfma_f16_32x32x16_tera_flops": round(ctx.measure_mfma_peak(2, 20000), 1),
         "copy_kernel_GBps_read_plus_write_1GiB": round(ctx.measure_copy_bandwidth(1 << 30, 10), 0),
+        "pure_read_of_the_step_bytes": {"bytes": layer_bytes[1], "us_per_launch": round(read_layer_us, 2),
+                                        "GBps": round(layer_bytes[1] / read_layer_us / 1e3, 0),
+                                        "step_time_over_read_time": round(ms_step * 1e3 / read_layer_us, 3)},
+        "pure_read_of_the_down_gemv_bytes": {"bytes": wl.matmul_algorithmic_bytes(1, 11008, 4096, Q4),
+                                             "us_per_launch": round(read_down_us, 2)},
     }
     log("device ceilings:", peaks)
 
@@ -397,10 +505,11 @@ def main():
         except Exception as e:  # no compiler on this machine: time the portable build
             log("native oracle build failed (%s); timing the portable build" % e)
             native = orc
-        cores = min(os.cpu_count() or 1, 16)
+        nproc = os.cpu_count() or 1
+        cores = min(nproc, 16)
         t0 = time.perf_counter()
         reps = 0
-        while time.perf_counter() - t0 < 10.0:
+        while time.perf_counter() - t0 < 8.0:
             for name, n, k in shapes:
                 native.mat_mul_q8_0_act(act_q[(1, ACT_OF[name])], uniq[(n, k)], 1, k, n, Q4, n_threads=cores)
             reps += 1
@@ -409,13 +518,57 @@ def main():
         for name, n, k in shapes:
             native.mat_mul_q8_0_act(act_q[(1, ACT_OF[name])], uniq[(n, k)], 1, k, n, Q4, n_threads=1)
         t_1 = time.perf_counter() - t0
+
+        def timed(fn, budget_s=2.0):
+            t0 = time.perf_counter()
+            n_ = 0
+            while True:
+                fn()
+                n_ += 1
+                if time.perf_counter() - t0 >= budget_s:
+                    return (time.perf_counter() - t0) / n_
+
+        others = {}
+        # prefill GEMM: 512 rows against a 256-column slice of gate (1/43 of the launch), all threads
+        aq = prefill_inputs[(11008, 4096)]
+        w_slice = np.ascontiguousarray(uniq[(11008, 4096)][:256])
+        t = timed(lambda: native.mat_mul_q8_0_act(aq, w_slice, 512, 4096, 256, Q4, n_threads=cores))
+        others["prefill_gemm_m512_n11008_k4096"] = {
+            "tera_ops": round(2.0 * 512 * 256 * 4096 / t / 1e12, 4), "threads": cores,
+            "sample": "256 of the 11008 weight rows, all 512 activation rows",
+            "us_full_launch_extrapolated": round(t * 11008 / 256 * 1e6, 0)}
+        # Q8_0 block at m = 1, all threads
+        t = timed(lambda: [native.mat_mul_q8_0_act(act8_m1[ACT_OF[name]], uniq8[(n, k)], 1, k, n, Q8, n_threads=cores)
+                           for name, n, k in shapes8])
+        others["q8_0_block_m1"] = {"us_per_step": round(t * 1e6, 1), "threads": cores, "sample": "the whole block"}
+        # attention (single thread: the oracle's attention is not threaded)
+        q1, k1, v1 = attn_inputs[(1, 4096)]
+        t = timed(lambda: native.flash_attn(q1, k1, v1, None, nh, nkv, hd, causal=True))
+        others["attention_decode_kv4096"] = {"us": round(t * 1e6, 1), "threads": 1, "sample": "the whole call"}
+        q2, k2, v2 = attn_inputs[(2048, 2048)]
+        q2s = np.ascontiguousarray(q2[-64:, :4])  # the last 64 query rows of 4 heads (1 KV head)
+        k2s, v2s = np.ascontiguousarray(k2[:, :1]), np.ascontiguousarray(v2[:, :1])
+        mask = wl.make_causal_mask(2048, 2048)[-64:]
+        t = timed(lambda: native.flash_attn(q2s, k2s, v2s, mask, 4, 1, hd, causal=False), 1.0)
+        others["attention_prefill_2048x2048"] = {
+            "us_sample": round(t * 1e6, 1), "threads": 1,
+            "sample": "the last 64 of 2048 query rows (all keys visible) of 4 of 32 heads: 1/256 of the rows x heads, about 1/130 of the causal work"}
+        xn = wl.make_activations(rng5, 512, 4096)
+        gn = np.ones(4096, np.float32)
+        t = timed(lambda: native.rms_norm(xn, gn, 1e-6), 1.0)
+        others["rms_norm_m512_k4096"] = {"us": round(t * 1e6, 1), "GBps": round(2 * xn.nbytes / t / 1e9, 2), "threads": 1,
+                                         "sample": "the whole call"}
+        t = timed(lambda: native.quantize_q8_0(xn), 1.0)
+        others["quantize_q8_0_m512_k4096"] = {"us": round(t * 1e6, 1), "threads": 1, "sample": "the whole call"}
         cpu = {"value": round(layer_bytes[1] / t_mt / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
                "sample": "the same 7-GEMV layer at m=1 with the scalar C oracle (gcc -O3 -march=native, pthreads over output "
-                         "rows), %d passes in ~10 s" % reps,
+                         "rows), %d passes in ~8 s" % reps,
                "us_per_step": round(t_mt * 1e6, 1),
-               "single_thread_GBps": round(layer_bytes[1] / t_1 / 1e9, 3)}
-        log("CPU baseline: %.2f GB/s on %d threads (%.0f us/layer); 1 thread %.3f GB/s" % (
-            cpu["value"], cores, t_mt * 1e6, cpu["single_thread_GBps"]))
+               "single_thread_GBps": round(layer_bytes[1] / t_1 / 1e9, 3),
+               "nproc": nproc, "cpu_model": cpu_model(), "others": others}
+        log("CPU baseline (%s, %d logical CPUs): %.2f GB/s on %d threads (%.0f us/layer); 1 thread %.3f GB/s" % (
+            cpu["cpu_model"], nproc, cpu["value"], cores, t_mt * 1e6, cpu["single_thread_GBps"]))
+        log("CPU baseline, other ops:", others)
 
     result = {
         "metric": "Q4_0 GEMV HBM GB/s (% peak) + M=512 prefill int8 MFMA TOPS, 1 GPU",
@@ -430,14 +583,16 @@ def main():
         "vs_baseline": None,
         "dtype": "i8",
         "data": "synthetic",
-        "config": {"workload": "configs[1]: Llama-7B decode layer, 7 Q4_0xQ8_0 GEMVs at m=1 submitted as one message, "
-                               "%d layers of distinct weights rotated (cold HBM reads)" % LAYERS,
+        "config": {"workload": "configs[1]: Llama-7B decode layer, 7 Q4_0xQ8_0 GEMVs at m=1 submitted as one message "
+                               "(one launch), %d layers of distinct weights rotated (cold HBM reads)" % LAYERS,
                    "algorithmic_bytes_per_step": layer_bytes[1], "pct_of_hbm_peak": round(value / HBM_PEAK_GBPS * 100, 2),
-                   "wall_ms_per_step": round(wall_step, 6)},
-        "roofline": {"bound": "hbm", "achieved": dominant["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": dominant["frac_of_hbm_peak"], "traffic": measured_traffic(dominant["launch"]),
-                     "kernel": "gemv_shared_act_kernel<Q4_0, 64 lanes per row>, grouped launch %s (k=4096, m=1)" % dominant["launch"],
-                     "bytes_per_launch": dominant["bytes_per_launch"], "us_per_launch": dominant["us_per_launch"]},
+                   "wall_ms_per_step": round(wall_step, 6), "launches_per_step": subs1},
+        "roofline": {"bound": "hbm", "achieved": round(value, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(value / HBM_PEAK_GBPS, 4), "traffic": measured_traffic("layer"),
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this script, profiled offline",
+                     "kernel": "gemv_members_kernel<Q4_0>: the seven GEMVs of the layer message in one launch (m=1)",
+                     "bytes_per_launch": layer_bytes[1], "us_per_launch": round(ms_step * 1e3, 3)},
+        "step_us": step_stats,
         "launches": launches,
         "cpu_baseline": cpu,
         "prefill_gemm": prefill,
@@ -446,6 +601,7 @@ def main():
         "recorded_message_us_per_step": None if args.skip_recorded else
         {"m1": round(rec_step[1] * 1e3, 2), "m8": round(rec_step[8] * 1e3, 2)},
         "decode_chain_us": round(chain_us, 2),
+        "elementwise": elementwise,
         "attention": attention,
         "q8_0_block": [q8_block[1], q8_block[128]],
         "peaks": peaks,

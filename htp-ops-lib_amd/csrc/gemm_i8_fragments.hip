@@ -75,13 +75,34 @@ __global__ __launch_bounds__(256) void weights_to_i8_fragments_kernel(uint4 *__r
   }
 }
 
-__global__ __launch_bounds__(256) void act_to_i8_fragments_kernel(uint4 *__restrict__ frag, uint32_t *__restrict__ scales,
-                                                                  const uint16_t *__restrict__ act, int m, int nblk,
-                                                                  int m_tiles) {
-  const size_t t    = (size_t) blockIdx.x * 256 + threadIdx.x;
-  const int    lane = (int) (t & 63);
-  const size_t f    = t >> 6;
-  const int    kb = (int) (f % (size_t) nblk), tile = (int) (f / (size_t) nblk);
+// up to kGemmGroupMax activation matrices of the same row count in one launch
+struct ActMember {
+  uint4          *frag;
+  uint32_t       *scales;
+  const uint16_t *act;
+  int             nblk;
+  unsigned        piece_begin;  // first thread of this member (a multiple of 64)
+};
+struct ActMembers {
+  ActMember m[kGemmGroupMax];
+  int       count;
+};
+
+__global__ __launch_bounds__(256) void act_to_i8_fragments_kernel(ActMembers grp, int m, int m_tiles, unsigned pieces) {
+  const unsigned g = blockIdx.x * 256 + threadIdx.x;
+  if (g >= pieces) {
+    return;
+  }
+  int mi = 0;
+  for (int i = 1; i < grp.count; ++i) {
+    mi = g >= grp.m[i].piece_begin ? i : mi;
+  }
+  const ActMember &mem  = grp.m[mi];
+  const size_t     t    = g - mem.piece_begin;
+  const int        nblk = mem.nblk;
+  const int        lane = (int) (t & 63);
+  const size_t     f    = t >> 6;
+  const int        kb = (int) (f % (size_t) nblk), tile = (int) (f / (size_t) nblk);
   if (tile >= m_tiles) {
     return;
   }
@@ -90,16 +111,16 @@ __global__ __launch_bounds__(256) void act_to_i8_fragments_kernel(uint4 *__restr
   uint32_t  o[4] = { 0, 0, 0, 0 };
   uint32_t  sc   = 0;
   if (row < m) {
-    const uint16_t *blk = act + ((size_t) row * nblk + kb) * 17;
+    const uint16_t *blk = mem.act + ((size_t) row * nblk + kb) * 17;
     sc = blk[0];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       o[i] = (uint32_t) blk[1 + 8 * h + 2 * i] | ((uint32_t) blk[2 + 8 * h + 2 * i] << 16);
     }
   }
-  frag[t] = make_uint4(o[0], o[1], o[2], o[3]);
+  mem.frag[t] = make_uint4(o[0], o[1], o[2], o[3]);
   if (h == 0) {
-    scales[((size_t) tile * nblk + kb) * 32 + c] = sc;
+    mem.scales[((size_t) tile * nblk + kb) * 32 + c] = sc;
   }
 }
 
@@ -123,13 +144,25 @@ struct FragSet {
 
 // KSPLIT waves share one tile of U x U units (each takes every KSPLIT-th block); a workgroup holds 4 / KSPLIT tiles
 // that are neighbours along n (they read the same activation fragments).
+// A launch serves up to kGemmGroupMax matmuls of the same row count ("members"): each has its own operands, n and k,
+// and a range of workgroups that starts at a multiple of 8 (so that the XCD of a workgroup is the same function of
+// its index within the member as in a launch of that member alone).
+struct FragMember {
+  const uint4    *a_frag;
+  const uint32_t *a_scale;
+  const uint4    *b_frag;
+  const uint32_t *b_scale;
+  float          *out;
+  int             n, nblk, n_tiles;
+  unsigned        wg_begin;
+};
+struct FragMembers {
+  FragMember m[kGemmGroupMax];
+  int        count;
+};
+
 template <int KSPLIT, int U>
-__global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__restrict__ out,
-                                                                       const uint4 *__restrict__ a_frag,
-                                                                       const uint32_t *__restrict__ a_scale,
-                                                                       const uint4 *__restrict__ b_frag,
-                                                                       const uint32_t *__restrict__ b_scale, int m, int n,
-                                                                       int nblk, int m_tiles, int n_tiles) {
+__global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembers grp, int m, int m_tiles) {
   // fragment sets in flight per wave: small tiles run one wave per SIMD and must cover the memory latency alone
   constexpr int kGiDepth = U == 1 ? GI_DEPTH_U1 : GI_DEPTH_U2;
   constexpr int TILES = kGiWaves / KSPLIT;
@@ -140,11 +173,21 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(float *__
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int ks = wave % KSPLIT, tw = wave / KSPLIT;
   const int c = lane & 31, h = lane >> 5;
+  int       mi = 0;
+  for (int i = 1; i < grp.count; ++i) {
+    mi = blockIdx.x >= grp.m[i].wg_begin ? i : mi;
+  }
+  const FragMember &mem     = grp.m[mi];
+  float *__restrict__ out   = mem.out;
+  const uint4    *a_frag    = mem.a_frag, *b_frag = mem.b_frag;
+  const uint32_t *a_scale   = mem.a_scale, *b_scale = mem.b_scale;
+  const int       n = mem.n, nblk = mem.nblk, n_tiles = mem.n_tiles;
+  const unsigned  wg = blockIdx.x - mem.wg_begin;
   // tile of this wave, in units of 32: m tiles mt0 .. mt0 + U - 1; n tiles nt0 .. nt0 + U - 1
   // Workgroup ids go round-robin over the 8 XCDs (each with its own L2). All row blocks of one column group are
   // given consecutive slots of ONE XCD, so the weight fragments they share are fetched into that L2 once.
   const int gy = (m_tiles + U - 1) / U, gx = (n_tiles + U * TILES - 1) / (U * TILES);
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int xcd = wg & 7, slot = wg >> 3;
   const int by = slot % gy, bx = (slot / gy) * 8 + xcd;
   if (bx >= gx) {
     return;  // whole workgroup (the grid is padded to a multiple of 8 column groups)
@@ -325,48 +368,122 @@ hipError_t launch_weights_to_i8_fragments(hipStream_t stream, void *dst, const v
   return hipGetLastError();
 }
 
+namespace {
+
+struct TileConfig {
+  int unit, ksplit;
+};
+
+// enough waves for two per SIMD: split K four ways when the tile count alone gives fewer than ~1500 waves; when even
+// that leaves fewer than two workgroups per CU, 32 x 32 tiles
+TileConfig tile_config(int m, int n) {
+  const int m_tiles = (m + 31) / 32, n_tiles = (n + 31) / 32;
+  const int wave_tiles  = ((m_tiles + 1) / 2) * ((n_tiles + 1) / 2);
+  const int forced_unit = env_int("HTPOPS_GEMM_TILE_UNITS", 0);  // read per call: tests run both tile sizes
+  const int unit        = forced_unit == 1 || forced_unit == 2 ? forced_unit : (wave_tiles < 512 ? 1 : 2);
+  return { unit, unit == 1 ? 4 : (wave_tiles * 2 < 1536 ? 4 : 2) };
+}
+
+unsigned member_workgroups(int m_tiles, int n_tiles, TileConfig cfg) {
+  const unsigned tiles_per_wg = kGiWaves / cfg.ksplit;
+  const unsigned gy = (unsigned) ((m_tiles + cfg.unit - 1) / cfg.unit);
+  const unsigned gx = (unsigned) ((n_tiles + cfg.unit * tiles_per_wg - 1) / (cfg.unit * tiles_per_wg));
+  return (gx + 7) / 8 * 8 * gy;
+}
+
+const uint32_t *scales_of(const void *fragments, size_t tiles, size_t nblk) {
+  return reinterpret_cast<const uint32_t *>(static_cast<const uint8_t *>(fragments) + round256(tiles * nblk * 1024));
+}
+
+}  // namespace
+
+bool gemm_i8_fragments_groupable(int m, int n) {
+  return tile_config(m, n).unit == 1;
+}
+
+hipError_t launch_act_to_i8_fragments_group(hipStream_t stream, int count, void *const *act_fragments,
+                                            const void *const *acts_q8_0, const int *ks, int m) {
+  if (count < 1 || count > kGemmGroupMax || m <= 0) {
+    return hipErrorInvalidValue;
+  }
+  const int  m_tiles = (m + 31) / 32;
+  ActMembers grp;
+  size_t     pieces = 0;
+  for (int i = 0; i < count; ++i) {
+    if (ks[i] <= 0 || ks[i] % 32 != 0 || (reinterpret_cast<uintptr_t>(acts_q8_0[i]) & 1) != 0) {
+      return hipErrorInvalidValue;
+    }
+    const int nblk      = ks[i] / 32;
+    grp.m[i].frag        = static_cast<uint4 *>(act_fragments[i]);
+    grp.m[i].scales      = const_cast<uint32_t *>(scales_of(act_fragments[i], (size_t) m_tiles, (size_t) nblk));
+    grp.m[i].act         = static_cast<const uint16_t *>(acts_q8_0[i]);
+    grp.m[i].nblk        = nblk;
+    grp.m[i].piece_begin = (unsigned) pieces;
+    pieces += (size_t) m_tiles * nblk * 64;
+  }
+  if (pieces > 0xffffff00u) {
+    return hipErrorNotSupported;
+  }
+  grp.count = count;
+  hipLaunchKernelGGL(act_to_i8_fragments_kernel, dim3((unsigned) ((pieces + 255) / 256)), dim3(256), 0, stream, grp, m,
+                     m_tiles, (unsigned) pieces);
+  return hipGetLastError();
+}
+
+hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *const *outs,
+                                          const void *const *act_fragments, const void *const *weight_fragments,
+                                          const int *ns, const int *ks, int m) {
+  if (count < 1 || count > kGemmGroupMax || m <= 0) {
+    return hipErrorInvalidValue;
+  }
+  const int   m_tiles = (m + 31) / 32;
+  FragMembers grp;
+  unsigned    total = 0;
+  TileConfig  cfg   = { 0, 0 };
+  for (int i = 0; i < count; ++i) {
+    if (ks[i] <= 0 || ks[i] % 32 != 0 || ns[i] <= 0) {
+      return hipErrorInvalidValue;
+    }
+    const TileConfig c = tile_config(m, ns[i]);
+    if (i > 0 && (c.unit != cfg.unit || c.ksplit != cfg.ksplit)) {
+      return hipErrorNotSupported;  // every member runs in the configuration it would get alone
+    }
+    cfg               = c;
+    const int nblk = ks[i] / 32, n_tiles = (ns[i] + 31) / 32;
+    grp.m[i].a_frag   = static_cast<const uint4 *>(act_fragments[i]);
+    grp.m[i].a_scale  = scales_of(act_fragments[i], (size_t) m_tiles, (size_t) nblk);
+    grp.m[i].b_frag   = static_cast<const uint4 *>(weight_fragments[i]);
+    grp.m[i].b_scale  = scales_of(weight_fragments[i], (size_t) n_tiles, (size_t) nblk);
+    grp.m[i].out      = outs[i];
+    grp.m[i].n        = ns[i];
+    grp.m[i].nblk     = nblk;
+    grp.m[i].n_tiles  = n_tiles;
+    grp.m[i].wg_begin = total;
+    total += member_workgroups(m_tiles, n_tiles, cfg);
+  }
+  grp.count = count;
+  if (cfg.unit == 1) {
+    hipLaunchKernelGGL((gemm_i8_fragments_kernel<4, 1>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
+  } else if (cfg.ksplit == 4) {
+    hipLaunchKernelGGL((gemm_i8_fragments_kernel<4, 2>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
+  } else {
+    hipLaunchKernelGGL((gemm_i8_fragments_kernel<2, 2>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
+  }
+  return hipGetLastError();
+}
+
 hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_fragments,
                                     int m, int k, int n, void *act_fragments, bool act_fragments_ready) {
   if (k % 32 != 0 || m <= 0 || n <= 0) {
     return hipErrorInvalidValue;
   }
-  const int    nblk = k / 32, n_tiles = (n + 31) / 32, m_tiles = (m + 31) / 32;
-  uint4       *af  = static_cast<uint4 *>(act_fragments);
-  uint32_t    *as  = reinterpret_cast<uint32_t *>(static_cast<uint8_t *>(act_fragments) + round256((size_t) m_tiles * nblk * 1024));
-  const uint4 *bf  = static_cast<const uint4 *>(weight_fragments);
-  const uint32_t *bs = reinterpret_cast<const uint32_t *>(static_cast<const uint8_t *>(weight_fragments) +
-                                                          round256((size_t) n_tiles * nblk * 1024));
   if (!act_fragments_ready) {
-    const size_t a_pieces = (size_t) m_tiles * nblk * 64;
-    hipLaunchKernelGGL(act_to_i8_fragments_kernel, dim3((unsigned) ((a_pieces + 255) / 256)), dim3(256), 0, stream, af,
-                       as, static_cast<const uint16_t *>(act_q8_0), m, nblk, m_tiles);
-    if (hipError_t e = hipGetLastError(); e != hipSuccess) {
+    if (hipError_t e = launch_act_to_i8_fragments_group(stream, 1, &act_fragments, &act_q8_0, &k, m); e != hipSuccess) {
       return e;
     }
   }
-  // enough waves for two per SIMD: split K four ways when the tile count alone gives fewer than ~1500 waves; when even
-  // that leaves fewer than two workgroups per CU, 32 x 32 tiles
-  const int    wave_tiles = ((m_tiles + 1) / 2) * ((n_tiles + 1) / 2);
-  static const int forced = env_int("HTPOPS_GEMM_KSPLIT", 0);
-  const int    forced_unit = env_int("HTPOPS_GEMM_TILE_UNITS", 0);  // read per call: tests run both tile sizes
-  const int    unit = forced_unit == 1 || forced_unit == 2 ? forced_unit : (wave_tiles < 512 ? 1 : 2);
-  const int    ksplit = unit == 1 ? 4 : forced ? forced : (wave_tiles * 2 < 1536 ? 4 : 2);
-  const unsigned gy = (unsigned) ((m_tiles + unit - 1) / unit);
-  auto grid = [&](int tiles_per_wg) {
-    const unsigned gx = (unsigned) ((n_tiles + unit * tiles_per_wg - 1) / (unit * tiles_per_wg));
-    return dim3((gx + 7) / 8 * 8 * gy);
-  };
-  if (unit == 1) {
-    hipLaunchKernelGGL((gemm_i8_fragments_kernel<4, 1>), grid(1), dim3(kGiThreads), 0, stream, out, af, as, bf, bs, m, n,
-                       nblk, m_tiles, n_tiles);
-  } else if (ksplit == 4) {
-    hipLaunchKernelGGL((gemm_i8_fragments_kernel<4, 2>), grid(1), dim3(kGiThreads), 0, stream, out, af, as, bf, bs, m, n,
-                       nblk, m_tiles, n_tiles);
-  } else {
-    hipLaunchKernelGGL((gemm_i8_fragments_kernel<2, 2>), grid(2), dim3(kGiThreads), 0, stream, out, af, as, bf, bs, m, n,
-                       nblk, m_tiles, n_tiles);
-  }
-  return hipGetLastError();
+  const void *af = act_fragments;
+  return launch_gemm_i8_fragments_group(stream, 1, &out, &af, &weight_fragments, &n, &k, m);
 }
 
 }  // namespace htpops

@@ -1154,6 +1154,64 @@ struct GemvBatch {
   int                   k[htpops::kGemvGroupMax];
 };
 
+// The many-row members of a batch: converted weights from the cache (made now where missing), the distinct activation
+// matrices converted side by side in the workspace by one launch, then one launch for all the products. Returns a
+// status, or 1 when the members have to be run one by one after all.
+static_assert(htpops::kGemmGroupMax == htpops::kGemvGroupMax, "one batch structure serves both");
+int run_fragment_group(htpops_context *ctx, GemvBatch &b) {
+  const void *wf[htpops::kGemmGroupMax];
+  for (int i = 0; i < b.count; ++i) {
+    MatMulPlan plan = plan_mat_mul(ctx, b.w[i], true, b.m, b.k[i], b.n[i], b.wt);
+    if (plan.kind != kPlanFragments || !(plan.cached || plan.cacheable)) {
+      return 1;  // (a converted copy went away since the member joined: the caller runs the members one by one)
+    }
+    if (!plan.cached) {
+      void *fresh = nullptr;
+      HTPOPS_HIP(ctx, hipMalloc(&fresh, plan.weight_bytes));
+      const hipError_t e = htpops::launch_weights_to_i8_fragments(ctx->stream, fresh, b.w[i], b.k[i], b.n[i], (htpops::WeightType) b.wt);
+      if (e != hipSuccess) {
+        (void) hipFree(fresh);
+        return fail(ctx, HTPOPS_ERR_HIP, "weight conversion: %s", hipGetErrorString(e));
+      }
+      ctx->frag_cache.push_back({ b.w[i], weight_bytes((size_t) b.n[i], (size_t) b.k[i], b.wt), plan.frag_kind, b.k[i], b.n[i], fresh });
+      plan.cached = fresh;
+    }
+    wf[i] = plan.cached;
+  }
+  // distinct (activation, k) pairs and where their conversions go
+  const void *acts[htpops::kGemmGroupMax];
+  int         act_k[htpops::kGemmGroupMax], act_of[htpops::kGemmGroupMax], n_acts = 0;
+  size_t      offset[htpops::kGemmGroupMax], total = 0;
+  for (int i = 0; i < b.count; ++i) {
+    int j = 0;
+    while (j < n_acts && !(acts[j] == b.act[i] && act_k[j] == b.k[i])) {
+      ++j;
+    }
+    if (j == n_acts) {
+      acts[j] = b.act[i], act_k[j] = b.k[i], offset[j] = total;
+      total += (htpops::gemm_i8_act_fragment_bytes(b.m, b.k[i]) + 255) & ~(size_t) 255;
+      ++n_acts;
+    }
+    act_of[i] = j;
+  }
+  if (int r = ensure_workspace(ctx, total)) {
+    return r;
+  }
+  ctx->act_fragments.src = nullptr;
+  uint8_t    *ws = static_cast<uint8_t *>(ctx->workspace);
+  void       *act_dst[htpops::kGemmGroupMax];
+  const void *af[htpops::kGemmGroupMax];
+  for (int j = 0; j < n_acts; ++j) {
+    act_dst[j] = ws + offset[j];
+  }
+  for (int i = 0; i < b.count; ++i) {
+    af[i] = act_dst[act_of[i]];
+  }
+  HTPOPS_HIP(ctx, htpops::launch_act_to_i8_fragments_group(ctx->stream, n_acts, act_dst, acts, act_k, b.m));
+  HTPOPS_HIP(ctx, htpops::launch_gemm_i8_fragments_group(ctx->stream, b.count, b.out, af, wf, b.n, b.k, b.m));
+  return HTPOPS_OK;
+}
+
 void flush_batch(htpops_context *ctx, GemvBatch &b) {
   if (b.count == 0) {
     return;
@@ -1167,7 +1225,11 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
     const int        k0 = b.k[0];
     const void      *a0 = b.act[0];
     hipError_t e;
-    if (b.m == 1) {
+    if (b.m > kBatchMaxM) {
+      ret = run_fragment_group(ctx, b);
+      e   = ret == 1 ? hipErrorNotSupported : hipSuccess;
+      ret = ret == 1 ? HTPOPS_OK : ret;
+    } else if (b.m == 1) {
       e = htpops::launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k, (htpops::WeightType) b.wt);
     } else if (htpops::gemv_rows_fits(b.m, k0, (htpops::WeightType) b.wt)) {
       // 2..4 rows: the decode kernel's weight stream with the rows staged in LDS, whatever n and the weight type
@@ -1235,9 +1297,10 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
     return false;
   }
   const auto *p = reinterpret_cast<const MatMulParams *>(req->payload);
-  if (p->m < 1 || p->m > kBatchMaxM || p->k <= 0 || p->n <= 0 || p->k % 64 != 0) {
-    return false;  // one activation row, or the few rows of the weight-streaming small-batch kernels
+  if (p->m < 1 || p->k <= 0 || p->n <= 0 || p->k % 64 != 0) {
+    return false;
   }
+  // one activation row, the few rows of the weight-streaming small-batch kernels, or many rows on small tiles
   const int    wt        = req->op == HTP_OPS_MAT_MUL_Q4_0_Q8_0 ? htpops::kQ4_0 : htpops::kQ8_0;
   const size_t out_bytes = (size_t) p->m * p->n * 4, act_bytes = q8_0_bytes((size_t) p->m, (size_t) p->k);
   const size_t w_bytes   = weight_bytes((size_t) p->n, (size_t) p->k, wt);
@@ -1248,8 +1311,20 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
       ranges_overlap(out, out_bytes, act, act_bytes) || ranges_overlap(out, out_bytes, w, w_bytes)) {
     return false;  // the ordinary path reports what is wrong, or handles the aliasing in order
   }
+  const bool many_rows = p->m > kBatchMaxM;
+  if (many_rows) {
+    // only matmuls that take the fragment kernel in its small-tile configuration over a converted copy kept with the
+    // weight buffer; everything else runs on its own
+    if (!htpops::gemm_i8_fragments_groupable(p->m, p->n)) {
+      return false;
+    }
+    const MatMulPlan plan = plan_mat_mul(ctx, w, true, p->m, p->k, p->n, wt);
+    if (plan.kind != kPlanFragments || !(plan.cached || plan.cacheable)) {
+      return false;
+    }
+  }
   bool join = b.count > 0 && b.count < htpops::kGemvGroupMax && b.wt == wt && b.m == p->m &&
-              (p->m == 1 || (b.k[0] == p->k && b.act[0] == act));
+              (p->m == 1 || many_rows || (b.k[0] == p->k && b.act[0] == act));
   for (int i = 0; join && i < b.count; ++i) {
     const size_t wi = weight_bytes((size_t) b.n[i], (size_t) b.k[i], b.wt), oi = (size_t) b.m * b.n[i] * 4;
     const size_t ai = q8_0_bytes((size_t) b.m, (size_t) b.k[i]);
@@ -1737,6 +1812,49 @@ extern "C" int htpops_measure_mfma_peak(htpops_context *ctx, int kind, int iters
   const double ops_per_mfma = kind == 0 ? 2.0 * 32 * 32 * 32 : (kind == 1 ? 2.0 * 16 * 16 * 64 : 2.0 * 32 * 32 * 16);
   const double total        = (double) n_blocks * 4 /*waves*/ * (double) iters * 4 /*chains*/ * ops_per_mfma;
   *tera_ops                 = total / ((double) ms * 1e-3) / 1e12;
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_measure_read_us(htpops_context *ctx, size_t bytes, int buffers, int iters, double *us_per_launch) {
+  if (!ctx || !us_per_launch || iters <= 0 || buffers <= 0 || buffers > 64 || bytes < 16) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  std::vector<void *> bufs;
+  unsigned           *sink = nullptr;
+  hipError_t          e    = hipMalloc(reinterpret_cast<void **>(&sink), 256);
+  for (int b = 0; b < buffers && e == hipSuccess; ++b) {
+    void *p = nullptr;
+    e       = hipMalloc(&p, bytes);
+    if (e == hipSuccess) {
+      bufs.push_back(p);
+      e = hipMemsetAsync(p, 1, bytes, ctx->stream);
+    }
+  }
+  float ms = 0.f;
+  for (size_t b = 0; b < bufs.size() && e == hipSuccess; ++b) {
+    e = htpops::launch_read(ctx->stream, bufs[b], bytes, sink);
+  }
+  if (e == hipSuccess) e = hipEventRecord(ctx->ev_start, ctx->stream);
+  for (int i = 0; i < iters && e == hipSuccess; ++i) {
+    for (size_t b = 0; b < bufs.size() && e == hipSuccess; ++b) {
+      e = htpops::launch_read(ctx->stream, bufs[b], bytes, sink);
+    }
+  }
+  if (e == hipSuccess) e = hipEventRecord(ctx->ev_stop, ctx->stream);
+  if (e == hipSuccess) e = hipEventSynchronize(ctx->ev_stop);
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop);
+  (void) hipStreamSynchronize(ctx->stream);
+  for (void *p : bufs) {
+    (void) hipFree(p);
+  }
+  (void) hipFree(sink);
+  if (e != hipSuccess) {
+    return hip_fail(ctx, e, "read loop");
+  }
+  *us_per_launch = (double) ms * 1e3 / ((double) iters * buffers);
   return HTPOPS_OK;
 }
 

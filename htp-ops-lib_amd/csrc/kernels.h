@@ -81,6 +81,18 @@ hipError_t launch_weights_to_i8_fragments(hipStream_t stream, void *dst, const v
                                           WeightType wt);
 hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_fragments,
                                     int m, int k, int n, void *act_fragments, bool act_fragments_ready);
+// The same for up to kGemmGroupMax matmuls of one row count m in one launch each for the conversions and the products:
+// member i multiplies the converted activations act_fragments[i] (gemm_i8_act_fragment_bytes(m, ks[i]) each; members
+// that read the same rows may share one) by weight_fragments[i]. Every member must be `groupable` (the tile
+// configuration it gets depends on (m, n) alone, and a launch has one), else hipErrorNotSupported; a member's result
+// is bit for bit what its own launch gives.
+constexpr int kGemmGroupMax = 8;
+bool       gemm_i8_fragments_groupable(int m, int n);
+hipError_t launch_act_to_i8_fragments_group(hipStream_t stream, int count, void *const *act_fragments,
+                                            const void *const *acts_q8_0, const int *ks, int m);
+hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *const *outs,
+                                          const void *const *act_fragments, const void *const *weight_fragments,
+                                          const int *ns, const int *ks, int m);
 // picks between the one-row and the small-batch kernel by m (any m; many rows are better served by the fragment path)
 size_t     mat_mul_workspace_bytes(int m, int k, int n);
 hipError_t launch_mat_mul_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
@@ -105,6 +117,8 @@ hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const v
 
 // measurement helpers
 hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t bytes);
+// one pass over `bytes` (16-byte multiples) that keeps nothing; `sink` is one device word the kernel never writes in practice
+hipError_t launch_read(hipStream_t stream, const void *src, size_t bytes, unsigned *sink);
 hipError_t launch_mfma_loop(hipStream_t stream, int kind, int iters, int *sink, int n_blocks);
 
 // Tuning override hooks read once from the environment (HTPOPS_GEMV_ROWS etc.); 0 = heuristic.

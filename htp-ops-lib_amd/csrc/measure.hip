@@ -21,6 +21,27 @@ __global__ __launch_bounds__(256) void copy_kernel(uint4 *__restrict__ dst, cons
   }
 }
 
+// Every wave reads 4 KiB once (16 bytes per lane and load, four loads in flight) and keeps nothing: the time of one
+// such launch over a buffer is what any one-pass read of that many bytes costs on this device, launch included.
+__global__ __launch_bounds__(256) void read_kernel(const uint4 *__restrict__ src, size_t n16, unsigned *sink) {
+  const size_t wave = (size_t) blockIdx.x * 4 + (threadIdx.x >> 6);
+  const size_t base = wave * 256 + (threadIdx.x & 63);
+  uint4        v[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const size_t at = base + (size_t) i * 64;
+    v[i]            = src[at < n16 ? at : n16 - 1];
+  }
+  unsigned s = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    s += v[i].x ^ v[i].y ^ v[i].z ^ v[i].w;
+  }
+  if (s == 0x12345678u) {
+    sink[0] = s;  // (never true for the buffers the probe fills; keeps the loads alive)
+  }
+}
+
 // Four independent accumulator chains per wave keep the matrix pipe full.
 template <int KIND>
 __global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, int *sink) {
@@ -73,6 +94,13 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int iters, int *sink) {
 hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t bytes) {
   const size_t n16 = bytes / 16;
   hipLaunchKernelGGL(copy_kernel, dim3(256 * 8), dim3(256), 0, stream, (uint4 *) dst, (const uint4 *) src, n16);
+  return hipGetLastError();
+}
+
+hipError_t launch_read(hipStream_t stream, const void *src, size_t bytes, unsigned *sink) {
+  const size_t n16   = bytes / 16;
+  const size_t waves = (n16 + 255) / 256;
+  hipLaunchKernelGGL(read_kernel, dim3((unsigned) ((waves + 3) / 4)), dim3(256), 0, stream, static_cast<const uint4 *>(src), n16, sink);
   return hipGetLastError();
 }
 

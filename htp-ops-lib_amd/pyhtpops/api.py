@@ -55,7 +55,7 @@ EXPORTED_SYMBOLS = [
     "htpops_mat_mul_permuted_w16a32", "htpops_rms_norm_f32_ex_ptr", "htpops_quantize_q8_0_ptr",
     "htpops_rms_norm_quantize_q8_0_ptr", "htpops_mat_mul_q8_0_act_ptr", "htpops_mat_mul_f32_act_ptr",
     "htpops_flash_attn_ptr", "htpops_flash_attn_noalloc_ptr", "htpops_timer_start", "htpops_timer_stop", "htpops_timer_elapsed_ms",
-    "htpops_measure_mfma_peak", "htpops_measure_copy_bandwidth",
+    "htpops_measure_mfma_peak", "htpops_measure_copy_bandwidth", "htpops_measure_read_us",
 ]
 
 
@@ -110,6 +110,7 @@ def load_library(path=None):
         "htpops_timer_elapsed_ms": (ci, [vp, ctypes.POINTER(ctypes.c_float)]),
         "htpops_measure_mfma_peak": (ci, [vp, ci, ci, ctypes.POINTER(ctypes.c_double)]),
         "htpops_measure_copy_bandwidth": (ci, [vp, sz, ci, ctypes.POINTER(ctypes.c_double)]),
+        "htpops_measure_read_us": (ci, [vp, sz, ci, ci, ctypes.POINTER(ctypes.c_double)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -300,6 +301,11 @@ class Context:
         v = ctypes.c_double()
         self._check(self.lib.htpops_measure_mfma_peak(self._ctx, kind, iters, ctypes.byref(v)))
         return float(v.value)
+
+    def measure_read_us(self, nbytes, buffers, iters=10):
+        v = ctypes.c_double()
+        self._check(self.lib.htpops_measure_read_us(self._ctx, int(nbytes), buffers, iters, ctypes.byref(v)))
+        return v.value
 
     def measure_copy_bandwidth(self, nbytes, iters=20):
         v = ctypes.c_double()

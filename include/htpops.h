@@ -213,6 +213,11 @@ int htpops_measure_mfma_peak(htpops_context *ctx, int kind, int iters, double *t
  * measure the attainable copy bandwidth; reports bytes read + written per second in GB/s. */
 int htpops_measure_copy_bandwidth(htpops_context *ctx, size_t bytes, int iters, double *gbps);
 
+/* Time of one launch that reads `bytes` once and keeps nothing (every wave 4 KiB, 16 bytes per lane and load), averaged
+ * over `iters` rounds over `buffers` distinct buffers of that size read in turn (buffers x bytes beyond the 256 MB
+ * memory-side cache = every launch reads HBM). The floor under any one-launch weight stream of that size. */
+int htpops_measure_read_us(htpops_context *ctx, size_t bytes, int buffers, int iters, double *us_per_launch);
+
 #ifdef __cplusplus
 }
 #endif

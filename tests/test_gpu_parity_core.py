@@ -681,6 +681,48 @@ def test_message_groups_independent_gemvs_of_different_activations(ctx, oracle, 
             ctx.release(h)
 
 
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+def test_message_groups_independent_many_row_matmuls(ctx, oracle, wt):
+    # Many-row matmuls on small output tiles (the projections of a small model at a prefill chunk of 128 rows) share
+    # one launch for the products and one for the activation conversions when nothing orders them; members read
+    # different activation matrices with different k. Every request must equal its own launch bit for bit. A request
+    # that writes what an earlier one reads ends the group.
+    rng = wl.rng_for(75, wt)
+    op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
+    m = 100
+    shapes = [(192, 1536), (64, 1536), (40, 1536), (192, 1536), (1120, 1536), (1120, 1536), (192, 8960)]   # (n, k)
+    act_of = [0, 0, 0, 1, 2, 2, 3]
+    act_k = [1536, 1536, 1536, 8960]
+    ws = [wl.make_weights(rng, n, k, wt) for n, k in shapes]
+    acts = [oracle.quantize_q8_0(wl.make_activations(rng, m, k)) for k in act_k]
+    has = [ctx.upload(a) for a in acts]
+    hws = [ctx.upload(w) for w in ws]
+    hos = [ctx.alloc(m * n * 4) for n, _ in shapes]
+    try:
+        reqs = [_mm(op, ho, has[g], hw, m, k, n) for ho, g, hw, (n, k) in zip(hos, act_of, hws, shapes)]
+        msg = api.build_message(reqs)
+        for _ in range(2):
+            for ho, (n, _) in zip(hos, shapes):
+                ctx.write(ho, np.full(m * n, np.nan, np.float32))
+            assert ctx.process_message(msg) == 0
+            assert api.message_request_states(msg) == [0] * len(shapes), ctx.last_error()
+            assert ctx.last_message_submissions() == 1
+            for ho, g, w, (n, k) in zip(hos, act_of, ws, shapes):
+                got = ctx.read(ho, np.float32, m * n).reshape(m, n)
+                assert np.array_equal(got, ctx.run_mat_mul(acts[g], w, m, k, n, wt)), "a request differs from its own launch"
+                want, mag = oracle.mat_mul_q8_0_act_f64(acts[g], w, m, k, n, wt)
+                assert np.all(np.abs(got - want) <= MATMUL_RTOL * mag)
+        # the same output twice: two launches, the later request wins
+        msg2 = api.build_message([_mm(op, hos[0], has[0], hws[0], m, 1536, 192), _mm(op, hos[0], has[1], hws[3], m, 1536, 192)])
+        assert ctx.process_message(msg2) == 0
+        assert ctx.last_message_submissions() == 2
+        assert np.array_equal(ctx.read(hos[0], np.float32, m * 192).reshape(m, 192),
+                              ctx.run_mat_mul(acts[1], ws[3], m, 1536, 192, wt))
+    finally:
+        for h in has + hws + hos:
+            ctx.release(h)
+
+
 def test_message_keeps_dependent_gemvs_in_order(ctx, oracle):
     # Requests with a data dependency must not share a launch. (1) read-after-write: request 1's fp32 output bytes are
     # request 2's Q8_0 activation row (unit scales and small integers make those bytes finite Q8_0 blocks);
