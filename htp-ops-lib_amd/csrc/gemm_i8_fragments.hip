@@ -32,7 +32,9 @@ typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 
 // ---- operand conversion -------------------------------------------------------------------------------------------
 // fragment (tile, block): lane (c = lane % 32, h = lane / 32) holds elements 16 h .. 16 h + 15 of block `block` of row
-// 32 tile + c; the scale array holds one dword (fp16 scale, 0) per row and block: [tile][block][32].
+// 32 tile + c; the scale array holds one dword (fp16 scale, 0) per row and block: weights [tile][block][32],
+// activations [tile][block][64] with zeros in the upper 32 (the operand of the scale product as it is loaded), followed
+// by one row of 64 zeros.
 
 template <int WT>
 __global__ __launch_bounds__(256) void weights_to_i8_fragments_kernel(uint4 *__restrict__ frag, uint32_t *__restrict__ scales,
@@ -119,8 +121,10 @@ __global__ __launch_bounds__(256) void act_to_i8_fragments_kernel(ActMembers grp
     }
   }
   mem.frag[t] = make_uint4(o[0], o[1], o[2], o[3]);
-  if (h == 0) {
-    mem.scales[((size_t) tile * nblk + kb) * 32 + c] = sc;
+  // scale rows of 64 dwords: lanes 32..63 of the scale-product instruction hold K slots that must contribute nothing
+  mem.scales[((size_t) tile * nblk + kb) * 64 + lane] = h == 0 ? sc : 0u;
+  if (t < 64) {
+    mem.scales[(size_t) m_tiles * nblk * 64 + t] = 0u;  // the row that blocks past the end of K are pointed at
   }
 }
 
@@ -129,7 +133,7 @@ __global__ __launch_bounds__(256) void act_to_i8_fragments_kernel(ActMembers grp
 constexpr int kGiThreads = 256;
 constexpr int kGiWaves   = 4;
 #ifndef GI_DEPTH_U1
-#define GI_DEPTH_U1 6
+#define GI_DEPTH_U1 4
 #endif
 #ifndef GI_DEPTH_U2
 #define GI_DEPTH_U2 2
@@ -139,7 +143,6 @@ template <int U>
 struct FragSet {
   uint4    a[U], b[U];
   uint32_t da[U], dw[U];
-  uint32_t live;  // all ones, or zero for a block past the end of K (wave-uniform)
 };
 
 // KSPLIT waves share one tile of U x U units (each takes every KSPLIT-th block); a workgroup holds 4 / KSPLIT tiles
@@ -154,6 +157,7 @@ struct FragMember {
   const uint32_t *b_scale;
   float          *out;
   int             n, nblk, n_tiles;
+  int             ksplit;  // waves that share a tile's K (used by the instantiation that takes it at run time)
   unsigned        wg_begin;
 };
 struct FragMembers {
@@ -161,23 +165,26 @@ struct FragMembers {
   int        count;
 };
 
-template <int KSPLIT, int U>
+// KSPLIT_T = 0: the split is the member's own (1, 2 or 4), so that members with short and long K share a launch.
+template <int KSPLIT_T, int U>
 __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembers grp, int m, int m_tiles) {
   // fragment sets in flight per wave: small tiles run one wave per SIMD and must cover the memory latency alone
   constexpr int kGiDepth = U == 1 ? GI_DEPTH_U1 : GI_DEPTH_U2;
-  constexpr int TILES = kGiWaves / KSPLIT;
-  __shared__ float red[TILES][KSPLIT - 1][U * U][16][64];  // partial accumulators of the waves with ks > 0
+  constexpr int kRedSlots = KSPLIT_T ? (kGiWaves / KSPLIT_T) * (KSPLIT_T - 1) : kGiWaves - 1;
+  __shared__ float red[kRedSlots][U * U][16][64];  // partial accumulators of the waves with ks > 0
 
   // the wave index (and everything derived from it) is made scalar so that fragment addresses are scalar base +
   // per-lane offset and cost no vector instructions in the loop
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int ks = wave % KSPLIT, tw = wave / KSPLIT;
   const int c = lane & 31, h = lane >> 5;
   int       mi = 0;
   for (int i = 1; i < grp.count; ++i) {
     mi = blockIdx.x >= grp.m[i].wg_begin ? i : mi;
   }
   const FragMember &mem     = grp.m[mi];
+  const int         KSPLIT  = KSPLIT_T ? KSPLIT_T : mem.ksplit;
+  const int         TILES   = kGiWaves / KSPLIT;
+  const int         ks = wave % KSPLIT, tw = wave / KSPLIT;
   float *__restrict__ out   = mem.out;
   const uint4    *a_frag    = mem.a_frag, *b_frag = mem.b_frag;
   const uint32_t *a_scale   = mem.a_scale, *b_scale = mem.b_scale;
@@ -195,27 +202,33 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
   const int mt0 = by * U, nt0 = (bx * TILES + tw) * U;
   const bool tile_ok = nt0 < n_tiles;  // mt0 < m_tiles by construction
 
-  const uint4    *ap[U], *bp[U];
-  const uint32_t *asp[U], *bsp[U];
+  // Operand streams as buffer resources: a load is then resource (scalar) + per-lane offset (a register that never
+  // changes) + scalar offset of the block, and costs no vector-ALU instruction.
+  typedef unsigned v4u __attribute__((ext_vector_type(4)));
+  auto resource = [](const void *base) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int) 0xffffffffu, 0x00020000);
+  };
+  __amdgpu_buffer_rsrc_t ra[U], rb[U], rsa[U], rsb[U];
+  int                    zero_row[U];  // byte offset of the row of zero scales from this tile's scale rows
 #pragma unroll
   for (int i = 0; i < U; ++i) {
     const size_t mt = (size_t) min(mt0 + i, m_tiles - 1), nt = (size_t) min(nt0 + i, n_tiles - 1);
-    ap[i]  = a_frag + mt * nblk * 64;
-    bp[i]  = b_frag + nt * nblk * 64;
-    asp[i] = a_scale + mt * nblk * 32;
-    bsp[i] = b_scale + nt * nblk * 32;
+    ra[i]       = resource(a_frag + mt * nblk * 64);
+    rb[i]       = resource(b_frag + nt * nblk * 64);
+    rsa[i]      = resource(a_scale + mt * nblk * 64);
+    rsb[i]      = resource(b_scale + nt * nblk * 32);
+    zero_row[i] = (int) (((size_t) m_tiles - mt) * nblk * 256);
   }
+  const int lane16 = lane * 16, lane4 = lane * 4, c4 = c * 4;
   auto load = [&](FragSet<U> &s, int kb_raw) {
-    const size_t kb = (size_t) min(kb_raw, nblk - 1);  // branch-free: blocks past the end repeat the last one ...
-    // ... with activation scales of zero: they add nothing. The mask is applied where the scale is used, not here: an
-    // instruction on a freshly loaded register here would make the wave wait for the loads it has just issued.
-    s.live = kb_raw < nblk ? 0xffffffffu : 0u;
+    const int  kb   = min(kb_raw, nblk - 1);  // branch-free: blocks past the end repeat the last one ...
+    const bool live = kb_raw < nblk;          // ... with activation scales of zero: they add nothing
 #pragma unroll
     for (int i = 0; i < U; ++i) {
-      s.a[i]  = (ap[i] + kb * 64)[lane];
-      s.b[i]  = (bp[i] + kb * 64)[lane];
-      s.da[i] = (asp[i] + kb * 32)[c];
-      s.dw[i] = (bsp[i] + kb * 32)[c];
+      s.a[i]  = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ra[i], lane16, kb * 1024, 0));
+      s.b[i]  = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb[i], lane16, kb * 1024, 0));
+      s.da[i] = __builtin_amdgcn_raw_buffer_load_b32(rsa[i], lane4, live ? kb * 256 : zero_row[i], 0);
+      s.dw[i] = __builtin_amdgcn_raw_buffer_load_b32(rsb[i], c4, kb * 128, 0);
     }
   };
 
@@ -238,9 +251,10 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
   }
   const v16f zf = { 0 };
   const v16i zi = { 0 };
-  // scale operands of a unit: (scale, 0, 0, 0) in the lanes of K slots 0..3, zeros in the other lane half
+  // scale operands of a unit: (scale, 0, 0, 0) in K slot 0; the activation side holds zeros in the lanes of K slots
+  // 4..7, so whatever the weight side holds there contributes nothing
   auto scale_operand = [&](uint32_t packed) {
-    const uint2 u = make_uint2(h == 0 ? packed : 0u, 0u);
+    const uint2 u = make_uint2(packed, 0u);
     return __builtin_bit_cast(v4h, u);
   };
   auto mfma_sum = [&](const FragSet<U> &s, int i, int j) {
@@ -249,7 +263,7 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, zi, 0, 0, 0);
   };
   auto mfma_scale = [&](const FragSet<U> &s, int i, int j) {
-    return __builtin_amdgcn_mfma_f32_32x32x8f16(scale_operand(s.da[i] & s.live), scale_operand(s.dw[j]), zf, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x8f16(scale_operand(s.da[i]), scale_operand(s.dw[j]), zf, 0, 0, 0);
   };
 
   // Software pipeline over units (block, i, j): the two matrix instructions of the NEXT unit are issued between the
@@ -299,7 +313,7 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
       for (int j = 0; j < U; ++j) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          red[tw][ks - 1][i * U + j][r][lane] = acc[i][j][r];
+          red[tw * (KSPLIT - 1) + ks - 1][i * U + j][r][lane] = acc[i][j][r];
         }
       }
     }
@@ -315,9 +329,8 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             float v = acc[i][j][r];
-#pragma unroll
             for (int s = 0; s < KSPLIT - 1; ++s) {
-              v += red[tw][s][i * U + j][r][lane];
+              v += red[tw * (KSPLIT - 1) + s][i * U + j][r][lane];
             }
             // D[row][col]: col = lane % 32, row = 8 (r / 4) + 4 (lane / 32) + r % 4
             const int row = (mt0 + i) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
@@ -345,7 +358,7 @@ size_t gemm_i8_weight_fragment_bytes(int k, int n) {
 
 size_t gemm_i8_act_fragment_bytes(int m, int k) {
   const size_t m_tiles = ((size_t) m + 31) / 32, nblk = (size_t) k / 32;
-  return round256(m_tiles * nblk * 1024) + m_tiles * nblk * 128;
+  return round256(m_tiles * nblk * 1024) + m_tiles * nblk * 256 + 256;
 }
 
 hipError_t launch_weights_to_i8_fragments(hipStream_t stream, void *dst, const void *weight, int k, int n,
@@ -376,12 +389,18 @@ struct TileConfig {
 
 // enough waves for two per SIMD: split K four ways when the tile count alone gives fewer than ~1500 waves; when even
 // that leaves fewer than two workgroups per CU, 32 x 32 tiles
-TileConfig tile_config(int m, int n) {
-  const int m_tiles = (m + 31) / 32, n_tiles = (n + 31) / 32;
+// With 32 x 32 tiles the split follows K alone: a wave should have some 48 blocks or more to work through (its ring of
+// loads and its epilogue are paid once), so short K is not split at all and the four waves of a workgroup take four
+// neighbouring column tiles instead.
+TileConfig tile_config(int m, int n, int k) {
+  const int m_tiles = (m + 31) / 32, n_tiles = (n + 31) / 32, nblk = k / 32;
   const int wave_tiles  = ((m_tiles + 1) / 2) * ((n_tiles + 1) / 2);
   const int forced_unit = env_int("HTPOPS_GEMM_TILE_UNITS", 0);  // read per call: tests run both tile sizes
   const int unit        = forced_unit == 1 || forced_unit == 2 ? forced_unit : (wave_tiles < 512 ? 1 : 2);
-  return { unit, unit == 1 ? 4 : (wave_tiles * 2 < 1536 ? 4 : 2) };
+  if (unit == 1) {
+    return { 1, nblk >= 192 ? 4 : nblk >= 96 ? 2 : 1 };
+  }
+  return { 2, wave_tiles * 2 < 1536 ? 4 : 2 };
 }
 
 unsigned member_workgroups(int m_tiles, int n_tiles, TileConfig cfg) {
@@ -398,7 +417,7 @@ const uint32_t *scales_of(const void *fragments, size_t tiles, size_t nblk) {
 }  // namespace
 
 bool gemm_i8_fragments_groupable(int m, int n) {
-  return tile_config(m, n).unit == 1;
+  return tile_config(m, n, 32).unit == 1;
 }
 
 hipError_t launch_act_to_i8_fragments_group(hipStream_t stream, int count, void *const *act_fragments,
@@ -444,8 +463,8 @@ hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *
     if (ks[i] <= 0 || ks[i] % 32 != 0 || ns[i] <= 0) {
       return hipErrorInvalidValue;
     }
-    const TileConfig c = tile_config(m, ns[i]);
-    if (i > 0 && (c.unit != cfg.unit || c.ksplit != cfg.ksplit)) {
+    const TileConfig c = tile_config(m, ns[i], ks[i]);
+    if (i > 0 && (c.unit != cfg.unit || (c.unit != 1 && c.ksplit != cfg.ksplit))) {
       return hipErrorNotSupported;  // every member runs in the configuration it would get alone
     }
     cfg               = c;
@@ -458,12 +477,13 @@ hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *
     grp.m[i].n        = ns[i];
     grp.m[i].nblk     = nblk;
     grp.m[i].n_tiles  = n_tiles;
+    grp.m[i].ksplit   = c.ksplit;
     grp.m[i].wg_begin = total;
     total += member_workgroups(m_tiles, n_tiles, cfg);
   }
   grp.count = count;
   if (cfg.unit == 1) {
-    hipLaunchKernelGGL((gemm_i8_fragments_kernel<4, 1>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
+    hipLaunchKernelGGL((gemm_i8_fragments_kernel<0, 1>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
   } else if (cfg.ksplit == 4) {
     hipLaunchKernelGGL((gemm_i8_fragments_kernel<4, 2>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
   } else {
