@@ -486,13 +486,9 @@ hipError_t launch_gemm_fp6_lds(hipStream_t stream, float *out, const void *act_q
   // A K group is 4 waves and one LDS ring, and a compute unit holds three rings: one group per workgroup when the
   // tiles alone give every compute unit three workgroups, otherwise up to three groups per workgroup, each with its
   // share of K, so that the same tiles put more waves on a compute unit.
-  static const int forced_ks = env_int("HTPOPS_GEMM_KGROUPS", 0);
   const long       out_tiles = (long) ((m + kBM - 1) / kBM) * ((n + kBN - 1) / kBN);
   int              ks        = out_tiles >= 640 ? 1 : out_tiles >= 384 ? 2 : 3;
   ks                         = std::max(1, std::min(ks, pairs / 4));
-  if (forced_ks >= 1 && forced_ks <= 3) {
-    ks = forced_ks;
-  }
   const uint8_t *wt = static_cast<const uint8_t *>(weight_tiles);
   switch (ks) {
     case 1:

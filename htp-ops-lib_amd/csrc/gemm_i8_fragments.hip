@@ -204,7 +204,6 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
 
   // Operand streams as buffer resources: a load is then resource (scalar) + per-lane offset (a register that never
   // changes) + scalar offset of the block, and costs no vector-ALU instruction.
-  typedef unsigned v4u __attribute__((ext_vector_type(4)));
   auto resource = [](const void *base) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int) 0xffffffffu, 0x00020000);
   };

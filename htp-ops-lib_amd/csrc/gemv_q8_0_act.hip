@@ -488,8 +488,6 @@ __global__ __launch_bounds__(THREADS) void gemv_members_kernel(int b1, int b2, i
 // Fills shape, r and block0 of every member and launches.
 template <int WT>
 hipError_t launch_gemv_members(hipStream_t stream, GemvMembers &grp) {
-  static const int forced_r       = env_int("HTPOPS_GEMV_ROWS", 0);
-  static const int forced_threads = env_int("HTPOPS_GEMV_THREADS", 0);
   // measured on MI355X: short-lived waves (one row set each) stream best; only very wide launches of short rows
   // (gate + up of a 7B layer: 22016 rows of 64 pairs) gain from two rows per lane group
   long total_short_rows = 0;
@@ -525,19 +523,10 @@ hipError_t launch_gemv_members(hipStream_t stream, GemvMembers &grp) {
     }
     mem.shape = p <= 16 ? kShapeG16 : p <= 32 ? kShapeG32 : p <= 64 ? kShapeG64 : p <= 128 ? kShapeG64x2 : kShapeG64x2S2;
     mem.r     = (p <= 64 && total_short_rows >= 16384) ? 2 : 1;
-    if (forced_r == 1 || forced_r == 2) {
-      mem.r = forced_r;
-    }
-    if (p > 64) {
-      mem.r = 1;
-    }
     max_pairs = p > max_pairs ? p : max_pairs;
     any_long  = any_long || p > 64;
   }
-  int threads = place(512, false) >= 1024 ? 512 : kThreads;
-  if (forced_threads == 256 || forced_threads == 512) {
-    threads = forced_threads;
-  }
+  const int threads = place(512, false) >= 1024 ? 512 : kThreads;
   const int blocks = place(threads, true);
   // the table stride of the widest body among the members (see TS in gemv_row_sets)
   const int    table_pairs = max_pairs <= 16 ? 16 : max_pairs <= 32 ? 32 : max_pairs <= 64 ? 64 : max_pairs <= 128 ? 128 : kSharedActMaxPairs;

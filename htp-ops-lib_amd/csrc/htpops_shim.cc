@@ -133,6 +133,7 @@ int fail(htpops_context *ctx, int code, const char *fmt, ...) {
 }
 
 int hip_fail(htpops_context *ctx, hipError_t e, const char *what) {
+  (void) hipGetLastError();  // the runtime keeps the error for the next caller that asks: it is reported here, once
   return fail(ctx, HTPOPS_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
@@ -420,6 +421,7 @@ bool in_owned_buffer(htpops_context *ctx, const void *ptr, size_t bytes) {
 
 constexpr int kSkinnyGroupMaxM = 8;   // rows of the K-sliced kernel's grouped launch
 constexpr int kBatchMaxM       = 16;  // rows up to which same-activation requests of a message are grouped
+constexpr int kManyRowsMinM    = 33;  // rows from which a matmul takes the matrix-core kernels
 
 bool ranges_overlap(const void *a, size_t a_bytes, const void *b, size_t b_bytes) {
   const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
@@ -483,9 +485,8 @@ struct MatMulPlan {
 
 // `act_aligned`: the Q8_0 activations start on a 4-byte boundary (the re-tiling pass of the FP6 kernel reads dwords)
 MatMulPlan plan_mat_mul(htpops_context *ctx, const void *weight, bool act_aligned, int m, int k, int n, int wt) {
-  static const int frag_min_m = htpops::env_int("HTPOPS_GEMM_FRAG_MIN_M", 33);
-  MatMulPlan       p;
-  if (m < frag_min_m || k % 32 != 0) {
+  MatMulPlan p;
+  if (m < kManyRowsMinM || k % 32 != 0) {
     p.ws_bytes = htpops::mat_mul_workspace_bytes(m, k, n);
     return p;
   }
@@ -1291,8 +1292,7 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
 
 // true: the request is now part of the batch and its state is set; false: run it the ordinary way (after a flush)
 bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct RequestHeader *hdr, GemvBatch &b) {
-  static const int enabled = htpops::env_int("HTPOPS_BATCH_GEMV", 1);
-  if (!enabled || !ctx->has_device ||
+  if (!ctx->has_device ||
       (req->op != HTP_OPS_MAT_MUL_Q4_0_Q8_0 && req->op != HTP_OPS_MAT_MUL_Q8_0_Q8_0)) {
     return false;
   }

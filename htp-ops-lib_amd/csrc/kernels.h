@@ -121,7 +121,7 @@ hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t by
 hipError_t launch_read(hipStream_t stream, const void *src, size_t bytes, unsigned *sink);
 hipError_t launch_mfma_loop(hipStream_t stream, int kind, int iters, int *sink, int n_blocks);
 
-// Tuning override hooks read once from the environment (HTPOPS_GEMV_ROWS etc.); 0 = heuristic.
+// Integer value of an environment switch (the few there are select a kernel for tests and A/B measurements).
 int env_int(const char *name, int fallback);
 
 }  // namespace htpops

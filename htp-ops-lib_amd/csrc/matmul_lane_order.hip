@@ -378,8 +378,8 @@ hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *
   for (int i = 0; i < count; ++i) {
     pairs += (ns[i] / kLoRows + 1) / 2;
   }
-  const int    forced = env_int("HTPOPS_LANE_ORDER_TILES", 0);  // read per call: tests run both
-  const int    tpw    = forced == 1 || forced == 2 ? forced : (pairs >= 512 ? 2 : 1);
+  const int    forced = env_int("HTPOPS_LANE_ORDER", 1);  // 2 / 3: one / two tiles per workgroup (read per call: tests run both)
+  const int    tpw    = forced == 2 || forced == 3 ? forced - 1 : (pairs >= 512 ? 2 : 1);
   const dim3   grid((unsigned) ((n_max / kLoRows + tpw - 1) / tpw), (unsigned) count);
   const int    rows = panel_rows(m);
   const size_t lds  = panel_bytes(k, rows);

@@ -525,10 +525,9 @@ template <WeightType WT, int MR>
 hipError_t launch_skinny(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k, int n,
                          void *workspace, unsigned *tickets, int ticket_slots) {
   const int nblk = k / 32;
-  static const int use_slices = env_int("HTPOPS_SKINNY_SLICES", 1);
   SkinnyGroupArgs  one = {};
   one.w[0] = static_cast<const uint8_t *>(weight), one.out[0] = out, one.n[0] = n, one.tile0[0] = 0;
-  if (use_slices && slices_fit<WT>(one, 1, k, workspace, tickets, ticket_slots)) {
+  if (slices_fit<WT>(one, 1, k, workspace, tickets, ticket_slots)) {
     return launch_skinny_slices<WT, MR>(stream, one, 1, act, m, k, workspace, tickets);
   }
   constexpr int per_kb = ActChunk<MR>::PER_KB;

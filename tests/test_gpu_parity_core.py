@@ -438,14 +438,13 @@ def test_few_rows_over_repacked_weights(ctx, oracle, monkeypatch, wt, m, k, n):
     a = oracle.quantize_q8_0(x)
     assert np.array_equal(ctx.run_mat_mul(a, w, m, k, n, wt), got)
     _, mag = oracle.mat_mul_q8_0_act_f64(a, w, m, k, n, wt)
-    # one and two weight tiles per workgroup (the launcher picks by the number of tiles) sum the same blocks in
-    # different wave order
-    for tiles in ("1", "2"):
-        monkeypatch.setenv("HTPOPS_LANE_ORDER_TILES", tiles)
+    # one and two weight tiles per workgroup (the launcher picks by the number of tiles; HTPOPS_LANE_ORDER=2 / 3 force
+    # one / two) sum the same blocks in different wave order
+    for tiles in ("2", "3"):
+        monkeypatch.setenv("HTPOPS_LANE_ORDER", tiles)
         forced = ctx.run_mat_mul(a, w, m, k, n, wt)
         assert np.all(np.abs(forced - got) <= 2 * MATMUL_RTOL * mag)
         assert np.array_equal(forced, ctx.run_mat_mul(a, w, m, k, n, wt))
-    monkeypatch.delenv("HTPOPS_LANE_ORDER_TILES")
     monkeypatch.setenv("HTPOPS_LANE_ORDER", "0")
     plain = ctx.run_mat_mul(a, w, m, k, n, wt)
     assert np.all(np.abs(plain - got) <= 2 * MATMUL_RTOL * mag)
@@ -776,3 +775,24 @@ def test_message_keeps_dependent_gemvs_in_order(ctx, oracle):
     finally:
         for v in h.values():
             ctx.release(v)
+
+
+def test_a_failed_device_allocation_is_reported_and_the_context_stays_usable(ctx, oracle):
+    # Split-KV partials of a decode attention over 2^31 - 64 keys and 4096 heads would need some 70 TB of workspace:
+    # the allocation fails before anything is launched, the call returns HTPOPS_ERR_HIP with the runtime's message,
+    # and the error is not left behind for the next op to trip over.
+    h = ctx.alloc(4096)
+    try:
+        p = ctx.device_ptr(h)
+        ret = ctx.lib.htpops_flash_attn_ptr(ctx._ctx, p, p, p, p, None, 1, 2**31 - 64, 4096, 4096, 128, 0, 1)
+        assert ret == api.HTPOPS_ERR_HIP, ret
+        assert "hipMalloc" in ctx.last_error(), ctx.last_error()
+        x = wl.make_activations(wl.rng_for(76, 0), 3, 256)
+        assert np.array_equal(ctx.run_quantize_q8_0(x), oracle.quantize_q8_0(x))
+        w = wl.make_q4_0_weights(wl.rng_for(76, 1), 48, 256)
+        a = oracle.quantize_q8_0(x)
+        got = ctx.run_mat_mul(a, w, 3, 256, 48, wl.GGML_TYPE_Q4_0)
+        want, mag = oracle.mat_mul_q8_0_act_f64(a, w, 3, 256, 48, wl.GGML_TYPE_Q4_0)
+        assert np.all(np.abs(got - want) <= MATMUL_RTOL * mag)
+    finally:
+        ctx.release(h)
