@@ -20,11 +20,13 @@
 // straight into LDS and ds_read into operand registers, with no data shuffling and no vector-ALU work:
 //   weights      converted once per weight buffer (1 byte per weight incl. scales) and cached by the caller
 //   activations  converted per call from block_q8_0 rows; shared by the matmuls of a message that read the same rows
-// A workgroup owns 128 x 64 outputs over all of K (no exchange between workgroups, results independent of the grid):
-// 8 waves, one 32 x 32 accumulator tile each, few registers per wave, several waves per SIMD -- while one accumulates,
-// another one's matrix instructions run. K advances in steps of two blocks through a ring of three LDS stages filled
-// two steps ahead. With KS = 2 a second group of 8 waves takes the other half of K (shapes with too few tiles to fill
-// the device) and the two partial tiles are added through LDS in a fixed order.
+// A workgroup owns 128 x 64 or 128 x 96 outputs over all of K (no exchange between workgroups; a result depends on the
+// shape alone): one wave per 64 x 32 outputs (two accumulator tiles, so that an operand read from LDS serves two matrix
+// instructions). K advances in steps of two blocks through a ring of LDS stages filled ahead by DMA: three stages of
+// 17 KB and three workgroups per compute unit for 128 x 64, four stages of 19 KB and two workgroups for 128 x 96 (a
+// third fewer activation bytes per unit of work, for shapes with enough such tiles). With KS = 2 or 3, further groups
+// of waves take the other shares of K (shapes with too few tiles to fill the device) and the partial tiles are added
+// through LDS in a fixed order.
 #include "device_utils.h"
 #include "kernels.h"
 
@@ -41,10 +43,8 @@ typedef int      v8i __attribute__((ext_vector_type(8)));
 typedef float    v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 
-constexpr int kBM = 128, kBN = 64;  // outputs per workgroup
-constexpr int kGroupWaves = 4;      // each wave: 64 x 32 outputs (two accumulator tiles)
-constexpr int kNA = 3;              // LDS stages
-constexpr int kMinTiles = 192;      // output tiles from which the kernel is used
+constexpr int kBM = 128;        // output rows per workgroup; its columns: 32 NT, NT = 2 or 3
+constexpr int kMinTiles = 192;  // 128 x 64 output tiles from which the kernel is used
 
 // ---- tiles ----------------------------------------------------------------------------------------------------------
 // The 32 FP6 codes of one row (column) of a block are 24 bytes, element e at bits [6 e, 6 e + 6). A step = a block
@@ -53,18 +53,17 @@ constexpr int kMinTiles = 192;      // output tiles from which the kernel is use
 //   plane 2 = [lane][block 1 bytes 0..15]
 // so that each block's operand registers are filled by one 16-byte and one 8-byte LDS read.
 //   activation tile (32 rows, step): 3 planes x 64 lanes x 16 bytes; lane (c, h): row c, h = 0 the hi parts, h = 1 the lo
-//                                    parts. Row scales apart: one dword per row and step (even block | odd block << 16).
-//   weight tile (64 columns, step):  3 planes x 64 columns x 16 bytes, then the scales as operand dwords of the scale
-//                                    product: [block][column tile of 32][64 lanes], lane l < 32: the column's fp16
-//                                    scale in the half-word of its block (K slot 0 or 1), lanes 32..63: 0.
+//                                    parts. Row scales apart, per 128 rows and step 1 KiB: row r at dwords 2 r, 2 r + 1
+//                                    = (even block | odd block << 16, 0): the operand of the scale product as it is read.
+//   weight tile (32 columns, step):  2 KiB: plane 0 (32 x 16 B), plane 1 (32 x 8 B block 0, 32 x 8 B block 1), plane 2,
+//                                    then the scales as operand dwords of the scale product: [block][64 lanes], lane
+//                                    l < 32: the column's fp16 scale in the half-word of its block (K slot 0 or 1),
+//                                    lanes 32..63: 0.
 constexpr int kATile  = 3 * 1024;
-constexpr int kWTile  = 4 * 1024;
+constexpr int kWTile  = 2 * 1024;
+constexpr int kSaTile = 1024;
 constexpr int kOffA   = 0;
 constexpr int kOffW   = kOffA + (kBM / 32) * kATile;
-constexpr int kOffSa  = kOffW + kWTile;
-constexpr int kStage  = kOffSa + (kBM / 32) * 256;
-constexpr int kRing   = kNA * kStage;
-constexpr int kDmaPerStep = (kBM / 32) * 3 + 4 + (kBM / 32);  // 12 activation planes, 4 weight KiB, 4 scale rows
 
 __device__ __forceinline__ uint32_t fp6_code(int t) {  // integer |t| <= 15 as E2M3 value t / 8
   const uint32_t mag = (uint32_t) (t < 0 ? -t : t);
@@ -96,17 +95,17 @@ __device__ __forceinline__ void store_planes(uint8_t *tile, int lane, const uint
   q[64] = make_uint2(b1[4], b1[5]);
 }
 
-// one thread per (column tile, step, column)
+// one thread per (column tile of 32, step, column)
 __global__ __launch_bounds__(256) void q4_0_to_fp6_tiles_kernel(uint8_t *__restrict__ tiles, const uint32_t *__restrict__ w,
                                                                 int n, int pairs, size_t total) {
   const size_t t = (size_t) blockIdx.x * 256 + threadIdx.x;
   if (t >= total) {
     return;
   }
-  const int    c = (int) (t & 63);
-  const size_t rec = t >> 6;  // tile * pairs + step
+  const int    c = (int) (t & 31);
+  const size_t rec = t >> 5;  // tile * pairs + step
   const int    step = (int) (rec % (size_t) pairs), tile = (int) (rec / (size_t) pairs);
-  const int    col = tile * kBN + c;
+  const int    col = tile * 32 + c;
   uint32_t     o0[6] = { 0, 0, 0, 0, 0, 0 }, o1[6] = { 0, 0, 0, 0, 0, 0 };
   uint32_t     d0 = 0, d1 = 0;
   if (col < n) {
@@ -136,13 +135,15 @@ __global__ __launch_bounds__(256) void q4_0_to_fp6_tiles_kernel(uint8_t *__restr
     pack_fp6(o1, v1);
   }
   uint8_t *tile_base = tiles + rec * kWTile;
-  store_planes(tile_base, c, o0, o1);
-  uint32_t *sc = reinterpret_cast<uint32_t *>(tile_base + 3 * 1024);
-  const int nt = c >> 5, l = c & 31;
-  sc[(0 * 2 + nt) * 64 + l]      = d0;
-  sc[(0 * 2 + nt) * 64 + 32 + l] = 0u;
-  sc[(1 * 2 + nt) * 64 + l]      = d1;
-  sc[(1 * 2 + nt) * 64 + 32 + l] = 0u;
+  reinterpret_cast<uint4 *>(tile_base)[c]        = make_uint4(o0[0], o0[1], o0[2], o0[3]);
+  reinterpret_cast<uint2 *>(tile_base + 512)[c]  = make_uint2(o0[4], o0[5]);
+  reinterpret_cast<uint2 *>(tile_base + 768)[c]  = make_uint2(o1[4], o1[5]);
+  reinterpret_cast<uint4 *>(tile_base + 1024)[c] = make_uint4(o1[0], o1[1], o1[2], o1[3]);
+  uint32_t *sc = reinterpret_cast<uint32_t *>(tile_base + 1536);
+  sc[c]      = d0;
+  sc[32 + c] = 0u;
+  sc[64 + c] = d1;
+  sc[96 + c] = 0u;
 }
 
 // one thread per (row of the padded row count, step)
@@ -192,21 +193,34 @@ __global__ __launch_bounds__(256) void q8_0_to_fp6_tiles_kernel(uint8_t *__restr
   uint8_t *tile = tiles + ((size_t) (r / 32) * pairs + step) * kATile;
   store_planes(tile, r % 32, oh[0], oh[1]);
   store_planes(tile, 32 + r % 32, ol[0], ol[1]);
-  scales[((size_t) (r / 32) * pairs + step) * 32 + (r % 32)] = (a[0] & 0xffffu) | (a[8] & 0xffff0000u);
+  *reinterpret_cast<uint2 *>(scales + (((size_t) (r / kBM) * pairs + step) * kBM + (r % kBM)) * 2) =
+      make_uint2((a[0] & 0xffffu) | (a[8] & 0xffff0000u), 0u);
 }
 
 // ---- the matmul -----------------------------------------------------------------------------------------------------
-template <int KS>
-__global__ __launch_bounds__(kGroupWaves * kWave * KS) void gemm_fp6_lds_kernel(float *__restrict__ out,
-                                                                                const uint8_t *__restrict__ a_tiles,
-                                                                                const uint32_t *__restrict__ a_scales,
-                                                                                const uint8_t *__restrict__ w_tiles, int m, int n,
-                                                                                int pairs, int tiles_m, int tiles_n) {
+// NT: column tiles of 32 per workgroup (2 or 3; a K group has 2 NT waves), NS: LDS stages, KS: K groups
+template <int NT>
+struct Shape {
+  static constexpr int kWaves    = 2 * NT;                            // per K group: 2 (rows of 64) x NT (columns of 32)
+  static constexpr int kOffSa    = kOffW + NT * kWTile;
+  static constexpr int kStage    = kOffSa + kSaTile;
+  static constexpr int kDma      = (kBM / 32) * 3 + 2 * NT + 1;       // 12 activation planes, 2 NT weight KiB, 1 KiB of scales
+  static constexpr int kPerWave  = (kDma + kWaves - 1) / kWaves;      // transfers of the waves that issue the most
+};
+
+template <int NT, int NS, int KS>
+__global__ __launch_bounds__(Shape<NT>::kWaves *kWave *KS) void gemm_fp6_lds_kernel(float *__restrict__ out,
+                                                                                   const uint8_t *__restrict__ a_tiles,
+                                                                                   const uint8_t *__restrict__ a_scales,
+                                                                                   const uint8_t *__restrict__ w_tiles, int m,
+                                                                                   int n, int pairs, int tiles_m, int tiles_n) {
+  using S = Shape<NT>;
+  constexpr int kStage = S::kStage, kRing = NS * S::kStage, kOffSa = S::kOffSa;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int kg = wave / kGroupWaves, u = wave % kGroupWaves;  // K group, wave of the group
-  const int wm = u >> 1, nt = u & 1;                          // rows 64 wm .. 64 wm + 63, columns 32 nt .. 32 nt + 31
+  const int kg = wave / S::kWaves, u = wave % S::kWaves;  // K group, wave of the group
+  const int wm = u / NT, nt = u % NT;                     // rows 64 wm .. 64 wm + 63, columns 32 nt .. 32 nt + 31
 
   // Workgroups are handed to the 8 XCDs round-robin, and each XCD has its own L2: the row blocks of one column tile
   // (which read the same weights) are consecutive workgroups of ONE XCD.
@@ -226,46 +240,64 @@ __global__ __launch_bounds__(kGroupWaves * kWave * KS) void gemm_fp6_lds_kernel(
   const uint32_t ring0 = (uint32_t) (uintptr_t) ring;
 
   // ---- DMA: everything this kernel reads from memory goes straight into LDS (written out as instructions: the
-  // compiler would make every LDS read after a DMA it knows of wait for ALL DMA in flight). The kDmaPerStep = 20
-  // transfers of a step are dealt to the 4 waves of a K group, 5 each: wave u issues activation planes u, u + 4 and
-  // u + 8 (of 12: row tile p / 3, plane p % 3), weight KiB u and the scales of row tile u. Addresses are a scalar base
-  // (tile and step) plus a per-lane offset that never changes, so a transfer costs no vector ALU work. ----
+  // compiler would make every LDS read after a DMA it knows of wait for ALL DMA in flight). The transfers of a step
+  // (1 KiB each: 12 activation planes, 2 NT weight KiB, the row scales) are dealt to the waves of a K group round
+  // robin: wave u issues transfers u, u + kWaves, ... Addresses are a scalar base (tile and step) plus a per-lane
+  // offset that never changes, so a transfer costs no vector ALU work. ----
   auto dma16 = [&](const uint8_t *base, uint32_t lane_off, uint32_t dst) {
     asm volatile("s_mov_b32 m0, %2\n s_nop 0\n global_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(dst) : "memory");
   };
-  auto dma4 = [&](const void *base, uint32_t lane_off, uint32_t dst) {
-    asm volatile("s_mov_b32 m0, %2\n s_nop 0\n global_load_lds_dword %0, %1" ::"v"(lane_off), "s"(base), "s"(dst) : "memory");
-  };
-  const int last_mt = (m + 31) / 32 - 1;
-  auto      row_tile = [&](int i) { return (size_t) min(tile_m * (kBM / 32) + i, last_mt); };
-  const uint8_t *src_a[3];
-  uint32_t       dst_a[3];
+  const int last_mt  = (m + 31) / 32 - 1;
+  const int last_ct  = (n + 31) / 32 - 1;  // column tiles past the end re-read the last one (their outputs are not stored)
+  const uint8_t *src[S::kPerWave];
+  uint32_t       dst[S::kPerWave], stride[S::kPerWave];
 #pragma unroll
-  for (int i = 0; i < 3; ++i) {
-    const int p = u + 4 * i;
-    src_a[i] = a_tiles + row_tile(p / 3) * pairs * kATile + (p % 3) * 1024;
-    dst_a[i] = ring0 + kOffA + (p / 3) * kATile + (p % 3) * 1024;
+  for (int i = 0; i < S::kPerWave; ++i) {
+    const int p = u + S::kWaves * i;  // (p >= kDma: this wave has one transfer less; the entry is never used)
+    if (p < 12) {
+      const size_t rt = (size_t) min(tile_m * (kBM / 32) + p / 3, last_mt);
+      src[i]    = a_tiles + rt * pairs * kATile + (p % 3) * 1024;
+      dst[i]    = ring0 + kOffA + (p / 3) * kATile + (p % 3) * 1024;
+      stride[i] = kATile;
+    } else if (p < 12 + 2 * NT) {
+      const int    q  = p - 12;
+      const size_t ct = (size_t) min(tile_n * NT + q / 2, last_ct);
+      src[i]    = w_tiles + ct * pairs * kWTile + (q % 2) * 1024;
+      dst[i]    = ring0 + kOffW + (q / 2) * kWTile + (q % 2) * 1024;
+      stride[i] = kWTile;
+    } else {
+      src[i]    = a_scales + (size_t) tile_m * pairs * kSaTile;
+      dst[i]    = ring0 + kOffSa;
+      stride[i] = kSaTile;
+    }
   }
-  const uint8_t  *src_w  = w_tiles + (size_t) tile_n * pairs * kWTile + u * 1024;
-  const uint32_t  dst_w  = ring0 + kOffW + u * 1024;
-  const uint32_t *src_s  = a_scales + row_tile(u) * pairs * 32;
-  const uint32_t  dst_s  = ring0 + kOffSa + u * 256;
-  const uint32_t  lane16 = lane * 16, lane4 = (lane & 31) * 4;
+  const int      mine   = (S::kDma - u + S::kWaves - 1) / S::kWaves;  // transfers of this wave per step
+  const uint32_t lane16 = lane * 16;
   auto issue_group = [&](int x, int stage) {  // the transfers of step x into `stage`
     const size_t   s  = (size_t) step_of(x);
     const uint32_t so = (uint32_t) stage * kStage;
-    dma4(src_s + s * 32, lane4, dst_s + so);
-    dma16(src_w + s * kWTile, lane16, dst_w + so);
 #pragma unroll
-    for (int i = 0; i < 3; ++i) {
-      dma16(src_a[i] + s * kATile, lane16, dst_a[i] + so);
+    for (int i = 0; i < S::kPerWave; ++i) {
+      if (i < S::kPerWave - 1 || mine == S::kPerWave) {
+        dma16(src[i] + s * stride[i], lane16, dst[i] + so);
+      }
     }
   };
-  static_assert(kDmaPerStep == 5 * kGroupWaves, "five transfers per wave and step");
+  // this wave's transfers of the oldest step in flight have landed (NS - 2 younger groups may stay in flight; s_waitcnt
+  // operand: vmcnt in bits 3:0 and 15:14, expcnt 7 = no wait in 6:4, lgkmcnt(0) in 11:8)
+  auto wait_oldest_group = [&]() {
+    static_assert((NS - 2) * S::kPerWave < 16, "vmcnt fits the low four bits");
+    if (mine == S::kPerWave) {
+      __builtin_amdgcn_s_waitcnt(0x0070 | ((NS - 2) * S::kPerWave));
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0070 | ((NS - 2) * (S::kPerWave - 1)));
+    }
+  };
 
-  static_assert(kNA == 3, "the loop below is unrolled over the three stages");
-  issue_group(0, 0);
-  issue_group(1, 1);
+#pragma unroll
+  for (int x = 0; x < NS - 1; ++x) {
+    issue_group(x, x);
+  }
 
   const v16f zero_f = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
   v16f       acc0 = zero_f, acc1 = zero_f;  // rows 64 wm .. + 31 and 64 wm + 32 .. + 63
@@ -273,14 +305,17 @@ __global__ __launch_bounds__(kGroupWaves * kWave * KS) void gemm_fp6_lds_kernel(
   const int scale_a = (lane >> 5) ? 127 + 3 : 127 + 7, scale_b = 127 + 3;
   const uint32_t a_rd  = ring0 + kOffA + (2 * wm) * kATile + lane * 16;
   const uint32_t a_rd8 = ring0 + kOffA + (2 * wm) * kATile + 1024 + lane * 8;  // plane 1: [block 0 tails: 64 x 8][block 1 tails]
-  const uint32_t w_rd  = ring0 + kOffW + (nt * 32 + (lane & 31)) * 16;
-  const uint32_t w_rd8 = ring0 + kOffW + 1024 + (nt * 32 + (lane & 31)) * 8;
-  const uint32_t sb_rd = ring0 + kOffW + 3 * 1024 + nt * 256 + lane * 4;
-  const uint32_t sa_rd = ring0 + kOffSa + (2 * wm) * 256 + lane * 4;
+  const uint32_t w_rd  = ring0 + kOffW + nt * kWTile + (lane & 31) * 16;       // plane 0; plane 2 at + 1024
+  const uint32_t w_rd8 = ring0 + kOffW + nt * kWTile + 512 + (lane & 31) * 8;  // block 0 tails; block 1 at + 256
+  const uint32_t sb_rd = ring0 + kOffW + nt * kWTile + 1536 + lane * 4;        // block 0; block 1 at + 256
+  const uint32_t sa_rd = ring0 + kOffSa + (2 * wm) * 256 + (lane & 31) * 8;    // upper row tile; the lower one at + 256
 
   typedef __attribute__((address_space(3))) const uint8_t *lds_ptr;
   auto lds_v4i = [](uint32_t addr, int off) {
     return *reinterpret_cast<__attribute__((address_space(3))) const v4i *>((lds_ptr) (uintptr_t) addr + off);
+  };
+  auto lds_v2i = [](uint32_t addr, int off) {
+    return *reinterpret_cast<__attribute__((address_space(3))) const v2i *>((lds_ptr) (uintptr_t) addr + off);
   };
   auto lds_u32 = [](uint32_t addr, int off) {
     return *reinterpret_cast<__attribute__((address_space(3))) const uint32_t *>((lds_ptr) (uintptr_t) addr + off);
@@ -308,9 +343,8 @@ __global__ __launch_bounds__(kGroupWaves * kWave * KS) void gemm_fp6_lds_kernel(
   auto step = [&](auto stage_tag, int t) {
     constexpr int ST = decltype(stage_tag)::value;
     constexpr int so = ST * kStage;
-    // step t is complete in LDS: this wave's transfers of it have landed (the next step's five may stay in flight;
-    // s_waitcnt operand: vmcnt in bits 3:0 and 15:14, expcnt 7 = no wait in 6:4, lgkmcnt(0) in 11:8), then everybody's
-    __builtin_amdgcn_s_waitcnt(0x0070 | 5);
+    // step t is complete in LDS: this wave's transfers of it have landed, then everybody's
+    wait_oldest_group();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     v2i a00hi, a01hi, a10hi, a11hi, b0hi, b1hi;  // a<row tile><block>
@@ -318,23 +352,23 @@ __global__ __launch_bounds__(kGroupWaves * kWave * KS) void gemm_fp6_lds_kernel(
         "ds_read_b64 %0, %6 offset:%c8\n ds_read_b64 %1, %6 offset:%c9\n ds_read_b64 %2, %6 offset:%c10\n"
         " ds_read_b64 %3, %6 offset:%c11\n ds_read_b64 %4, %7 offset:%c12\n ds_read_b64 %5, %7 offset:%c13"
         : "=&v"(a00hi), "=&v"(a01hi), "=&v"(a10hi), "=&v"(a11hi), "=&v"(b0hi), "=&v"(b1hi)
-        : "v"(a_rd8), "v"(w_rd8), "i"(so), "i"(so + 512), "i"(so + kATile), "i"(so + kATile + 512), "i"(so), "i"(so + 512)
+        : "v"(a_rd8), "v"(w_rd8), "i"(so), "i"(so + 512), "i"(so + kATile), "i"(so + kATile + 512), "i"(so), "i"(so + 256)
         : "memory");
     const v4i      a00lo = lds_v4i(a_rd, so), a01lo = lds_v4i(a_rd, so + 2048);
     const v4i      a10lo = lds_v4i(a_rd, so + kATile), a11lo = lds_v4i(a_rd, so + kATile + 2048);
-    const v4i      b0lo = lds_v4i(w_rd, so), b1lo = lds_v4i(w_rd, so + 2048);
-    const uint32_t sb0 = lds_u32(sb_rd, so), sb1 = lds_u32(sb_rd, so + 512);
-    uint32_t       sa0 = lds_u32(sa_rd, so), sa1 = lds_u32(sa_rd, so + 256);
-    // everybody has left step t - 1: its stage takes step t + 2
-    issue_group(t + 2, (ST + 2) % kNA);
+    const v4i      b0lo = lds_v4i(w_rd, so), b1lo = lds_v4i(w_rd, so + 1024);
+    const uint32_t sb0 = lds_u32(sb_rd, so), sb1 = lds_u32(sb_rd, so + 256);
+    v2i            sa0 = lds_v2i(sa_rd, so), sa1 = lds_v2i(sa_rd, so + 256);  // (scale pair, 0): operands as they are
+    // everybody has left step t - 1: its stage takes step t + NS - 1
+    issue_group(t + NS - 1, (ST + NS - 1) % NS);
     if (KS > 1) {
-      sa0 = t < steps ? sa0 : 0u;  // an iteration past this K group's last step adds zeros
-      sa1 = t < steps ? sa1 : 0u;
+      sa0[0] = t < steps ? sa0[0] : 0;  // an iteration past this K group's last step adds zeros
+      sa1[0] = t < steps ? sa1[0] : 0;
     }
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(a00hi), "+v"(a01hi), "+v"(a10hi), "+v"(a11hi), "+v"(b0hi), "+v"(b1hi)::"memory");
     const v8i fa00 = operand(a00lo, a00hi), fa01 = operand(a01lo, a01hi), fa10 = operand(a10lo, a10hi), fa11 = operand(a11lo, a11hi);
     const v8i fb0 = operand(b0lo, b0hi), fb1 = operand(b1lo, b1hi);
-    const v4h sa0_op = __builtin_bit_cast(v4h, make_uint2(sa0, 0u)), sa1_op = __builtin_bit_cast(v4h, make_uint2(sa1, 0u));
+    const v4h sa0_op = __builtin_bit_cast(v4h, sa0), sa1_op = __builtin_bit_cast(v4h, sa1);
     const v4h sb0_op = __builtin_bit_cast(v4h, make_uint2(sb0, 0u)), sb1_op = __builtin_bit_cast(v4h, make_uint2(sb1, 0u));
 #define HTPOPS_FP6_SUMS(fa, fb) __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa, fb, zero_f, 2, 2, 0, scale_a, 0, scale_b)
 #define HTPOPS_SCALE_PRODUCTS(sa, sb) __builtin_amdgcn_mfma_f32_32x32x8f16(sa, sb, zero_f, 0, 0, 0)
@@ -360,13 +394,17 @@ __global__ __launch_bounds__(kGroupWaves * kWave * KS) void gemm_fp6_lds_kernel(
 #undef HTPOPS_SCALE_PRODUCTS
 #undef HTPOPS_FENCE
   };
-  for (int t = 0; t < iters; t += 3) {
+  static_assert(NS == 3 || NS == 4, "the loop is unrolled over the stages");
+  for (int t = 0; t < iters; t += NS) {
     step(std::integral_constant<int, 0>(), t);
     if (t + 1 < iters) {
       step(std::integral_constant<int, 1>(), t + 1);
     }
     if (t + 2 < iters) {
       step(std::integral_constant<int, 2>(), t + 2);
+    }
+    if (NS == 4 && t + 3 < iters) {
+      step(std::integral_constant<int, (NS == 4 ? 3 : 0)>(), t + 3);
     }
   }
   fma_half(acc1, sy, cy, 0);  // the last step's unit (1, 1)
@@ -375,13 +413,14 @@ __global__ __launch_bounds__(kGroupWaves * kWave * KS) void gemm_fp6_lds_kernel(
   // -- the K groups meet: group g > 0 leaves its tiles in LDS, group 0 adds them in order --
   __builtin_amdgcn_s_waitcnt(0x0070);  // (transfers of steps past the end must have landed before LDS is reused or released)
   if (KS > 1) {
+    static_assert((KS - 1) * S::kWaves * 32 * 64 * 4 <= KS * kRing, "the partial tiles fit the rings");
     __builtin_amdgcn_s_barrier();
     float *red = reinterpret_cast<float *>(lds);
     if (kg > 0) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        red[(((kg - 1) * kGroupWaves + u) * 32 + i) * 64 + lane]      = acc0[i];
-        red[(((kg - 1) * kGroupWaves + u) * 32 + 16 + i) * 64 + lane] = acc1[i];
+        red[(((kg - 1) * S::kWaves + u) * 32 + i) * 64 + lane]      = acc0[i];
+        red[(((kg - 1) * S::kWaves + u) * 32 + 16 + i) * 64 + lane] = acc1[i];
       }
     }
     __syncthreads();
@@ -392,13 +431,13 @@ __global__ __launch_bounds__(kGroupWaves * kWave * KS) void gemm_fp6_lds_kernel(
     for (int g = 1; g < KS; ++g) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        acc0[i] += red[(((g - 1) * kGroupWaves + u) * 32 + i) * 64 + lane];
-        acc1[i] += red[(((g - 1) * kGroupWaves + u) * 32 + 16 + i) * 64 + lane];
+        acc0[i] += red[(((g - 1) * S::kWaves + u) * 32 + i) * 64 + lane];
+        acc1[i] += red[(((g - 1) * S::kWaves + u) * 32 + 16 + i) * 64 + lane];
       }
     }
   }
 
-  const int col = tile_n * kBN + nt * 32 + (lane & 31);
+  const int col = (tile_n * NT + nt) * 32 + (lane & 31);
   if (col < n) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
@@ -413,13 +452,15 @@ __global__ __launch_bounds__(kGroupWaves * kWave * KS) void gemm_fp6_lds_kernel(
   }
 }
 
-template <int KS>
-hipError_t launch_instance(hipStream_t stream, float *out, const uint8_t *a_tiles, const uint32_t *a_scales,
+template <int NT, int NS, int KS>
+hipError_t launch_instance(hipStream_t stream, float *out, const uint8_t *a_tiles, const uint8_t *a_scales,
                            const uint8_t *w_tiles, int m, int n, int pairs) {
-  const int    tiles_m = (m + kBM - 1) / kBM, tiles_n = (n + kBN - 1) / kBN;
-  const size_t lds     = (size_t) KS * kRing;
+  using S = Shape<NT>;
+  const int    tiles_m = (m + kBM - 1) / kBM, tiles_n = (n + 32 * NT - 1) / (32 * NT);
+  const size_t lds     = (size_t) KS * NS * S::kStage;
+  static_assert((size_t) KS * NS * S::kStage <= 160 * 1024, "the rings fit LDS");
   const dim3   grid((unsigned) (((tiles_n + 7) / 8) * 8 * tiles_m));
-  auto         kernel  = gemm_fp6_lds_kernel<KS>;
+  auto         kernel  = gemm_fp6_lds_kernel<NT, NS, KS>;
   static bool  raised  = false;
   if (!raised) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
@@ -428,7 +469,7 @@ hipError_t launch_instance(hipStream_t stream, float *out, const uint8_t *a_tile
     }
     raised = true;
   }
-  hipLaunchKernelGGL(kernel, grid, dim3(kGroupWaves * kWave * KS), lds, stream, out, a_tiles, a_scales, w_tiles, m, n, pairs,
+  hipLaunchKernelGGL(kernel, grid, dim3(S::kWaves * kWave * KS), lds, stream, out, a_tiles, a_scales, w_tiles, m, n, pairs,
                      tiles_m, tiles_n);
   return hipGetLastError();
 }
@@ -442,16 +483,16 @@ bool gemm_fp6_lds_fits(int m, int k, int n) {
 bool gemm_fp6_lds_fills_device(int m, int n) {
   // Below this the kernel's workgroups (one per tile, K split over at most three wave groups inside it) leave compute
   // units idle, and the fragment kernel, which splits K over workgroups, is faster.
-  return (long) ((m + kBM - 1) / kBM) * ((n + kBN - 1) / kBN) >= kMinTiles;
+  return (long) ((m + kBM - 1) / kBM) * ((n + 63) / 64) >= kMinTiles;
 }
 
 size_t gemm_fp6_lds_weight_tile_bytes(int k, int n) {
-  return (size_t) ((n + kBN - 1) / kBN) * (size_t) (k / 64) * kWTile;
+  return (size_t) ((n + 31) / 32) * (size_t) (k / 64) * kWTile;
 }
 
 size_t gemm_fp6_lds_act_tile_bytes(int m, int k) {
-  const size_t m_tiles = ((size_t) m + 31) / 32, pairs = (size_t) k / 64;
-  return m_tiles * pairs * kATile + m_tiles * pairs * 128;
+  const size_t m_tiles = ((size_t) m + 31) / 32, m_blocks = ((size_t) m + kBM - 1) / kBM, pairs = (size_t) k / 64;
+  return m_tiles * pairs * kATile + m_blocks * pairs * kSaTile;
 }
 
 hipError_t launch_q4_0_to_fp6_tiles(hipStream_t stream, void *dst, const void *weight, int k, int n) {
@@ -459,7 +500,7 @@ hipError_t launch_q4_0_to_fp6_tiles(hipStream_t stream, void *dst, const void *w
     return hipErrorNotSupported;
   }
   const int    pairs = k / 64;
-  const size_t total = (size_t) ((n + kBN - 1) / kBN) * pairs * 64;
+  const size_t total = (size_t) ((n + 31) / 32) * pairs * 32;
   hipLaunchKernelGGL(q4_0_to_fp6_tiles_kernel, dim3((unsigned) ((total + 255) / 256)), dim3(256), 0, stream,
                      static_cast<uint8_t *>(dst), static_cast<const uint32_t *>(weight), n, pairs, total);
   return hipGetLastError();
@@ -473,30 +514,33 @@ hipError_t launch_gemm_fp6_lds(hipStream_t stream, float *out, const void *act_q
   const int pairs   = k / 64;
   const int m_tiles = (m + 31) / 32;
   uint8_t  *tiles   = static_cast<uint8_t *>(act_tiles);
-  uint32_t *scales  = reinterpret_cast<uint32_t *>(tiles + (size_t) m_tiles * pairs * kATile);
+  uint8_t  *scales  = tiles + (size_t) m_tiles * pairs * kATile;
   if (!act_tiles_ready) {
     const size_t threads = (size_t) m_tiles * 32 * pairs;
-    hipLaunchKernelGGL(q8_0_to_fp6_tiles_kernel, dim3((unsigned) ((threads + 255) / 256)), dim3(256), 0, stream, tiles, scales,
-                       static_cast<const uint32_t *>(act_q8_0), m, pairs, m_tiles * 32);
+    hipLaunchKernelGGL(q8_0_to_fp6_tiles_kernel, dim3((unsigned) ((threads + 255) / 256)), dim3(256), 0, stream, tiles,
+                       reinterpret_cast<uint32_t *>(scales), static_cast<const uint32_t *>(act_q8_0), m, pairs, m_tiles * 32);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
       return e;
     }
   }
-  // A K group is 4 waves and one LDS ring, and a compute unit holds three rings: one group per workgroup when the
-  // tiles alone give every compute unit three workgroups, otherwise up to three groups per workgroup, each with its
-  // share of K, so that the same tiles put more waves on a compute unit.
-  const long       out_tiles = (long) ((m + kBM - 1) / kBM) * ((n + kBN - 1) / kBN);
-  int              ks        = out_tiles >= 640 ? 1 : out_tiles >= 384 ? 2 : 3;
-  ks                         = std::max(1, std::min(ks, pairs / 4));
-  const uint8_t *wt = static_cast<const uint8_t *>(weight_tiles);
+  const uint8_t *wt      = static_cast<const uint8_t *>(weight_tiles);
+  const long     tiles64 = (long) ((m + kBM - 1) / kBM) * ((n + 63) / 64);
+  // 128 x 64 tiles: a K group is 4 waves (one per SIMD) and one ring of three stages, and a compute unit holds three
+  // rings: one group per workgroup when the tiles alone give every compute unit three workgroups, otherwise up to
+  // three groups per workgroup, each with its share of K, so that the same tiles put more waves on a compute unit.
+  // (128 x 96 tiles -- NT = 3, four stages, two workgroups of 6 waves per compute unit, a third fewer activation bytes
+  // per unit of work -- measured slower, 84 against 64 us at 512 x 11008 x 4096: six waves do not spread evenly over
+  // four SIMDs.)
+  int ks = tiles64 >= 640 ? 1 : tiles64 >= 384 ? 2 : 3;
+  ks     = std::max(1, std::min(ks, pairs / 4));
   switch (ks) {
     case 1:
-      return launch_instance<1>(stream, out, tiles, scales, wt, m, n, pairs);
+      return launch_instance<2, 3, 1>(stream, out, tiles, scales, wt, m, n, pairs);
     case 2:
-      return launch_instance<2>(stream, out, tiles, scales, wt, m, n, pairs);
+      return launch_instance<2, 3, 2>(stream, out, tiles, scales, wt, m, n, pairs);
     default:
-      return launch_instance<3>(stream, out, tiles, scales, wt, m, n, pairs);
+      return launch_instance<2, 3, 3>(stream, out, tiles, scales, wt, m, n, pairs);
   }
 }
 
