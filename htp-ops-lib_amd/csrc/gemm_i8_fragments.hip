@@ -128,6 +128,64 @@ __global__ __launch_bounds__(256) void act_to_i8_fragments_kernel(ActMembers grp
   }
 }
 
+// The same for even block counts (k % 64 == 0) and 4-byte aligned rows: one thread per (row, block PAIR) reads its 68
+// bytes as dwords (five loads instead of eighteen 2-byte ones) and writes the four 16-byte pieces of the pair.
+__global__ __launch_bounds__(256) void act_pairs_to_i8_fragments_kernel(ActMembers grp, int m, int m_tiles, unsigned threads) {
+  const unsigned g = blockIdx.x * 256 + threadIdx.x;
+  if (g >= threads) {
+    return;
+  }
+  int mi = 0;
+  for (int i = 1; i < grp.count; ++i) {
+    mi = g >= grp.m[i].piece_begin / 4 ? i : mi;  // (a pair of blocks is four pieces)
+  }
+  const ActMember &mem   = grp.m[mi];
+  const unsigned   t     = g - mem.piece_begin / 4;
+  const int        nblk  = mem.nblk, pairs = nblk / 2;
+  const int        c     = (int) (t & 31);
+  const unsigned   f     = t >> 5;
+  const int        pr = (int) (f % (unsigned) pairs), tile = (int) (f / (unsigned) pairs);
+  if (tile >= m_tiles) {
+    return;
+  }
+  const int row = tile * 32 + c;
+  uint32_t  a[17];
+  if (row < m) {
+    const uint32_t *src = reinterpret_cast<const uint32_t *>(mem.act) + ((size_t) row * pairs + pr) * 17;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const u32x4_a4 v = *reinterpret_cast<const u32x4_a4 *>(src + 4 * i);
+      a[4 * i] = v.x, a[4 * i + 1] = v.y, a[4 * i + 2] = v.z, a[4 * i + 3] = v.w;
+    }
+    a[16] = src[16];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 17; ++i) {
+      a[i] = 0u;
+    }
+  }
+  // block 0: scale in the low half of a[0], quants at bytes 2 .. 33; block 1: scale in the high half of a[8], quants
+  // at bytes 36 .. 67 (dwords 9 .. 16)
+  uint32_t q0[8], q1[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    q0[i] = __builtin_amdgcn_alignbyte(a[i + 1], a[i], 2);
+    q1[i] = a[9 + i];
+  }
+  const size_t base0 = ((size_t) tile * nblk + 2 * pr) * 64, base1 = base0 + 64;
+  mem.frag[base0 + c]      = make_uint4(q0[0], q0[1], q0[2], q0[3]);
+  mem.frag[base0 + 32 + c] = make_uint4(q0[4], q0[5], q0[6], q0[7]);
+  mem.frag[base1 + c]      = make_uint4(q1[0], q1[1], q1[2], q1[3]);
+  mem.frag[base1 + 32 + c] = make_uint4(q1[4], q1[5], q1[6], q1[7]);
+  mem.scales[base0 + c]      = a[0] & 0xffffu;
+  mem.scales[base0 + 32 + c] = 0u;
+  mem.scales[base1 + c]      = a[8] >> 16;
+  mem.scales[base1 + 32 + c] = 0u;
+  if (t < 64) {
+    mem.scales[(size_t) m_tiles * nblk * 64 + t] = 0u;  // the row that blocks past the end of K are pointed at
+  }
+}
+
 // ---- the matmul ---------------------------------------------------------------------------------------------------
 
 constexpr int kGiThreads = 256;
@@ -427,10 +485,12 @@ hipError_t launch_act_to_i8_fragments_group(hipStream_t stream, int count, void 
   const int  m_tiles = (m + 31) / 32;
   ActMembers grp;
   size_t     pieces = 0;
+  bool       by_pairs = true;
   for (int i = 0; i < count; ++i) {
     if (ks[i] <= 0 || ks[i] % 32 != 0 || (reinterpret_cast<uintptr_t>(acts_q8_0[i]) & 1) != 0) {
       return hipErrorInvalidValue;
     }
+    by_pairs = by_pairs && ks[i] % 64 == 0 && (reinterpret_cast<uintptr_t>(acts_q8_0[i]) & 3) == 0;
     const int nblk      = ks[i] / 32;
     grp.m[i].frag        = static_cast<uint4 *>(act_fragments[i]);
     grp.m[i].scales      = const_cast<uint32_t *>(scales_of(act_fragments[i], (size_t) m_tiles, (size_t) nblk));
@@ -443,8 +503,14 @@ hipError_t launch_act_to_i8_fragments_group(hipStream_t stream, int count, void 
     return hipErrorNotSupported;
   }
   grp.count = count;
-  hipLaunchKernelGGL(act_to_i8_fragments_kernel, dim3((unsigned) ((pieces + 255) / 256)), dim3(256), 0, stream, grp, m,
-                     m_tiles, (unsigned) pieces);
+  if (by_pairs) {
+    const unsigned threads = (unsigned) (pieces / 4);
+    hipLaunchKernelGGL(act_pairs_to_i8_fragments_kernel, dim3((threads + 255) / 256), dim3(256), 0, stream, grp, m, m_tiles,
+                       threads);
+  } else {
+    hipLaunchKernelGGL(act_to_i8_fragments_kernel, dim3((unsigned) ((pieces + 255) / 256)), dim3(256), 0, stream, grp, m,
+                       m_tiles, (unsigned) pieces);
+  }
   return hipGetLastError();
 }
 

@@ -545,7 +545,7 @@ int run_few_rows(htpops_context *ctx, float *dst, const void *act, const void *w
     return r;
   }
   if (lw) {
-    const hipError_t e = htpops::launch_matmul_lane_order_group(ctx->stream, 1, &dst, act, &lw, &n, m, k,
+    const hipError_t e = htpops::launch_matmul_lane_order_group(ctx->stream, 1, &dst, &act, &lw, &n, m, k,
                                                                 (htpops::WeightType) wt);
     if (e == hipSuccess) {
       return HTPOPS_OK;
@@ -1144,7 +1144,9 @@ namespace {
 //  * one activation row (decode): members may read different activation buffers and have different k -- a whole
 //    hazard-free run of matrix-vector products (the seven projections of a layer whose inputs are all ready) is one
 //    launch; where a real data dependency exists (o after attention after q/k/v) the run is split there;
-//  * 2..16 rows: members must read the SAME activation rows (q/k/v or gate/up), which the few-row kernels stage once.
+//  * 2..16 rows: members of the same k; those that take the repacked-weight kernel share its launch whatever rows
+//    they read, the others only with members that read the same rows (q/k/v or gate/up);
+//  * many rows on small output tiles: one launch for the products, one for the activation conversions.
 struct GemvBatch {
   int                   wt = 0, m = 0, count = 0;
   struct RequestHeader *hdr[htpops::kGemvGroupMax];
@@ -1232,42 +1234,53 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
       ret = ret == 1 ? HTPOPS_OK : ret;
     } else if (b.m == 1) {
       e = htpops::launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k, (htpops::WeightType) b.wt);
-    } else if (htpops::gemv_rows_fits(b.m, k0, (htpops::WeightType) b.wt)) {
-      // 2..4 rows: the decode kernel's weight stream with the rows staged in LDS, whatever n and the weight type
-      e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, b.count, b.out, a0, b.w, b.n, b.m, k0,
-                                                  (htpops::WeightType) b.wt);
     } else {
-      // Members whose weights have (or get) a repacked copy go to the kernel that streams it, the others to the
-      // K-sliced kernel: which kernel a matrix gets depends on that matrix alone, so a request gives the same bits
-      // grouped or alone.
-      float      *out_a[htpops::kGemvGroupMax], *out_b[htpops::kGemvGroupMax];
-      const void *w_a[htpops::kGemvGroupMax], *w_b[htpops::kGemvGroupMax];
-      int         n_a[htpops::kGemvGroupMax], n_b[htpops::kGemvGroupMax], count_a = 0, count_b = 0;
-      for (int i = 0; i < b.count; ++i) {
-        const void *lw = nullptr;
-        if (int r = lane_order_weights(ctx, b.w[i], a0, b.m, k0, b.n[i], b.wt, &lw)) {
-          b.hdr[i]->state = r;
-        } else if (lw) {
-          out_a[count_a] = b.out[i], w_a[count_a] = lw, n_a[count_a++] = b.n[i];
-        } else if (b.m <= kSkinnyGroupMaxM) {
-          out_b[count_b] = b.out[i], w_b[count_b] = b.w[i], n_b[count_b++] = b.n[i];
-        } else {
-          // more rows than the K-sliced group launch takes: on its own
-          b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], a0, b.w[i], b.m, k0, b.n[i], b.wt);
+      // 2..16 rows, same k. Members whose weights have (or get) a repacked copy go to the kernel that streams it,
+      // each with its own activation rows; the others share a launch only when they read the same rows (the 2..4-row
+      // weight stream and the K-sliced kernel stage one set of rows per launch). Which kernel a matrix gets depends
+      // on that matrix alone.
+      bool same_act = true;
+      for (int i = 1; i < b.count; ++i) {
+        same_act = same_act && b.act[i] == a0;
+      }
+      if (same_act && htpops::gemv_rows_fits(b.m, k0, (htpops::WeightType) b.wt)) {
+        e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, b.count, b.out, a0, b.w, b.n, b.m, k0,
+                                                    (htpops::WeightType) b.wt);
+      } else {
+        float      *out_a[htpops::kGemvGroupMax], *out_b[htpops::kGemvGroupMax];
+        const void *w_a[htpops::kGemvGroupMax], *w_b[htpops::kGemvGroupMax], *act_a[htpops::kGemvGroupMax];
+        int         n_a[htpops::kGemvGroupMax], n_b[htpops::kGemvGroupMax], count_a = 0, count_b = 0;
+        const bool  rows_kernel = htpops::gemv_rows_fits(b.m, k0, (htpops::WeightType) b.wt);
+        for (int i = 0; i < b.count; ++i) {
+          const void *lw = nullptr;
+          int         r  = HTPOPS_OK;
+          if (!rows_kernel) {
+            r = lane_order_weights(ctx, b.w[i], b.act[i], b.m, k0, b.n[i], b.wt, &lw);
+          }
+          if (r) {
+            b.hdr[i]->state = r;
+          } else if (lw) {
+            out_a[count_a] = b.out[i], w_a[count_a] = lw, act_a[count_a] = b.act[i], n_a[count_a++] = b.n[i];
+          } else if (same_act && !rows_kernel && b.m <= kSkinnyGroupMaxM) {
+            out_b[count_b] = b.out[i], w_b[count_b] = b.w[i], n_b[count_b++] = b.n[i];
+          } else {
+            // different rows than the rest, or more rows than the K-sliced group launch takes: on its own
+            b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act[i], b.w[i], b.m, k0, b.n[i], b.wt);
+          }
         }
-      }
-      e = hipSuccess;
-      if (count_a > 0) {
-        e = htpops::launch_matmul_lane_order_group(ctx->stream, count_a, out_a, a0, w_a, n_a, b.m, k0,
-                                                   (htpops::WeightType) b.wt);
-      }
-      if (e == hipSuccess && count_b > 0) {
-        const size_t ws = htpops::matmul_skinny_group_workspace_bytes(count_b, n_b, b.m, k0);
-        if (int r = ensure_workspace(ctx, ws)) {
-          ret = r;
-        } else {
-          e = htpops::launch_matmul_skinny_group(ctx->stream, count_b, out_b, a0, w_b, n_b, b.m, k0,
-                                                 (htpops::WeightType) b.wt, ctx->workspace, ctx->tickets, kTicketSlots);
+        e = hipSuccess;
+        if (count_a > 0) {
+          e = htpops::launch_matmul_lane_order_group(ctx->stream, count_a, out_a, act_a, w_a, n_a, b.m, k0,
+                                                     (htpops::WeightType) b.wt);
+        }
+        if (e == hipSuccess && count_b > 0) {
+          const size_t ws = htpops::matmul_skinny_group_workspace_bytes(count_b, n_b, b.m, k0);
+          if (int r = ensure_workspace(ctx, ws)) {
+            ret = r;
+          } else {
+            e = htpops::launch_matmul_skinny_group(ctx->stream, count_b, out_b, a0, w_b, n_b, b.m, k0,
+                                                   (htpops::WeightType) b.wt, ctx->workspace, ctx->tickets, kTicketSlots);
+          }
         }
       }
     }
@@ -1324,7 +1337,7 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
     }
   }
   bool join = b.count > 0 && b.count < htpops::kGemvGroupMax && b.wt == wt && b.m == p->m &&
-              (p->m == 1 || many_rows || (b.k[0] == p->k && b.act[0] == act));
+              (p->m == 1 || many_rows || b.k[0] == p->k);
   for (int i = 0; join && i < b.count; ++i) {
     const size_t wi = weight_bytes((size_t) b.n[i], (size_t) b.k[i], b.wt), oi = (size_t) b.m * b.n[i] * 4;
     const size_t ai = q8_0_bytes((size_t) b.m, (size_t) b.k[i]);

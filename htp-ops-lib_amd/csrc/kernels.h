@@ -57,7 +57,8 @@ hipError_t launch_matmul_skinny_group(hipStream_t stream, int count, float *cons
 bool       matmul_lane_order_fits(int n, int m, int k, WeightType wt);
 size_t     matmul_lane_order_weight_bytes(int k, int n, WeightType wt);
 hipError_t launch_weights_to_lane_order(hipStream_t stream, void *dst, const void *weight, int k, int n, WeightType wt);
-hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *const *outs, const void *act,
+// (one launch for `count` matmuls of the same m, k and weight type; member i reads the activation rows acts[i])
+hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *const *outs, const void *const *acts,
                                           const void *const *lane_order_weights, const int *ns, int m, int k,
                                           WeightType wt);
 // many-row path for Q4_0 weights, k % 64 == 0: FP6 scaled MFMA (exact: int8 = 16 hi + lo, all parts |t| <= 15) over operand

@@ -113,7 +113,8 @@ __global__ __launch_bounds__(256) void q8_0_to_lane_order_kernel(uint8_t *__rest
 }
 
 struct LaneOrderGroupArgs {
-  const uint8_t *w[kGemvGroupMax];  // repacked weights
+  const uint8_t *w[kGemvGroupMax];    // repacked weights
+  const uint8_t *act[kGemvGroupMax];  // Q8_0 activation rows of each member (members may share them)
   float         *out[kGemvGroupMax];
   int            n[kGemvGroupMax];
 };
@@ -130,8 +131,7 @@ struct QuadRegs {
 //       traffic into a CU by a quarter; used when that still leaves enough workgroups.
 // WT:   weight type of the repacked copy; Q8_0 quads are twice the bytes, so half as many are fetched at a time
 template <int ROWS, int TPW, int WT>
-__global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrderGroupArgs grp,
-                                                                       const uint8_t *__restrict__ act, int m, int k) {
+__global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrderGroupArgs grp, int m, int k) {
   constexpr int kLoChunk    = WT == kQ4_0 ? 4 : 2;  // quads a wave fetches at a time
   constexpr int kQuadBytes  = quad_bytes(WT);
   constexpr int kLoads      = WT == kQ4_0 ? 2 : 3;  // load instructions per quad
@@ -149,7 +149,8 @@ __global__ __launch_bounds__(kLoThreads) void matmul_lane_order_kernel(LaneOrder
   // a second tile past the end of an odd tile count repeats the last one (never stored)
   const int tile = min((int) blockIdx.x * TPW + tw, n / kLoRows - 1);
   const int nblk = k / 32, nquads = nblk / 4;
-  const uint8_t *__restrict__ wt = grp.w[blockIdx.y] + (size_t) tile * nquads * kQuadBytes;
+  const uint8_t *__restrict__ wt  = grp.w[blockIdx.y] + (size_t) tile * nquads * kQuadBytes;
+  const uint8_t *__restrict__ act = grp.act[blockIdx.y];
   float *__restrict__         out = grp.out[blockIdx.y];
 
   auto fetch = [&](QuadRegs<WT> (&r)[kLoChunk], int q0) {  // quads q0, q0 + WQ, ... of this wave (clamped: extra ones unused)
@@ -337,7 +338,7 @@ hipError_t launch_weights_to_lane_order(hipStream_t stream, void *dst, const voi
   return hipGetLastError();
 }
 
-hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *const *outs, const void *act,
+hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *const *outs, const void *const *acts,
                                           const void *const *lane_order_weights, const int *ns, int m, int k,
                                           WeightType wt) {
   if (count < 1 || count > kGemvGroupMax) {
@@ -347,15 +348,16 @@ hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *
   int                n_max = 0;
   for (int i = 0; i < count; ++i) {
     if (!matmul_lane_order_fits(ns[i], m, k, wt) || (reinterpret_cast<uintptr_t>(lane_order_weights[i]) & 15) != 0 ||
-        (reinterpret_cast<uintptr_t>(act) & 15) != 0) {
+        (reinterpret_cast<uintptr_t>(acts[i]) & 15) != 0) {
       return hipErrorNotSupported;
     }
     grp.w[i]   = static_cast<const uint8_t *>(lane_order_weights[i]);
+    grp.act[i] = static_cast<const uint8_t *>(acts[i]);
     grp.out[i] = outs[i];
     grp.n[i]   = ns[i];
     n_max      = ns[i] > n_max ? ns[i] : n_max;
   }
-  typedef void (*Kernel)(LaneOrderGroupArgs, const uint8_t *, int, int);
+  typedef void (*Kernel)(LaneOrderGroupArgs, int, int);
   static const Kernel kernels[2][2][2] = {
     { { matmul_lane_order_kernel<8, 1, kQ4_0>, matmul_lane_order_kernel<8, 2, kQ4_0> },
       { matmul_lane_order_kernel<16, 1, kQ4_0>, matmul_lane_order_kernel<16, 2, kQ4_0> } },
@@ -383,8 +385,7 @@ hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *
   const dim3   grid((unsigned) ((n_max / kLoRows + tpw - 1) / tpw), (unsigned) count);
   const int    rows = panel_rows(m);
   const size_t lds  = panel_bytes(k, rows);
-  hipLaunchKernelGGL(kernels[wt == kQ8_0][rows == 16][tpw - 1], grid, dim3(kLoThreads), lds, stream, grp,
-                     static_cast<const uint8_t *>(act), m, k);
+  hipLaunchKernelGGL(kernels[wt == kQ8_0][rows == 16][tpw - 1], grid, dim3(kLoThreads), lds, stream, grp, m, k);
   return hipGetLastError();
 }
 

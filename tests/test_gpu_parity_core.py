@@ -245,8 +245,9 @@ def test_message_batches_same_activation_gemvs(ctx, oracle, wt):
 @pytest.mark.parametrize("wt,m,k", [(wl.GGML_TYPE_Q4_0, 8, 4096), (wl.GGML_TYPE_Q8_0, 3, 1536), (wl.GGML_TYPE_Q4_0, 2, 2048 + 64),
                                     (wl.GGML_TYPE_Q4_0, 12, 4096), (wl.GGML_TYPE_Q8_0, 10, 1536), (wl.GGML_TYPE_Q4_0, 16, 2048 + 64)])
 def test_message_batches_same_activation_small_batches(ctx, oracle, wt, m, k):
-    # The same grouping for 2..8 activation rows: matrices of different n on activation A run as one launch of the
-    # K-sliced kernel (each with its own partial tiles and ticket counters), then the same weights on activation B.
+    # The same grouping for 2..16 activation rows: matrices of different n on activation A, then the same weights on
+    # activation B. Members that take the repacked-weight kernel share launches across A and B (each member reads its
+    # own rows), those of the K-sliced kernel (each with its own partial tiles and ticket counters) only within A or B.
     # Every request must equal its own launch bit for bit, twice in a row (the counters come back to zero).
     rng = wl.rng_for(65, wt * 100 + m)
     op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
