@@ -146,13 +146,17 @@ __global__ __launch_bounds__(256) void q4_0_to_fp6_tiles_kernel(uint8_t *__restr
   sc[96 + c] = 0u;
 }
 
-// one thread per (row of the padded row count, step)
+// One thread per (row of the padded row count, step). A wave takes 8 rows x 8 consecutive steps (lane = row + 8 step):
+// it reads 544 contiguous bytes of each row and writes 128 contiguous bytes of each plane it touches.
 __global__ __launch_bounds__(256) void q8_0_to_fp6_tiles_kernel(uint8_t *__restrict__ tiles, uint32_t *__restrict__ scales,
                                                                 const uint32_t *__restrict__ act, int m, int pairs,
                                                                 int rows_padded) {
-  const size_t t = (size_t) blockIdx.x * 256 + threadIdx.x;
-  const int    r = (int) (t % (size_t) rows_padded), step = (int) (t / (size_t) rows_padded);
-  if (step >= pairs) {
+  const size_t t           = (size_t) blockIdx.x * 256 + threadIdx.x;
+  const int    lane        = (int) (t & 63);
+  const size_t wave        = t >> 6;
+  const int    step_groups = (pairs + 7) / 8;
+  const int    r = (int) (wave / (size_t) step_groups) * 8 + (lane & 7), step = (int) (wave % (size_t) step_groups) * 8 + (lane >> 3);
+  if (r >= rows_padded || step >= pairs) {
     return;
   }
   uint32_t a[17];
@@ -516,7 +520,7 @@ hipError_t launch_gemm_fp6_lds(hipStream_t stream, float *out, const void *act_q
   uint8_t  *tiles   = static_cast<uint8_t *>(act_tiles);
   uint8_t  *scales  = tiles + (size_t) m_tiles * pairs * kATile;
   if (!act_tiles_ready) {
-    const size_t threads = (size_t) m_tiles * 32 * pairs;
+    const size_t threads = (size_t) m_tiles * 4 * ((pairs + 7) / 8) * 64;  // waves of 8 rows x 8 steps
     hipLaunchKernelGGL(q8_0_to_fp6_tiles_kernel, dim3((unsigned) ((threads + 255) / 256)), dim3(256), 0, stream, tiles,
                        reinterpret_cast<uint32_t *>(scales), static_cast<const uint32_t *>(act_q8_0), m, pairs, m_tiles * 32);
     const hipError_t e = hipGetLastError();
