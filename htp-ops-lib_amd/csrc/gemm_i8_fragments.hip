@@ -197,13 +197,13 @@ constexpr int kGiWaves   = 4;
 #define GI_DEPTH_U2 2
 #endif
 
-template <int U>
+template <int UM, int UN>
 struct FragSet {
-  uint4    a[U], b[U];
-  uint32_t da[U], dw[U];
+  uint4    a[UM], b[UN];
+  uint32_t da[UM], dw[UN];
 };
 
-// KSPLIT waves share one tile of U x U units (each takes every KSPLIT-th block); a workgroup holds 4 / KSPLIT tiles
+// KSPLIT waves share one tile of UM x UN units (each takes every KSPLIT-th block); a workgroup holds 4 / KSPLIT tiles
 // that are neighbours along n (they read the same activation fragments).
 // A launch serves up to kGemmGroupMax matmuls of the same row count ("members"): each has its own operands, n and k,
 // and a range of workgroups that starts at a multiple of 8 (so that the XCD of a workgroup is the same function of
@@ -224,12 +224,12 @@ struct FragMembers {
 };
 
 // KSPLIT_T = 0: the split is the member's own (1, 2 or 4), so that members with short and long K share a launch.
-template <int KSPLIT_T, int U>
+template <int KSPLIT_T, int UM, int UN>
 __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembers grp, int m, int m_tiles) {
   // fragment sets in flight per wave: small tiles run one wave per SIMD and must cover the memory latency alone
-  constexpr int kGiDepth = U == 1 ? GI_DEPTH_U1 : GI_DEPTH_U2;
+  constexpr int kGiDepth = UM == 1 ? GI_DEPTH_U1 : GI_DEPTH_U2;
   constexpr int kRedSlots = KSPLIT_T ? (kGiWaves / KSPLIT_T) * (KSPLIT_T - 1) : kGiWaves - 1;
-  __shared__ float red[kRedSlots][U * U][16][64];  // partial accumulators of the waves with ks > 0
+  __shared__ float red[kRedSlots][UM * UN][16][64];  // partial accumulators of the waves with ks > 0
 
   // the wave index (and everything derived from it) is made scalar so that fragment addresses are scalar base +
   // per-lane offset and cost no vector instructions in the loop
@@ -248,16 +248,16 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
   const uint32_t *a_scale   = mem.a_scale, *b_scale = mem.b_scale;
   const int       n = mem.n, nblk = mem.nblk, n_tiles = mem.n_tiles;
   const unsigned  wg = blockIdx.x - mem.wg_begin;
-  // tile of this wave, in units of 32: m tiles mt0 .. mt0 + U - 1; n tiles nt0 .. nt0 + U - 1
+  // tile of this wave, in units of 32: m tiles mt0 .. mt0 + UM - 1; n tiles nt0 .. nt0 + UN - 1
   // Workgroup ids go round-robin over the 8 XCDs (each with its own L2). All row blocks of one column group are
   // given consecutive slots of ONE XCD, so the weight fragments they share are fetched into that L2 once.
-  const int gy = (m_tiles + U - 1) / U, gx = (n_tiles + U * TILES - 1) / (U * TILES);
+  const int gy = (m_tiles + UM - 1) / UM, gx = (n_tiles + UN * TILES - 1) / (UN * TILES);
   const int xcd = wg & 7, slot = wg >> 3;
   const int by = slot % gy, bx = (slot / gy) * 8 + xcd;
   if (bx >= gx) {
     return;  // whole workgroup (the grid is padded to a multiple of 8 column groups)
   }
-  const int mt0 = by * U, nt0 = (bx * TILES + tw) * U;
+  const int mt0 = by * UM, nt0 = (bx * TILES + tw) * UN;
   const bool tile_ok = nt0 < n_tiles;  // mt0 < m_tiles by construction
 
   // Operand streams as buffer resources: a load is then resource (scalar) + per-lane offset (a register that never
@@ -265,35 +265,42 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
   auto resource = [](const void *base) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int) 0xffffffffu, 0x00020000);
   };
-  __amdgpu_buffer_rsrc_t ra[U], rb[U], rsa[U], rsb[U];
-  int                    zero_row[U];  // byte offset of the row of zero scales from this tile's scale rows
+  __amdgpu_buffer_rsrc_t ra[UM], rb[UN], rsa[UM], rsb[UN];
+  int                    zero_row[UM];  // byte offset of the row of zero scales from this tile's scale rows
 #pragma unroll
-  for (int i = 0; i < U; ++i) {
-    const size_t mt = (size_t) min(mt0 + i, m_tiles - 1), nt = (size_t) min(nt0 + i, n_tiles - 1);
+  for (int i = 0; i < UM; ++i) {
+    const size_t mt = (size_t) min(mt0 + i, m_tiles - 1);
     ra[i]       = resource(a_frag + mt * nblk * 64);
-    rb[i]       = resource(b_frag + nt * nblk * 64);
     rsa[i]      = resource(a_scale + mt * nblk * 64);
-    rsb[i]      = resource(b_scale + nt * nblk * 32);
     zero_row[i] = (int) (((size_t) m_tiles - mt) * nblk * 256);
   }
+#pragma unroll
+  for (int j = 0; j < UN; ++j) {
+    const size_t nt = (size_t) min(nt0 + j, n_tiles - 1);
+    rb[j]  = resource(b_frag + nt * nblk * 64);
+    rsb[j] = resource(b_scale + nt * nblk * 32);
+  }
   const int lane16 = lane * 16, lane4 = lane * 4, c4 = c * 4;
-  auto load = [&](FragSet<U> &s, int kb_raw) {
+  auto load = [&](FragSet<UM, UN> &s, int kb_raw) {
     const int  kb   = min(kb_raw, nblk - 1);  // branch-free: blocks past the end repeat the last one ...
     const bool live = kb_raw < nblk;          // ... with activation scales of zero: they add nothing
 #pragma unroll
-    for (int i = 0; i < U; ++i) {
+    for (int i = 0; i < UM; ++i) {
       s.a[i]  = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ra[i], lane16, kb * 1024, 0));
-      s.b[i]  = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb[i], lane16, kb * 1024, 0));
       s.da[i] = __builtin_amdgcn_raw_buffer_load_b32(rsa[i], lane4, live ? kb * 256 : zero_row[i], 0);
-      s.dw[i] = __builtin_amdgcn_raw_buffer_load_b32(rsb[i], c4, kb * 128, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < UN; ++j) {
+      s.b[j]  = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb[j], lane16, kb * 1024, 0));
+      s.dw[j] = __builtin_amdgcn_raw_buffer_load_b32(rsb[j], c4, kb * 128, 0);
     }
   };
 
-  v16f acc[U][U];
+  v16f acc[UM][UN];
 #pragma unroll
-  for (int i = 0; i < U; ++i) {
+  for (int i = 0; i < UM; ++i) {
 #pragma unroll
-    for (int j = 0; j < U; ++j) {
+    for (int j = 0; j < UN; ++j) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         acc[i][j][r] = 0.0f;
@@ -301,7 +308,7 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
     }
   }
 
-  FragSet<U> ring[kGiDepth];
+  FragSet<UM, UN> ring[kGiDepth];
 #pragma unroll
   for (int d = 0; d < kGiDepth; ++d) {
     load(ring[d], ks + d * KSPLIT);
@@ -314,12 +321,12 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
     const uint2 u = make_uint2(packed, 0u);
     return __builtin_bit_cast(v4h, u);
   };
-  auto mfma_sum = [&](const FragSet<U> &s, int i, int j) {
+  auto mfma_sum = [&](const FragSet<UM, UN> &s, int i, int j) {
     const v4i af = { (int) s.a[i].x, (int) s.a[i].y, (int) s.a[i].z, (int) s.a[i].w };
     const v4i bf = { (int) s.b[j].x, (int) s.b[j].y, (int) s.b[j].z, (int) s.b[j].w };
     return __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, zi, 0, 0, 0);
   };
-  auto mfma_scale = [&](const FragSet<U> &s, int i, int j) {
+  auto mfma_scale = [&](const FragSet<UM, UN> &s, int i, int j) {
     return __builtin_amdgcn_mfma_f32_32x32x8f16(scale_operand(s.da[i]), scale_operand(s.dw[j]), zf, 0, 0, 0);
   };
 
@@ -332,13 +339,13 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
 #pragma unroll
     for (int d = 0; d < kGiDepth; ++d) {
 #pragma unroll
-      for (int u = 0; u < U * U; ++u) {
-        constexpr int     LAST = U * U - 1;
-        const int         i = u / U, j = u % U;
+      for (int u = 0; u < UM * UN; ++u) {
+        constexpr int     LAST = UM * UN - 1;
+        const int         i = u / UN, j = u % UN;
         const v16i        sum_cur = sum_next;
         const v16f        scl_cur = scl_next;
-        const FragSet<U> &nx = u < LAST ? ring[d] : ring[(d + 1) % kGiDepth];
-        const int         ni = u < LAST ? (u + 1) / U : 0, nj = u < LAST ? (u + 1) % U : 0;
+        const FragSet<UM, UN> &nx = u < LAST ? ring[d] : ring[(d + 1) % kGiDepth];
+        const int              ni = u < LAST ? (u + 1) / UN : 0, nj = u < LAST ? (u + 1) % UN : 0;
         // The empty volatile asm statements keep their program order and each pins the value it names: the next
         // unit's block sums exist (in registers of their own) before this unit's converts and fmas are done.
         sum_next = mfma_sum(nx, ni, nj);
@@ -365,12 +372,12 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
   // ---- the waves of a tile: ks > 0 park their sums in LDS, ks == 0 adds them in order and stores ----
   if (ks > 0) {
 #pragma unroll
-    for (int i = 0; i < U; ++i) {
+    for (int i = 0; i < UM; ++i) {
 #pragma unroll
-      for (int j = 0; j < U; ++j) {
+      for (int j = 0; j < UN; ++j) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          red[tw * (KSPLIT - 1) + ks - 1][i * U + j][r][lane] = acc[i][j][r];
+          red[tw * (KSPLIT - 1) + ks - 1][i * UN + j][r][lane] = acc[i][j][r];
         }
       }
     }
@@ -378,16 +385,16 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
   __syncthreads();
   if (ks == 0 && tile_ok) {
 #pragma unroll
-    for (int i = 0; i < U; ++i) {
+    for (int i = 0; i < UM; ++i) {
 #pragma unroll
-      for (int j = 0; j < U; ++j) {
+      for (int j = 0; j < UN; ++j) {
         if (mt0 + i < m_tiles && nt0 + j < n_tiles) {
           const int col = (nt0 + j) * 32 + c;
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             float v = acc[i][j][r];
             for (int s = 0; s < KSPLIT - 1; ++s) {
-              v += red[tw * (KSPLIT - 1) + s][i * U + j][r][lane];
+              v += red[tw * (KSPLIT - 1) + s][i * UN + j][r][lane];
             }
             // D[row][col]: col = lane % 32, row = 8 (r / 4) + 4 (lane / 32) + r % 4
             const int row = (mt0 + i) * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
@@ -460,10 +467,16 @@ TileConfig tile_config(int m, int n, int k) {
   return { 2, wave_tiles * 2 < 1536 ? 4 : 2 };
 }
 
+// Column tiles per wave in the small-tile configuration (32 x 32 kSmallUN outputs). Two (one activation fragment
+// serving two products: a quarter less operand traffic, half the waves) measured slower, 57-60 against 47.5 us for
+// the Qwen2-like block at m = 128: these launches want waves more than they want bytes saved.
+constexpr int kSmallUN = 1;
+
 unsigned member_workgroups(int m_tiles, int n_tiles, TileConfig cfg) {
   const unsigned tiles_per_wg = kGiWaves / cfg.ksplit;
+  const unsigned un = cfg.unit == 1 ? kSmallUN : cfg.unit;
   const unsigned gy = (unsigned) ((m_tiles + cfg.unit - 1) / cfg.unit);
-  const unsigned gx = (unsigned) ((n_tiles + cfg.unit * tiles_per_wg - 1) / (cfg.unit * tiles_per_wg));
+  const unsigned gx = (unsigned) ((n_tiles + un * tiles_per_wg - 1) / (un * tiles_per_wg));
   return (gx + 7) / 8 * 8 * gy;
 }
 
@@ -548,11 +561,11 @@ hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *
   }
   grp.count = count;
   if (cfg.unit == 1) {
-    hipLaunchKernelGGL((gemm_i8_fragments_kernel<0, 1>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
+    hipLaunchKernelGGL((gemm_i8_fragments_kernel<0, 1, kSmallUN>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
   } else if (cfg.ksplit == 4) {
-    hipLaunchKernelGGL((gemm_i8_fragments_kernel<4, 2>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
+    hipLaunchKernelGGL((gemm_i8_fragments_kernel<4, 2, 2>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
   } else {
-    hipLaunchKernelGGL((gemm_i8_fragments_kernel<2, 2>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
+    hipLaunchKernelGGL((gemm_i8_fragments_kernel<2, 2, 2>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
   }
   return hipGetLastError();
 }
