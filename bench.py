@@ -92,7 +92,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (every box of this pool has one); --gpus %d is not "
-                 "supported. The path shards by output rows (see DESIGN.md) but no multi-GPU code is built." % args.gpus)
+                 "supported. The path would shard by output rows and KV heads, but no multi-GPU code is built." % args.gpus)
 
     from pyhtpops import api, workloads as wl
     if not os.path.exists(api.LIB_PATH):
