@@ -29,8 +29,9 @@ def sampled_rows(n, count=96):
     return np.unique(np.concatenate([np.linspace(0, n - 1, count).astype(int), [0, 1, n - 2, n - 1]]))
 
 
-def run_layer_message(ctx, oracle, shapes, weights, acts, m, wt, act_rows=None):
-    """One message with one matmul request per entry of `shapes`; returns nothing, asserts parity of every output."""
+def run_layer_message(ctx, oracle, shapes, weights, acts, m, wt, act_rows=None, launches=None):
+    """One message with one matmul request per entry of `shapes`; returns nothing, asserts parity of every output
+    (and, with `launches`, how many submissions the message became)."""
     op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == Q4 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
     h_act = {g: ctx.upload(a) for g, a in acts.items()}
     h_w = [ctx.upload(weights[(n, k)]) for _, n, k in shapes]
@@ -47,6 +48,8 @@ def run_layer_message(ctx, oracle, shapes, weights, acts, m, wt, act_rows=None):
             assert ctx.process_message(msg) == 0
             assert api.message_request_states(msg) == [0] * len(shapes), ctx.last_error()
             assert msg[1] == 1
+            if launches is not None:
+                assert ctx.last_message_submissions() == launches
             for i, (name, n, k) in enumerate(shapes):
                 print("full-size message m=%d %s n=%d k=%d pass %d" % (m, name, n, k, rep), flush=True)
                 got = ctx.read(h_out[i], np.float32, m * n).reshape(m, n)
@@ -73,7 +76,8 @@ def test_llama7b_layer_message_at_full_size(ctx, oracle, llama_weights, m):
     # config 1: q/k/v/o 4096x4096, gate/up 11008x4096, down 4096x11008, seven requests in one message
     rng = wl.rng_for(1, 100 + m)
     acts = {g: oracle.quantize_q8_0(wl.make_activations(rng, m, k)) for g, k in {0: 4096, 1: 4096, 2: 4096, 3: 11008}.items()}
-    run_layer_message(ctx, oracle, wl.LLAMA7B_LAYER, llama_weights, acts, m, Q4)
+    # one row: the seven requests are one launch; eight rows: the six k = 4096 projections share one, down is alone
+    run_layer_message(ctx, oracle, wl.LLAMA7B_LAYER, llama_weights, acts, m, Q4, launches=1 if m == 1 else 2)
 
 
 @pytest.mark.parametrize("n,k", [(11008, 4096), (4096, 11008)])
@@ -114,4 +118,4 @@ def test_qwen2_q8_0_block_message_at_full_size(ctx, oracle, m):
     acts = {0: fused, 1: oracle.quantize_q8_0(wl.make_activations(rng, m, 1536)),
             2: oracle.quantize_q8_0(wl.make_activations(rng, m, 1536)), 3: oracle.quantize_q8_0(wl.make_activations(rng, m, 8960))}
     act_rows = None if m == 1 else np.array([0, 1, 31, 32, 63, 64, 100, 126, 127])
-    run_layer_message(ctx, oracle, wl.QWEN2_1P5B_LAYER, weights, acts, m, Q8, act_rows)
+    run_layer_message(ctx, oracle, wl.QWEN2_1P5B_LAYER, weights, acts, m, Q8, act_rows, launches=1)
