@@ -1235,36 +1235,28 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
     } else if (b.m == 1) {
       e = htpops::launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k, (htpops::WeightType) b.wt);
     } else {
-      // 2..16 rows, same k. Members whose weights have (or get) a repacked copy go to the kernel that streams it,
-      // each with its own activation rows; the others share a launch only when they read the same rows (the 2..4-row
-      // weight stream and the K-sliced kernel stage one set of rows per launch). Which kernel a matrix gets depends
-      // on that matrix alone.
-      bool same_act = true;
-      for (int i = 1; i < b.count; ++i) {
-        same_act = same_act && b.act[i] == a0;
-      }
-      if (same_act && htpops::gemv_rows_fits(b.m, k0, (htpops::WeightType) b.wt)) {
+      // 2..16 rows, same k. Shapes of the 2..4-row weight stream read the same rows (the join rule saw to that) and
+      // are one launch of it. Otherwise members whose weights have (or get) a repacked copy go to the kernel that
+      // streams it, each with its own activation rows; the rest go to the K-sliced kernel, one launch per set of rows
+      // (it stages one). Which kernel a matrix gets depends on that matrix alone.
+      if (htpops::gemv_rows_fits(b.m, k0, (htpops::WeightType) b.wt)) {
         e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, b.count, b.out, a0, b.w, b.n, b.m, k0,
                                                     (htpops::WeightType) b.wt);
       } else {
-        float      *out_a[htpops::kGemvGroupMax], *out_b[htpops::kGemvGroupMax];
-        const void *w_a[htpops::kGemvGroupMax], *w_b[htpops::kGemvGroupMax], *act_a[htpops::kGemvGroupMax];
-        int         n_a[htpops::kGemvGroupMax], n_b[htpops::kGemvGroupMax], count_a = 0, count_b = 0;
-        const bool  rows_kernel = htpops::gemv_rows_fits(b.m, k0, (htpops::WeightType) b.wt);
+        float      *out_a[htpops::kGemvGroupMax];
+        const void *w_a[htpops::kGemvGroupMax], *act_a[htpops::kGemvGroupMax];
+        int         n_a[htpops::kGemvGroupMax], count_a = 0;
+        bool        sliced[htpops::kGemvGroupMax] = {};
         for (int i = 0; i < b.count; ++i) {
           const void *lw = nullptr;
-          int         r  = HTPOPS_OK;
-          if (!rows_kernel) {
-            r = lane_order_weights(ctx, b.w[i], b.act[i], b.m, k0, b.n[i], b.wt, &lw);
-          }
-          if (r) {
+          if (int r = lane_order_weights(ctx, b.w[i], b.act[i], b.m, k0, b.n[i], b.wt, &lw)) {
             b.hdr[i]->state = r;
           } else if (lw) {
             out_a[count_a] = b.out[i], w_a[count_a] = lw, act_a[count_a] = b.act[i], n_a[count_a++] = b.n[i];
-          } else if (same_act && !rows_kernel && b.m <= kSkinnyGroupMaxM) {
-            out_b[count_b] = b.out[i], w_b[count_b] = b.w[i], n_b[count_b++] = b.n[i];
+          } else if (b.m <= kSkinnyGroupMaxM) {
+            sliced[i] = true;
           } else {
-            // different rows than the rest, or more rows than the K-sliced group launch takes: on its own
+            // more rows than the K-sliced group launch takes: on its own
             b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act[i], b.w[i], b.m, k0, b.n[i], b.wt);
           }
         }
@@ -1273,12 +1265,24 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
           e = htpops::launch_matmul_lane_order_group(ctx->stream, count_a, out_a, act_a, w_a, n_a, b.m, k0,
                                                      (htpops::WeightType) b.wt);
         }
-        if (e == hipSuccess && count_b > 0) {
+        for (int first = 0; first < b.count && e == hipSuccess && ret == HTPOPS_OK; ++first) {
+          if (!sliced[first]) {
+            continue;
+          }
+          float      *out_b[htpops::kGemvGroupMax];
+          const void *w_b[htpops::kGemvGroupMax];
+          int         n_b[htpops::kGemvGroupMax], count_b = 0;
+          for (int i = first; i < b.count; ++i) {  // everybody left that reads the rows of `first`
+            if (sliced[i] && b.act[i] == b.act[first]) {
+              out_b[count_b] = b.out[i], w_b[count_b] = b.w[i], n_b[count_b++] = b.n[i];
+              sliced[i] = false;
+            }
+          }
           const size_t ws = htpops::matmul_skinny_group_workspace_bytes(count_b, n_b, b.m, k0);
           if (int r = ensure_workspace(ctx, ws)) {
             ret = r;
           } else {
-            e = htpops::launch_matmul_skinny_group(ctx->stream, count_b, out_b, a0, w_b, n_b, b.m, k0,
+            e = htpops::launch_matmul_skinny_group(ctx->stream, count_b, out_b, b.act[first], w_b, n_b, b.m, k0,
                                                    (htpops::WeightType) b.wt, ctx->workspace, ctx->tickets, kTicketSlots);
           }
         }
@@ -1337,7 +1341,8 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
     }
   }
   bool join = b.count > 0 && b.count < htpops::kGemvGroupMax && b.wt == wt && b.m == p->m &&
-              (p->m == 1 || many_rows || b.k[0] == p->k);
+              (p->m == 1 || many_rows ||
+               (b.k[0] == p->k && (b.act[0] == act || !htpops::gemv_rows_fits(p->m, p->k, (htpops::WeightType) wt))));
   for (int i = 0; join && i < b.count; ++i) {
     const size_t wi = weight_bytes((size_t) b.n[i], (size_t) b.k[i], b.wt), oi = (size_t) b.m * b.n[i] * 4;
     const size_t ai = q8_0_bytes((size_t) b.m, (size_t) b.k[i]);
