@@ -478,6 +478,222 @@ hipError_t launch_instance(hipStream_t stream, float *out, const uint8_t *a_tile
   return hipGetLastError();
 }
 
+
+// ---- 128 x 128 tiles, eight waves ---------------------------------------------------------------------------------
+// For shapes with enough such tiles. A step moves 21 transfers of 1 KiB for 32 units instead of 17 for 16, and the
+// kernel is written for four waves per SIMD (two workgroups of eight waves per compute unit, at most 128 registers):
+// matrix and vector instructions of ONE wave issue far below the rate a SIMD sustains, so it is the number of
+// resident waves that keeps its pipes busy. A wave owns 64 x 32 outputs; per unit it issues the block-sum
+// instruction, the scale-product instruction and the sixteen fmas in that order, without the 128 x 64 kernel's
+// second set of result registers. (Two workgroups sharing a tile, one per half of K, with the partial tiles exchanged
+// through memory, did not pay on shapes with fewer tiles: 71 against 62 us at 512 x 11008 x 4096.)
+constexpr int kWdWaves  = 8;
+constexpr int kWdOffW   = 4 * kATile;
+constexpr int kWdOffSa  = kWdOffW + 4 * kWTile;
+constexpr int kWdStage  = kWdOffSa + kSaTile;
+constexpr int kWdStages = 3;
+constexpr int kWdDma    = 12 + 8 + 1;  // activation planes, weight KiB, row scales
+constexpr int kWdPerWave = (kWdDma + kWdWaves - 1) / kWdWaves;
+constexpr int kWdMinTiles = 512;  // 128 x 128 output tiles from which this kernel is used
+
+__global__ __launch_bounds__(kWdWaves *kWave, 2) void gemm_fp6_lds_wide_kernel(
+    float *__restrict__ out, const uint8_t *__restrict__ a_tiles, const uint8_t *__restrict__ a_scales,
+    const uint8_t *__restrict__ w_tiles, int m, int n, int pairs, int tiles_m, int tiles_n) {
+  constexpr int NS = kWdStages, kStage = kWdStage;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const int lane = threadIdx.x & 63;
+  const int u    = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = u >> 2, wn = u & 3;  // rows 64 wm .. + 63, columns 32 wn .. + 31 of the tile
+
+  // Consecutive workgroups of one XCD (each has its own L2): the row blocks of a column tile, which read the same
+  // weights.
+  const int xcd = blockIdx.x % 8, j = blockIdx.x / 8;
+  const int tile_m = j % tiles_m, tile_n = (j / tiles_m) * 8 + xcd;
+  if (tile_n >= tiles_n) {
+    return;  // whole workgroup
+  }
+  const int steps = pairs;
+  auto step_of = [&](int x) { return min(x, steps - 1); };  // (DMA for steps past the end re-reads the last one)
+
+  const uint32_t ring0 = (uint32_t) (uintptr_t) lds;
+  auto dma16 = [&](const uint8_t *base, uint32_t lane_off, uint32_t dst) {
+    asm volatile("s_mov_b32 m0, %2\n s_nop 0\n global_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(dst) : "memory");
+  };
+  const int last_mt = (m + 31) / 32 - 1;
+  const int last_ct = (n + 31) / 32 - 1;  // tiles past the end re-read the last one (their outputs are not stored)
+  const uint8_t *src[kWdPerWave];
+  uint32_t       dst[kWdPerWave], stride[kWdPerWave];
+#pragma unroll
+  for (int i = 0; i < kWdPerWave; ++i) {
+    const int p = u + kWdWaves * i;  // (p >= kWdDma: this wave has one transfer less; the entry is never used)
+    if (p < 12) {
+      const size_t rt = (size_t) min(tile_m * 4 + p / 3, last_mt);
+      src[i]    = a_tiles + rt * pairs * kATile + (p % 3) * 1024;
+      dst[i]    = ring0 + (p / 3) * kATile + (p % 3) * 1024;
+      stride[i] = kATile;
+    } else if (p < 20) {
+      const int    q  = p - 12;
+      const size_t ct = (size_t) min(tile_n * 4 + q / 2, last_ct);
+      src[i]    = w_tiles + ct * pairs * kWTile + (q % 2) * 1024;
+      dst[i]    = ring0 + kWdOffW + (q / 2) * kWTile + (q % 2) * 1024;
+      stride[i] = kWTile;
+    } else {
+      src[i]    = a_scales + (size_t) tile_m * pairs * kSaTile;
+      dst[i]    = ring0 + kWdOffSa;
+      stride[i] = kSaTile;
+    }
+  }
+  const int      mine   = (kWdDma - u + kWdWaves - 1) / kWdWaves;  // transfers of this wave per step: 3 or 2
+  const uint32_t lane16 = lane * 16;
+  auto issue_group = [&](int x, int stage) {
+    const size_t   s  = (size_t) step_of(x);
+    const uint32_t so = (uint32_t) stage * kStage;
+#pragma unroll
+    for (int i = 0; i < kWdPerWave; ++i) {
+      if (i < kWdPerWave - 1 || mine == kWdPerWave) {
+        dma16(src[i] + s * stride[i], lane16, dst[i] + so);
+      }
+    }
+  };
+  auto wait_oldest_group = [&]() {  // (see the 128 x 64 kernel: one younger group may stay in flight)
+    static_assert((NS - 2) * kWdPerWave < 16, "vmcnt fits the low four bits");
+    if (mine == kWdPerWave) {
+      __builtin_amdgcn_s_waitcnt(0x0070 | ((NS - 2) * kWdPerWave));
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0070 | ((NS - 2) * (kWdPerWave - 1)));
+    }
+  };
+#pragma unroll
+  for (int x = 0; x < NS - 1; ++x) {
+    issue_group(x, x);
+  }
+
+  const v16f zero_f = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 };
+  v16f       acc0 = zero_f, acc1 = zero_f;  // rows 64 wm .. + 31 and 64 wm + 32 .. + 63
+  const int  scale_a = (lane >> 5) ? 127 + 3 : 127 + 7, scale_b = 127 + 3;
+  const uint32_t a_rd  = ring0 + (2 * wm) * kATile + lane * 16;                    // lower row tile at + kATile; block 1 at + 2048
+  const uint32_t a_rd8 = ring0 + (2 * wm) * kATile + 1024 + lane * 8;              // tails; block 1 at + 512
+  const uint32_t w_rd  = ring0 + kWdOffW + wn * kWTile + (lane & 31) * 16;         // block 1 at + 1024
+  const uint32_t w_rd8 = ring0 + kWdOffW + wn * kWTile + 512 + (lane & 31) * 8;    // tails; block 1 at + 256
+  const uint32_t sb_rd = ring0 + kWdOffW + wn * kWTile + 1536 + lane * 4;          // block 1 at + 256
+  const uint32_t sa_rd = ring0 + kWdOffSa + (2 * wm) * 256 + (lane & 31) * 8;      // lower row tile at + 256
+
+  typedef __attribute__((address_space(3))) const uint8_t *lds_ptr;
+  auto lds_v4i = [](uint32_t addr, int off) {
+    return *reinterpret_cast<__attribute__((address_space(3))) const v4i *>((lds_ptr) (uintptr_t) addr + off);
+  };
+  auto lds_v2i = [](uint32_t addr, int off) {
+    return *reinterpret_cast<__attribute__((address_space(3))) const v2i *>((lds_ptr) (uintptr_t) addr + off);
+  };
+  auto lds_u32 = [](uint32_t addr, int off) {
+    return *reinterpret_cast<__attribute__((address_space(3))) const uint32_t *>((lds_ptr) (uintptr_t) addr + off);
+  };
+  auto operand = [](v4i lo, v2i hi) {
+    v8i f;
+    f[0] = lo[0], f[1] = lo[1], f[2] = lo[2], f[3] = lo[3], f[4] = hi[0], f[5] = hi[1];
+    return f;
+  };
+#define HTPOPS_FENCE __builtin_amdgcn_sched_barrier(0)
+  auto unit = [&](v16f &acc, const v8i &fa, const v8i &fb, v4h sa, v4h sb) {
+    const v16f s = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa, fb, zero_f, 2, 2, 0, scale_a, 0, scale_b);
+    const v16f c = __builtin_amdgcn_mfma_f32_32x32x8f16(sa, sb, zero_f, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      acc[i] = __builtin_fmaf(s[i], c[i], acc[i]);
+    }
+    HTPOPS_FENCE;
+  };
+  // One step out of stage ST (a compile-time constant: every LDS offset is an immediate). Block 1's operands are read
+  // from LDS while block 0 is being computed.
+  auto step = [&](auto stage_tag, int t) {
+    constexpr int ST = decltype(stage_tag)::value;
+    constexpr int so = ST * kStage;
+    wait_oldest_group();  // this wave's transfers of step t have landed, then everybody's
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    v2i a0hi, a1hi, b0hi;  // block 0: row tiles 0 / 1, the column tile
+    asm volatile("ds_read_b64 %0, %3 offset:%c5\n ds_read_b64 %1, %3 offset:%c6\n ds_read_b64 %2, %4 offset:%c7"
+                 : "=&v"(a0hi), "=&v"(a1hi), "=&v"(b0hi)
+                 : "v"(a_rd8), "v"(w_rd8), "i"(so), "i"(so + kATile), "i"(so)
+                 : "memory");
+    const v4i      a0lo = lds_v4i(a_rd, so), a1lo = lds_v4i(a_rd, so + kATile), b0lo = lds_v4i(w_rd, so);
+    const v2i      sa0 = lds_v2i(sa_rd, so), sa1 = lds_v2i(sa_rd, so + 256);  // (scale pair, 0): operands as they are
+    const uint32_t sb0 = lds_u32(sb_rd, so), sb1 = lds_u32(sb_rd, so + 256);
+    // everybody has left step t - 1: its stage takes step t + NS - 1
+    issue_group(t + NS - 1, (ST + NS - 1) % NS);
+    // (the wait as a builtin, so that the compiler knows these reads have landed; the empty statement ties the
+    // registers written by the reads above to it)
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    asm volatile("" : "+v"(a0hi), "+v"(a1hi), "+v"(b0hi)::"memory");
+    v2i c0hi, c1hi, d0hi;  // block 1, the same three
+    asm volatile("ds_read_b64 %0, %3 offset:%c5\n ds_read_b64 %1, %3 offset:%c6\n ds_read_b64 %2, %4 offset:%c7"
+                 : "=&v"(c0hi), "=&v"(c1hi), "=&v"(d0hi)
+                 : "v"(a_rd8), "v"(w_rd8), "i"(so + 512), "i"(so + kATile + 512), "i"(so + 256)
+                 : "memory");
+    const v4i c0lo = lds_v4i(a_rd, so + 2048), c1lo = lds_v4i(a_rd, so + kATile + 2048), d0lo = lds_v4i(w_rd, so + 1024);
+    const v4h sa0_op = __builtin_bit_cast(v4h, sa0), sa1_op = __builtin_bit_cast(v4h, sa1);
+    const v4h sb0_op = __builtin_bit_cast(v4h, make_uint2(sb0, 0u)), sb1_op = __builtin_bit_cast(v4h, make_uint2(sb1, 0u));
+    {
+      const v8i fa0 = operand(a0lo, a0hi), fa1 = operand(a1lo, a1hi), fb = operand(b0lo, b0hi);
+      HTPOPS_FENCE;
+      unit(acc0, fa0, fb, sa0_op, sb0_op);
+      unit(acc1, fa1, fb, sa1_op, sb0_op);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    asm volatile("" : "+v"(c0hi), "+v"(c1hi), "+v"(d0hi)::"memory");
+    {
+      const v8i fa0 = operand(c0lo, c0hi), fa1 = operand(c1lo, c1hi), fb = operand(d0lo, d0hi);
+      HTPOPS_FENCE;
+      unit(acc0, fa0, fb, sa0_op, sb1_op);
+      unit(acc1, fa1, fb, sa1_op, sb1_op);
+    }
+  };
+  for (int t = 0; t < steps; t += NS) {
+    step(std::integral_constant<int, 0>(), t);
+    if (t + 1 < steps) {
+      step(std::integral_constant<int, 1>(), t + 1);
+    }
+    if (t + 2 < steps) {
+      step(std::integral_constant<int, 2>(), t + 2);
+    }
+  }
+#undef HTPOPS_FENCE
+  __builtin_amdgcn_s_waitcnt(0x0070);  // (transfers of steps past the end must have landed before LDS is released)
+
+  const int col = tile_n * 128 + wn * 32 + (lane & 31);
+  if (col < n) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = tile_m * 128 + wm * 64 + (i / 4) * 8 + (lane >> 5) * 4 + (i & 3);
+      if (row < m) {
+        out[(size_t) row * n + col] = acc0[i];
+      }
+      if (row + 32 < m) {
+        out[(size_t) (row + 32) * n + col] = acc1[i];
+      }
+    }
+  }
+}
+
+hipError_t launch_wide(hipStream_t stream, float *out, const uint8_t *a_tiles, const uint8_t *a_scales, const uint8_t *w_tiles,
+                       int m, int n, int pairs) {
+  const int    tiles_m = (m + 127) / 128, tiles_n = (n + 127) / 128;
+  const size_t lds     = (size_t) kWdStages * kWdStage;
+  const dim3   grid((unsigned) (((tiles_n + 7) / 8) * 8 * tiles_m));
+  static bool  raised  = false;
+  if (!raised) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_fp6_lds_wide_kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) {
+      return e;
+    }
+    raised = true;
+  }
+  hipLaunchKernelGGL(gemm_fp6_lds_wide_kernel, grid, dim3(kWdWaves * kWave), lds, stream, out, a_tiles, a_scales, w_tiles, m,
+                     n, pairs, tiles_m, tiles_n);
+  return hipGetLastError();
+}
+
 }  // namespace
 
 bool gemm_fp6_lds_fits(int m, int k, int n) {
@@ -529,6 +745,11 @@ hipError_t launch_gemm_fp6_lds(hipStream_t stream, float *out, const void *act_q
     }
   }
   const uint8_t *wt      = static_cast<const uint8_t *>(weight_tiles);
+  // 128 x 128 tiles from where they fill two workgroups per compute unit (10 % faster there: 84 against 95 us at
+  // 512 x 16384 x 4096)
+  if ((long) ((m + 127) / 128) * ((n + 127) / 128) >= kWdMinTiles) {
+    return launch_wide(stream, out, tiles, scales, wt, m, n, pairs);
+  }
   const long     tiles64 = (long) ((m + kBM - 1) / kBM) * ((n + 63) / 64);
   // 128 x 64 tiles: a K group is 4 waves (one per SIMD) and one ring of three stages, and a compute unit holds three
   // rings: one group per workgroup when the tiles alone give every compute unit three workgroups, otherwise up to

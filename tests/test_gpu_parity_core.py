@@ -537,6 +537,36 @@ def test_gemm_fp6_whole_tiles_on_every_workgroup(ctx, oracle):
         assert np.abs(gemv[0] - got[r]).max() <= 2e-5 * np.abs(gemv).max()
 
 
+def test_gemm_fp6_128x128_tiles_ragged_and_exact(ctx, oracle):
+    # 1000 x 8200 outputs = 8 x 65 tiles of 128 x 128 (the last ones ragged both ways), from where the FP6 path uses
+    # its 128 x 128 kernel; k = 192 is three steps, one pass of its ring. Unit scales first (block sums exact, the
+    # extremes -127 x -8 included), then random scales against the oracle on sampled rows and against the one-row
+    # kernel.
+    rng = wl.rng_for(68, 0)
+    m, k, n = 1000, 192, 8200
+    w = wl.make_q4_0_weights(rng, n, k).reshape(n, k // 32, -1)
+    a = ctx.run_quantize_q8_0(wl.make_activations(rng, m, k)).reshape(m, k // 32, -1)
+    w1, a1 = w.copy(), a.copy()
+    w1[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    a1[:, :, 0:2] = np.array([1.0], np.float16).view(np.uint8)
+    w1[n - 1, :, 2:] = 0x00  # all weights -8
+    a1[m - 1, :, 2:] = np.int8(-127).view(np.uint8)
+    w1, a1, w, a = w1.reshape(n, -1), a1.reshape(m, -1), w.reshape(n, -1), a.reshape(m, -1)
+    got = ctx.run_mat_mul(a1, w1, m, k, n, wl.GGML_TYPE_Q4_0)
+    _, qa = wl.q8_0_split(a1, k)
+    _, qw = wl.q4_0_split(w1, k)
+    assert np.array_equal(got, (qa.astype(np.int64) @ qw.astype(np.int64).T).astype(np.float32))
+    assert got[m - 1, n - 1] == 32512.0 * (k // 32)
+    got = ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0)
+    assert np.array_equal(ctx.run_mat_mul(a, w, m, k, n, wl.GGML_TYPE_Q4_0), got)
+    rows = [0, 31, 64, 127, 128, 500, 895, 896, 999]
+    want64, mag = oracle.mat_mul_q8_0_act_f64(a[rows], w, len(rows), k, n, wl.GGML_TYPE_Q4_0)
+    assert np.all(np.abs(got[rows] - want64) <= MATMUL_RTOL * mag)
+    for r in (77, 999):
+        gemv = ctx.run_mat_mul(a[r:r + 1], w, 1, k, n, wl.GGML_TYPE_Q4_0)
+        assert np.abs(gemv[0] - got[r]).max() <= 2e-5 * np.abs(gemv).max()
+
+
 def test_gemm_weight_conversion_cache_follows_the_weights(ctx, oracle):
     # Many-row matmuls run on weights converted to MFMA operand order. For buffers the context allocated the converted
     # copy is cached and must be dropped when the buffer is rewritten; for caller-owned (registered) memory nothing is
