@@ -553,100 +553,6 @@ hipError_t launch_gemv_members(hipStream_t stream, GemvMembers &grp) {
   return hipGetLastError();
 }
 
-// the argument table of the two-to-four-row kernel below: members share the activation rows, blockIdx.y picks one
-struct GemvGroupArgs {
-  const uint32_t *w[kGemvGroupMax];
-  float          *out[kGemvGroupMax];
-  int             n[kGemvGroupMax];
-};
-
-// ---- two to four activation rows ------------------------------------------------------------------------------------
-// The same stream over the weights with M activation rows staged in LDS: a lane prepares its activation pairs of all M
-// rows once and dots every weight pair it loads against each of them (the nibble unpacking is shared), so the weights
-// are still read once and the extra rows cost vector-ALU work only. One row set per wave, 256 threads.
-template <int WT, int G, int ITERS, int M>
-__global__ __launch_bounds__(kThreads) void gemv_rows_shared_act_kernel(GemvGroupArgs grp, const uint32_t *__restrict__ act,
-                                                                        int pairs) {
-  extern __shared__ __attribute__((aligned(16))) uint32_t act_lds[];
-  constexpr int PD    = Pair<WT>::kDwords;
-  constexpr int SLOTS = kWave / G;
-  const int                    n   = grp.n[blockIdx.y];
-  float *__restrict__          out = grp.out[blockIdx.y];
-  const uint32_t *__restrict__ w   = grp.w[blockIdx.y];
-  if ((int) (blockIdx.x * (kWaves * SLOTS)) >= n) {
-    return;  // whole workgroup: this member has fewer rows than the widest one
-  }
-  const int    lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  const int    g = lane % G, slot = lane / G;
-  const int    row = (blockIdx.x * kWaves + wave) * SLOTS + slot;
-  const size_t row_dwords = (size_t) pairs * PD;
-
-  // the M activation rows are contiguous: requested first (they come from L2), in 16-byte pieces, the last piece slid
-  // back to the end; then the weights, which are in flight during the LDS exchange
-  constexpr int ACT_SLOTS = (M * 192 * kActPairDwords * 4 + kThreads * 16 - 1) / (kThreads * 16);
-  const int     act_bytes = M * pairs * kActPairDwords * 4;
-  uint4         areg[ACT_SLOTS];
-  int           aoff[ACT_SLOTS];
-#pragma unroll
-  for (int j = 0; j < ACT_SLOTS; ++j) {
-    const int off = (threadIdx.x + j * kThreads) * 16;
-    aoff[j]       = min(off, act_bytes - 16);
-    const u32x4_a4 v = *reinterpret_cast<const u32x4_a4 *>(reinterpret_cast<const uint8_t *>(act) + aoff[j]);
-    areg[j]       = make_uint4(v.x, v.y, v.z, v.w);
-  }
-  uint32_t  wreg[ITERS][PD];
-  const int wrow = min(row, n - 1);
-#pragma unroll
-  for (int i = 0; i < ITERS; ++i) {
-    const int p = min(g + i * G, pairs - 1);
-    load_dwords<PD>(wreg[i], w + (size_t) wrow * row_dwords + (size_t) p * PD);
-  }
-#pragma unroll
-  for (int j = 0; j < ACT_SLOTS; ++j) {
-    uint32_t *dst = act_lds + aoff[j] / 4;
-    dst[0] = areg[j].x, dst[1] = areg[j].y, dst[2] = areg[j].z, dst[3] = areg[j].w;
-  }
-  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the LDS writes have landed; vmcnt is left alone
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-
-  float acc[M];
-#pragma unroll
-  for (int mm = 0; mm < M; ++mm) {
-    acc[mm] = 0.0f;
-  }
-#pragma unroll
-  for (int i = 0; i < ITERS; ++i) {
-    const int     p    = g + i * G;
-    const bool    live = row < n && p < pairs;
-    constexpr int kScale1 = WT == kQ4_0 ? 4 : 8;  // dword holding the second block's scale (upper half)
-    wreg[i][0]       = live ? wreg[i][0] : 0u;
-    wreg[i][kScale1] = live ? wreg[i][kScale1] : 0u;
-#pragma unroll
-    for (int mm = 0; mm < M; ++mm) {
-      uint32_t a[kActPairDwords];
-      if (p < pairs) {
-#pragma unroll
-        for (int e = 0; e < kActPairDwords; ++e) {
-          a[e] = act_lds[(mm * pairs + p) * kActPairDwords + e];
-        }
-      } else {
-        zero_dwords<kActPairDwords>(a);
-      }
-      ActPair<WT> ap;
-      prepare(ap, a);
-      acc[mm] += pair_dot(wreg[i], ap);
-    }
-  }
-#pragma unroll
-  for (int mm = 0; mm < M; ++mm) {
-    const float v = group_sum_dpp<G>(acc[mm]);
-    if (g == G - 1 && row < n) {
-      out[(size_t) mm * n + row] = v;
-    }
-  }
-}
-
 // Catch-all (odd block counts, any m): one wave per weight row, 16-bit loads, scalar integer arithmetic.
 template <int WT>
 __global__ __launch_bounds__(kThreads) void gemv_blocks_generic_kernel(float *__restrict__ out,
@@ -688,48 +594,123 @@ __global__ __launch_bounds__(kThreads) void gemv_blocks_generic_kernel(float *__
   }
 }
 
-template <int WT, int G, int ITERS>
-hipError_t launch_rows_shared_act(hipStream_t stream, const GemvGroupArgs &grp, int count, const uint32_t *act, int pairs,
-                                  int m) {
-  constexpr int rows_per_group = kWaves * (kWave / G);
-  int           n_max          = 0;
-  for (int i = 0; i < count; ++i) {
-    n_max = grp.n[i] > n_max ? grp.n[i] : n_max;
+// ---- two to four activation rows, held in registers ---------------------------------------------------------------
+// The stream over the weights again, arranged so that nothing is shared and nothing waits: a wave owns one chunk of 64
+// pairs of K (lane = pair), prepares its pairs of all M activation rows ONCE into registers, and then walks a range of
+// weight rows -- one pair per lane and row, requested three rows ahead -- dotting each against the M rows (the nibble
+// unpacking is shared between them). A workgroup is the C waves that cover all of K for the same range of weight
+// rows: with C = 1 a wave stores its sums itself, otherwise the chunk sums of a row meet in LDS after the walk and are
+// added in chunk order. The extra rows cost vector-ALU work only (about 5 us per row and Llama-7B layer, which is why
+// the kernel is used up to three rows); every member of a launch brings its own activation rows.
+struct RowsMember {
+  const uint32_t *w;
+  const uint32_t *act;  // M rows
+  float          *out;  // [M][n]
+  int             n;
+  int             block0;  // first workgroup of this member
+};
+
+struct RowsMembers {
+  RowsMember m[kGemvGroupMax];
+  int        count;
+};
+
+constexpr int kRowsDepth   = 3;   // weight rows in flight per wave
+constexpr int kRowsMaxWalk = 64;  // weight rows per workgroup at most (the LDS image of the chunk sums)
+
+template <int WT, int M, int C>
+__global__ __launch_bounds__(C *kWave) void gemv_rows_in_registers_kernel(RowsMembers grp, int pairs, int walk) {
+  constexpr int PD = Pair<WT>::kDwords;
+  __shared__ float red[C > 1 ? kRowsMaxWalk * C * M : 1];
+  int mi = 0;
+#pragma unroll
+  for (int i = 1; i < kGemvGroupMax; ++i) {
+    mi = (i < grp.count && (int) blockIdx.x >= grp.m[i].block0) ? i : mi;
   }
-  const dim3   grid((unsigned) ((n_max + rows_per_group - 1) / rows_per_group), (unsigned) count);
-  const size_t lds = (size_t) m * pairs * kActPairDwords * 4;
-  switch (m) {
-    case 2:
-      hipLaunchKernelGGL((gemv_rows_shared_act_kernel<WT, G, ITERS, 2>), grid, dim3(kThreads), lds, stream, grp, act, pairs);
-      break;
-    case 3:
-      hipLaunchKernelGGL((gemv_rows_shared_act_kernel<WT, G, ITERS, 3>), grid, dim3(kThreads), lds, stream, grp, act, pairs);
-      break;
-    case 4:
-      hipLaunchKernelGGL((gemv_rows_shared_act_kernel<WT, G, ITERS, 4>), grid, dim3(kThreads), lds, stream, grp, act, pairs);
-      break;
-    default:
-      return hipErrorNotSupported;
+  const RowsMember &mem = grp.m[mi];
+  const int                    n   = mem.n;
+  const uint32_t *__restrict__ w   = mem.w;
+  float *__restrict__          out = mem.out;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int c    = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // chunk of K
+  const int row_begin = ((int) blockIdx.x - mem.block0) * walk;
+  const int row_end   = min(n, row_begin + walk);
+  const int  p    = c * kWave + lane;
+  const bool live = p < pairs;
+  const int  pc   = min(p, pairs - 1);
+  const size_t row_dwords = (size_t) pairs * PD;
+
+  // the first weight rows are requested before the activations are prepared
+  uint32_t        wreg[kRowsDepth][PD];
+  const uint32_t *wp = w + (size_t) pc * PD;
+#pragma unroll
+  for (int d = 0; d < kRowsDepth; ++d) {
+    load_dwords<PD>(wreg[d], wp + (size_t) min(row_begin + d, n - 1) * row_dwords);
   }
-  return hipGetLastError();
+  ActPair<WT> ap[M];
+#pragma unroll
+  for (int mm = 0; mm < M; ++mm) {
+    uint32_t a[kActPairDwords];
+    load_dwords<kActPairDwords>(a, mem.act + ((size_t) mm * pairs + pc) * kActPairDwords);
+    prepare(ap[mm], a);
+    if (!live) {
+      ap[mm].d0 = 0.0f, ap[mm].d1 = 0.0f;  // a pair past the end of the row adds nothing
+    }
+  }
+
+  for (int r0 = row_begin; r0 < row_end; r0 += kRowsDepth) {
+#pragma unroll
+    for (int d = 0; d < kRowsDepth; ++d) {
+      const int r = r0 + d;
+      if (r < row_end) {  // (uniform)
+        float v[M];
+#pragma unroll
+        for (int mm = 0; mm < M; ++mm) {
+          v[mm] = pair_dot(wreg[d], ap[mm]);
+        }
+        // the slot is free: its next row
+        load_dwords<PD>(wreg[d], wp + (size_t) min(r + kRowsDepth, n - 1) * row_dwords);
+#pragma unroll
+        for (int mm = 0; mm < M; ++mm) {
+          v[mm] = group_sum_dpp<kWave>(v[mm]);
+        }
+        if (lane == kWave - 1) {
+#pragma unroll
+          for (int mm = 0; mm < M; ++mm) {
+            if (C == 1) {
+              out[(size_t) mm * n + r] = v[mm];
+            } else {
+              red[((r - row_begin) * C + c) * M + mm] = v[mm];
+            }
+          }
+        }
+      }
+    }
+  }
+  if (C > 1) {
+    __syncthreads();
+    for (int t = threadIdx.x; t < (row_end - row_begin) * M; t += C * kWave) {
+      const int r = t / M, mm = t % M;
+      float     total = red[(r * C) * M + mm];
+#pragma unroll
+      for (int cc = 1; cc < C; ++cc) {
+        total += red[(r * C + cc) * M + mm];
+      }
+      out[(size_t) mm * n + row_begin + r] = total;
+    }
+  }
 }
 
-template <int WT>
-hipError_t launch_gemv_rows_shared(hipStream_t stream, const GemvGroupArgs &grp, int count, const uint32_t *act, int pairs,
-                                   int m) {
-  if (pairs <= 16) {
-    return launch_rows_shared_act<WT, 16, 1>(stream, grp, count, act, pairs, m);
+template <int WT, int C>
+hipError_t launch_rows_in_registers(hipStream_t stream, const RowsMembers &grp, int blocks, int m, int pairs, int walk) {
+  const dim3 grid((unsigned) blocks), block((unsigned) (C * kWave));
+  switch (m) {
+    case 2: hipLaunchKernelGGL((gemv_rows_in_registers_kernel<WT, 2, C>), grid, block, 0, stream, grp, pairs, walk); break;
+    case 3: hipLaunchKernelGGL((gemv_rows_in_registers_kernel<WT, 3, C>), grid, block, 0, stream, grp, pairs, walk); break;
+    case 4: hipLaunchKernelGGL((gemv_rows_in_registers_kernel<WT, 4, C>), grid, block, 0, stream, grp, pairs, walk); break;
+    default: return hipErrorNotSupported;
   }
-  if (pairs <= 32) {
-    return launch_rows_shared_act<WT, 32, 1>(stream, grp, count, act, pairs, m);
-  }
-  if (pairs <= 64) {
-    return launch_rows_shared_act<WT, 64, 1>(stream, grp, count, act, pairs, m);
-  }
-  if (pairs <= 128) {
-    return launch_rows_shared_act<WT, 64, 2>(stream, grp, count, act, pairs, m);
-  }
-  return launch_rows_shared_act<WT, 64, 3>(stream, grp, count, act, pairs, m);
+  return hipGetLastError();
 }
 
 template <int WT>
@@ -796,28 +777,49 @@ hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *cons
 }
 
 bool gemv_rows_fits(int m, int k, WeightType wt) {
-  // measured on Llama-7B shapes: with Q8_0 weights the kernel beats the K-sliced one up to 4 rows; with Q4_0 weights
-  // (whose activation pairs cost a sum of their bytes each) it beats the repacked-weight kernel at 2 rows only
+  // measured on Llama-7B (Q4_0) and Qwen2-1.5B (Q8_0) layers: up to three rows the kernel beats the repacked-weight and
+  // K-sliced kernels (32.8 / 35.8 against 38.9 / 39.3 us and 15.8 / 18.0 against 18.3 / 18.5 us); every further row
+  // costs it as much again while theirs come free up to eight
+  (void) wt;
   const int nblk = k / kQK;
-  return m >= 2 && m <= (wt == kQ4_0 ? 2 : 4) && k % (2 * kQK) == 0 && nblk / 2 <= kSharedActMaxPairs &&
+  return m >= 2 && m <= 3 && k % (2 * kQK) == 0 && nblk / 2 <= kSharedActMaxPairs &&
          env_int("HTPOPS_GEMV_ROWS_KERNEL", 1) != 0;
 }
 
-hipError_t launch_gemv_rows_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *act,
+hipError_t launch_gemv_rows_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *const *acts,
                                            const void *const *weights, const int *ns, int m, int k, WeightType wt) {
-  if (count < 1 || count > kGemvGroupMax || !gemv_rows_fits(m, k, wt) || (reinterpret_cast<uintptr_t>(act) & 3) != 0) {
+  const int pairs = k / (2 * kQK);
+  if (count < 1 || count > kGemvGroupMax || m < 2 || m > 4 || k % (2 * kQK) != 0 || pairs > kSharedActMaxPairs) {
     return hipErrorNotSupported;
   }
-  GemvGroupArgs grp = {};
+  const int chunks = (pairs + kWave - 1) / kWave;
+  long      rows   = 0;
   for (int i = 0; i < count; ++i) {
-    if ((reinterpret_cast<uintptr_t>(weights[i]) & 3) != 0) {
+    if (ns[i] < 1 || ((reinterpret_cast<uintptr_t>(weights[i]) | reinterpret_cast<uintptr_t>(acts[i])) & 3) != 0) {
       return hipErrorNotSupported;
     }
-    grp.w[i] = static_cast<const uint32_t *>(weights[i]), grp.out[i] = outs[i], grp.n[i] = ns[i];
+    rows += ns[i];
   }
-  const int pairs = k / kQK / 2;
-  return wt == kQ4_0 ? launch_gemv_rows_shared<kQ4_0>(stream, grp, count, static_cast<const uint32_t *>(act), pairs, m) :
-                       launch_gemv_rows_shared<kQ8_0>(stream, grp, count, static_cast<const uint32_t *>(act), pairs, m);
+  // about twelve waves per compute unit, each with at least eight weight rows to set its prepared activations against
+  // (measured on the Llama-7B layer at two rows: 4 / 8 / 16 / 32 rows per wave 45.9 / 41.9 / 48.6 / 75.4 us)
+  int walk = kRowsMaxWalk;
+  while (walk > 8 && rows / walk * chunks < 3072) {
+    walk /= 2;
+  }
+  RowsMembers grp = {};
+  grp.count       = count;
+  int blocks      = 0;
+  for (int i = 0; i < count; ++i) {
+    grp.m[i].w = static_cast<const uint32_t *>(weights[i]), grp.m[i].act = static_cast<const uint32_t *>(acts[i]);
+    grp.m[i].out = outs[i], grp.m[i].n = ns[i], grp.m[i].block0 = blocks;
+    blocks += (ns[i] + walk - 1) / walk;
+  }
+#define HTPOPS_ROWS(WT) \
+  (chunks == 1 ? launch_rows_in_registers<WT, 1>(stream, grp, blocks, m, pairs, walk) : \
+   chunks == 2 ? launch_rows_in_registers<WT, 2>(stream, grp, blocks, m, pairs, walk) : \
+                 launch_rows_in_registers<WT, 3>(stream, grp, blocks, m, pairs, walk))
+  return wt == kQ4_0 ? HTPOPS_ROWS(kQ4_0) : HTPOPS_ROWS(kQ8_0);
+#undef HTPOPS_ROWS
 }
 
 }  // namespace htpops

@@ -297,11 +297,13 @@ def test_small_batch_repeated_launches_are_bit_identical(ctx):
         assert np.abs(one[0] - first[r]).max() <= 2e-5 * np.abs(one).max()
 
 
-@pytest.mark.parametrize("wt,m", [(wl.GGML_TYPE_Q4_0, 2), (wl.GGML_TYPE_Q8_0, 2), (wl.GGML_TYPE_Q8_0, 3), (wl.GGML_TYPE_Q8_0, 4)])
-@pytest.mark.parametrize("k,n", [(64, 1), (128, 33), (1024, 100), (4096, 4096), (11008, 272), (12288, 64), (2048 + 64, 1000)])
-def test_two_to_four_rows_on_the_decode_kernels_weight_stream(ctx, oracle, monkeypatch, wt, m, k, n):
-    # 2 rows (Q4_0) and 2..4 rows (Q8_0) run the decode kernel's stream over the weights with the rows staged in LDS.
-    # Against the oracle, against the kernels they replace (HTPOPS_GEMV_ROWS_KERNEL=0), bit for bit on a repeat, and
+@pytest.mark.parametrize("wt,m", [(wl.GGML_TYPE_Q4_0, 2), (wl.GGML_TYPE_Q4_0, 3), (wl.GGML_TYPE_Q8_0, 2), (wl.GGML_TYPE_Q8_0, 3)])
+@pytest.mark.parametrize("k,n", [(64, 1), (128, 33), (1024, 100), (4096, 4096), (4096 + 64, 70), (8192, 9), (11008, 272),
+                                 (12288, 64), (2048 + 64, 1000)])
+def test_two_and_three_rows_on_the_decode_kernels_weight_stream(ctx, oracle, monkeypatch, wt, m, k, n):
+    # 2 and 3 rows run the decode kernel's stream over the weights with the rows held in registers: one, two or three
+    # waves per weight row (k <= 4096, <= 8192, <= 12288), rows past the last whole walk of a workgroup, one lane of a
+    # chunk only (k = 4096 + 64). Against the oracle, against the kernels they replace (HTPOPS_GEMV_ROWS_KERNEL=0), bit for bit on a repeat, and
     # every row against the one-row kernel (same block sums and lane mapping; the compiler is free to fuse the scale
     # multiplications differently in the two kernels, so to rounding).
     rng = wl.rng_for(69, wt * 1000 + m * 100 + k + n)
@@ -748,6 +750,40 @@ def test_message_groups_independent_many_row_matmuls(ctx, oracle, wt):
         assert ctx.last_message_submissions() == 2
         assert np.array_equal(ctx.read(hos[0], np.float32, m * 192).reshape(m, 192),
                               ctx.run_mat_mul(acts[1], ws[3], m, 1536, 192, wt))
+    finally:
+        for h in has + hws + hos:
+            ctx.release(h)
+
+
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+@pytest.mark.parametrize("m", [2, 3, 8])
+def test_message_groups_independent_few_row_matmuls(ctx, oracle, wt, m):
+    # Few-row matmuls of the same k that nothing orders share a launch although they read different activation rows
+    # (2, 3 rows: the weight stream with the rows in registers; 8: the kernel over repacked weights for Q4_0, one
+    # launch per set of rows otherwise). Every request must equal its own launch bit for bit.
+    rng = wl.rng_for(76, wt * 10 + m)
+    op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
+    k = 1024
+    ns = [256, 64, 48, 256, 1000]
+    act_of = [0, 0, 0, 1, 2]
+    ws = [wl.make_weights(rng, n, k, wt) for n in ns]
+    acts = [oracle.quantize_q8_0(wl.make_activations(rng, m, k)) for _ in range(3)]
+    has = [ctx.upload(a) for a in acts]
+    hws = [ctx.upload(w) for w in ws]
+    hos = [ctx.alloc(m * n * 4) for n in ns]
+    try:
+        msg = api.build_message([_mm(op, ho, has[g], hw, m, k, n) for ho, g, hw, n in zip(hos, act_of, hws, ns)])
+        for _ in range(2):
+            for ho, n in zip(hos, ns):
+                ctx.write(ho, np.full(m * n, np.nan, np.float32))
+            assert ctx.process_message(msg) == 0
+            assert api.message_request_states(msg) == [0] * len(ns), ctx.last_error()
+            assert ctx.last_message_submissions() == 1
+            for ho, g, w, n in zip(hos, act_of, ws, ns):
+                got = ctx.read(ho, np.float32, m * n).reshape(m, n)
+                assert np.array_equal(got, ctx.run_mat_mul(acts[g], w, m, k, n, wt)), "a request differs from its own launch"
+                want, mag = oracle.mat_mul_q8_0_act_f64(acts[g], w, m, k, n, wt)
+                assert np.all(np.abs(got - want) <= MATMUL_RTOL * mag)
     finally:
         for h in has + hws + hos:
             ctx.release(h)
