@@ -598,15 +598,17 @@ __global__ __launch_bounds__(kThreads) void gemv_blocks_generic_kernel(float *__
 // The stream over the weights again, arranged so that nothing is shared and nothing waits: a wave owns one chunk of 64
 // pairs of K (lane = pair), prepares its pairs of all M activation rows ONCE into registers, and then walks a range of
 // weight rows -- one pair per lane and row, requested three rows ahead -- dotting each against the M rows (the nibble
-// unpacking is shared between them). A workgroup is the C waves that cover all of K for the same range of weight
-// rows: with C = 1 a wave stores its sums itself, otherwise the chunk sums of a row meet in LDS after the walk and are
-// added in chunk order. The extra rows cost vector-ALU work only (about 5 us per row and Llama-7B layer, which is why
-// the kernel is used up to three rows); every member of a launch brings its own activation rows.
+// unpacking is shared between them). The C = 1, 2 or 3 waves that cover all of K for the same range of weight rows are
+// a team: with C = 1 a wave stores its sums itself, otherwise the chunk sums of a row meet in LDS after the walk and
+// are added in chunk order. A workgroup has three waves: three teams of short rows, or one team (and an idle wave
+// when C = 2). The extra rows cost vector-ALU work only (about 5 us per row and Llama-7B layer, which is why the
+// kernel is used up to three rows); every member of a launch brings its own activation rows and row length.
 struct RowsMember {
   const uint32_t *w;
   const uint32_t *act;  // M rows
   float          *out;  // [M][n]
   int             n;
+  int             pairs;   // block pairs per row (k / 64)
   int             block0;  // first workgroup of this member
 };
 
@@ -616,24 +618,29 @@ struct RowsMembers {
 };
 
 constexpr int kRowsDepth   = 3;   // weight rows in flight per wave
-constexpr int kRowsMaxWalk = 64;  // weight rows per workgroup at most (the LDS image of the chunk sums)
+constexpr int kRowsMaxWalk = 64;  // weight rows per team at most (the LDS image of the chunk sums)
+constexpr int kRowsWaves   = 3;   // = the most chunks a row has (kSharedActMaxPairs / 64)
 
-template <int WT, int M, int C>
-__global__ __launch_bounds__(C *kWave) void gemv_rows_in_registers_kernel(RowsMembers grp, int pairs, int walk) {
+template <int WT, int M>
+__global__ __launch_bounds__(kRowsWaves *kWave) void gemv_rows_in_registers_kernel(RowsMembers grp, int walk) {
   constexpr int PD = Pair<WT>::kDwords;
-  __shared__ float red[C > 1 ? kRowsMaxWalk * C * M : 1];
+  __shared__ float red[kRowsMaxWalk * kRowsWaves * M];
   int mi = 0;
 #pragma unroll
   for (int i = 1; i < kGemvGroupMax; ++i) {
     mi = (i < grp.count && (int) blockIdx.x >= grp.m[i].block0) ? i : mi;
   }
   const RowsMember &mem = grp.m[mi];
-  const int                    n   = mem.n;
-  const uint32_t *__restrict__ w   = mem.w;
-  float *__restrict__          out = mem.out;
+  const int                    n     = mem.n;
+  const int                    pairs = mem.pairs;
+  const uint32_t *__restrict__ w     = mem.w;
+  float *__restrict__          out   = mem.out;
   const int lane = threadIdx.x & (kWave - 1);
-  const int c    = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // chunk of K
-  const int row_begin = ((int) blockIdx.x - mem.block0) * walk;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int C    = (pairs + kWave - 1) / kWave;  // chunks of K = waves of a team
+  const int c = wave % C, team = wave / C, teams = kRowsWaves / C;
+  // (a wave without a team -- the third one when C = 2 -- and a team past the member's last row walk nothing)
+  const int row_begin = team < teams ? min(n, (((int) blockIdx.x - mem.block0) * teams + team) * walk) : n;
   const int row_end   = min(n, row_begin + walk);
   const int  p    = c * kWave + lane;
   const bool live = p < pairs;
@@ -687,27 +694,27 @@ __global__ __launch_bounds__(C *kWave) void gemv_rows_in_registers_kernel(RowsMe
       }
     }
   }
-  if (C > 1) {
+  if (C > 1) {  // (the same for the whole workgroup: one team)
     __syncthreads();
-    for (int t = threadIdx.x; t < (row_end - row_begin) * M; t += C * kWave) {
+    const int rb = min(n, ((int) blockIdx.x - mem.block0) * walk), re = min(n, rb + walk);  // the team's rows
+    for (int t = threadIdx.x; t < (re - rb) * M; t += kRowsWaves * kWave) {
       const int r = t / M, mm = t % M;
       float     total = red[(r * C) * M + mm];
-#pragma unroll
       for (int cc = 1; cc < C; ++cc) {
         total += red[(r * C + cc) * M + mm];
       }
-      out[(size_t) mm * n + row_begin + r] = total;
+      out[(size_t) mm * n + rb + r] = total;
     }
   }
 }
 
-template <int WT, int C>
-hipError_t launch_rows_in_registers(hipStream_t stream, const RowsMembers &grp, int blocks, int m, int pairs, int walk) {
-  const dim3 grid((unsigned) blocks), block((unsigned) (C * kWave));
+template <int WT>
+hipError_t launch_rows_in_registers(hipStream_t stream, const RowsMembers &grp, int blocks, int m, int walk) {
+  const dim3 grid((unsigned) blocks), block((unsigned) (kRowsWaves * kWave));
   switch (m) {
-    case 2: hipLaunchKernelGGL((gemv_rows_in_registers_kernel<WT, 2, C>), grid, block, 0, stream, grp, pairs, walk); break;
-    case 3: hipLaunchKernelGGL((gemv_rows_in_registers_kernel<WT, 3, C>), grid, block, 0, stream, grp, pairs, walk); break;
-    case 4: hipLaunchKernelGGL((gemv_rows_in_registers_kernel<WT, 4, C>), grid, block, 0, stream, grp, pairs, walk); break;
+    case 2: hipLaunchKernelGGL((gemv_rows_in_registers_kernel<WT, 2>), grid, block, 0, stream, grp, walk); break;
+    case 3: hipLaunchKernelGGL((gemv_rows_in_registers_kernel<WT, 3>), grid, block, 0, stream, grp, walk); break;
+    case 4: hipLaunchKernelGGL((gemv_rows_in_registers_kernel<WT, 4>), grid, block, 0, stream, grp, walk); break;
     default: return hipErrorNotSupported;
   }
   return hipGetLastError();
@@ -778,8 +785,9 @@ hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *cons
 
 bool gemv_rows_fits(int m, int k, WeightType wt) {
   // measured on Llama-7B (Q4_0) and Qwen2-1.5B (Q8_0) layers: up to three rows the kernel beats the repacked-weight and
-  // K-sliced kernels (32.8 / 35.8 against 38.9 / 39.3 us and 15.8 / 18.0 against 18.3 / 18.5 us); every further row
-  // costs it as much again while theirs come free up to eight
+  // K-sliced kernels (28.2 / 31.8 against 38.9 / 39.3 us and 13.3 / 14.8 against 18.3 / 18.5 us), at four rows they
+  // are level (39.0 against 38.2, 18.4 against 18.6 us); every further row costs it as much again while theirs come
+  // free up to eight
   (void) wt;
   const int nblk = k / kQK;
   return m >= 2 && m <= 3 && k % (2 * kQK) == 0 && nblk / 2 <= kSharedActMaxPairs &&
@@ -787,39 +795,38 @@ bool gemv_rows_fits(int m, int k, WeightType wt) {
 }
 
 hipError_t launch_gemv_rows_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *const *acts,
-                                           const void *const *weights, const int *ns, int m, int k, WeightType wt) {
-  const int pairs = k / (2 * kQK);
-  if (count < 1 || count > kGemvGroupMax || m < 2 || m > 4 || k % (2 * kQK) != 0 || pairs > kSharedActMaxPairs) {
+                                           const void *const *weights, const int *ns, int m, const int *ks,
+                                           WeightType wt) {
+  if (count < 1 || count > kGemvGroupMax || m < 2 || m > 4) {
     return hipErrorNotSupported;
   }
-  const int chunks = (pairs + kWave - 1) / kWave;
-  long      rows   = 0;
+  long waves_per_row = 0;  // summed over all weight rows
   for (int i = 0; i < count; ++i) {
-    if (ns[i] < 1 || ((reinterpret_cast<uintptr_t>(weights[i]) | reinterpret_cast<uintptr_t>(acts[i])) & 3) != 0) {
+    const int pairs = ks[i] / (2 * kQK);
+    if (ns[i] < 1 || ks[i] % (2 * kQK) != 0 || pairs < 1 || pairs > kSharedActMaxPairs ||
+        ((reinterpret_cast<uintptr_t>(weights[i]) | reinterpret_cast<uintptr_t>(acts[i])) & 3) != 0) {
       return hipErrorNotSupported;
     }
-    rows += ns[i];
+    waves_per_row += (long) ns[i] * ((pairs + kWave - 1) / kWave);
   }
   // about twelve waves per compute unit, each with at least eight weight rows to set its prepared activations against
   // (measured on the Llama-7B layer at two rows: 4 / 8 / 16 / 32 rows per wave 45.9 / 41.9 / 48.6 / 75.4 us)
   int walk = kRowsMaxWalk;
-  while (walk > 8 && rows / walk * chunks < 3072) {
+  while (walk > 8 && waves_per_row / walk < 3072) {
     walk /= 2;
   }
   RowsMembers grp = {};
   grp.count       = count;
   int blocks      = 0;
   for (int i = 0; i < count; ++i) {
+    const int pairs = ks[i] / (2 * kQK);
+    const int rows_per_block = walk * (kRowsWaves / ((pairs + kWave - 1) / kWave));
     grp.m[i].w = static_cast<const uint32_t *>(weights[i]), grp.m[i].act = static_cast<const uint32_t *>(acts[i]);
-    grp.m[i].out = outs[i], grp.m[i].n = ns[i], grp.m[i].block0 = blocks;
-    blocks += (ns[i] + walk - 1) / walk;
+    grp.m[i].out = outs[i], grp.m[i].n = ns[i], grp.m[i].pairs = pairs, grp.m[i].block0 = blocks;
+    blocks += (ns[i] + rows_per_block - 1) / rows_per_block;
   }
-#define HTPOPS_ROWS(WT) \
-  (chunks == 1 ? launch_rows_in_registers<WT, 1>(stream, grp, blocks, m, pairs, walk) : \
-   chunks == 2 ? launch_rows_in_registers<WT, 2>(stream, grp, blocks, m, pairs, walk) : \
-                 launch_rows_in_registers<WT, 3>(stream, grp, blocks, m, pairs, walk))
-  return wt == kQ4_0 ? HTPOPS_ROWS(kQ4_0) : HTPOPS_ROWS(kQ8_0);
-#undef HTPOPS_ROWS
+  return wt == kQ4_0 ? launch_rows_in_registers<kQ4_0>(stream, grp, blocks, m, walk) :
+                       launch_rows_in_registers<kQ8_0>(stream, grp, blocks, m, walk);
 }
 
 }  // namespace htpops

@@ -530,7 +530,7 @@ int run_few_rows(htpops_context *ctx, float *dst, const void *act, const void *w
   // hipErrorNotSupported from a launcher means "this kernel does not take the shape": try the next one. Any other
   // failure is reported.
   if (htpops::gemv_rows_fits(m, k, (htpops::WeightType) wt) && aligned(act, 4) && aligned(weight, 4)) {
-    const hipError_t e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, 1, &dst, &act, &weight, &n, m, k,
+    const hipError_t e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, 1, &dst, &act, &weight, &n, m, &k,
                                                                  (htpops::WeightType) wt);
     if (e == hipSuccess) {
       return HTPOPS_OK;
@@ -1234,12 +1234,12 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
     } else if (b.m == 1) {
       e = htpops::launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k, (htpops::WeightType) b.wt);
     } else {
-      // 2..16 rows, same k. Two or three rows are one launch of the weight stream that keeps them in registers, each
-      // member with its own rows. Otherwise members whose weights have (or get) a repacked copy go to the kernel that
-      // streams it, again each with its own activation rows; the rest go to the K-sliced kernel, one launch per set
-      // of rows (it stages one). Which kernel a matrix gets depends on that matrix alone.
+      // 2..16 rows. Two or three rows are one launch of the weight stream that keeps them in registers, each member
+      // with its own rows and row length. Otherwise (same k) members whose weights have (or get) a repacked copy go
+      // to the kernel that streams it, again each with its own activation rows; the rest go to the K-sliced kernel,
+      // one launch per set of rows (it stages one). Which kernel a matrix gets depends on that matrix alone.
       if (htpops::gemv_rows_fits(b.m, k0, (htpops::WeightType) b.wt)) {
-        e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.m, k0,
+        e = htpops::launch_gemv_rows_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.m, b.k,
                                                     (htpops::WeightType) b.wt);
       } else {
         float      *out_a[htpops::kGemvGroupMax];
@@ -1340,7 +1340,9 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
     }
   }
   bool join = b.count > 0 && b.count < htpops::kGemvGroupMax && b.wt == wt && b.m == p->m &&
-              (p->m == 1 || many_rows || b.k[0] == p->k);
+              (p->m == 1 || many_rows || b.k[0] == p->k ||
+               (htpops::gemv_rows_fits(p->m, p->k, (htpops::WeightType) wt) &&
+                htpops::gemv_rows_fits(b.m, b.k[0], (htpops::WeightType) wt)));
   for (int i = 0; join && i < b.count; ++i) {
     const size_t wi = weight_bytes((size_t) b.n[i], (size_t) b.k[i], b.wt), oi = (size_t) b.m * b.n[i] * 4;
     const size_t ai = q8_0_bytes((size_t) b.m, (size_t) b.k[i]);

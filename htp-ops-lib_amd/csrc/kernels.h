@@ -31,12 +31,13 @@ hipError_t launch_gemv_q8_0_act(hipStream_t stream, float *out, const void *act,
 constexpr int kGemvGroupMax = 8;
 hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *const *acts,
                                       const void *const *weights, const int *ns, const int *ks, WeightType wt);
-// 2 <= m <= 4 activation rows against several weight matrices of the same k in one launch: the decode kernel's stream
-// over the weights with the rows held in registers; member i reads the rows acts[i] (k % 64 == 0, k <= 12288, 4-byte
-// aligned buffers; else hipErrorNotSupported)
+// 2 <= m <= 4 activation rows against several weight matrices in one launch: the decode kernel's stream over the
+// weights with the rows held in registers; member i reads the rows acts[i] of length ks[i] (k % 64 == 0, k <= 12288,
+// 4-byte aligned buffers; else hipErrorNotSupported)
 bool       gemv_rows_fits(int m, int k, WeightType wt);  // whether the launch below is the kernel of choice
 hipError_t launch_gemv_rows_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *const *acts,
-                                           const void *const *weights, const int *ns, int m, int k, WeightType wt);
+                                           const void *const *weights, const int *ns, int m, const int *ks,
+                                           WeightType wt);
 // small-batch path (m <= 32, k % 64 == 0, else hipErrorNotSupported): one pass over the weight bytes for all rows,
 // block dots on v_mfma_i32_32x32x32_i8
 // `workspace` (matmul_skinny_workspace_bytes) holds per-slice partial tiles, `tickets` is an array of

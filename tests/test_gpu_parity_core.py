@@ -761,25 +761,27 @@ def test_message_groups_independent_few_row_matmuls(ctx, oracle, wt, m):
     # Few-row matmuls of the same k that nothing orders share a launch although they read different activation rows
     # (2, 3 rows: the weight stream with the rows in registers; 8: the kernel over repacked weights for Q4_0, one
     # launch per set of rows otherwise). Every request must equal its own launch bit for bit.
+    # With two and three rows the members may also differ in k (one, two and three waves per weight row here).
     rng = wl.rng_for(76, wt * 10 + m)
     op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
-    k = 1024
-    ns = [256, 64, 48, 256, 1000]
-    act_of = [0, 0, 0, 1, 2]
-    ws = [wl.make_weights(rng, n, k, wt) for n in ns]
-    acts = [oracle.quantize_q8_0(wl.make_activations(rng, m, k)) for _ in range(3)]
+    ns = [256, 64, 48, 256, 1000, 130]
+    act_of = [0, 0, 0, 1, 2, 3]
+    ks = [1024] * 4 + ([1024, 1024] if m == 8 else [8192, 11008])
+    act_k = [1024, 1024, ks[4], ks[5]]
+    ws = [wl.make_weights(rng, n, k, wt) for n, k in zip(ns, ks)]
+    acts = [oracle.quantize_q8_0(wl.make_activations(rng, m, k)) for k in act_k]
     has = [ctx.upload(a) for a in acts]
     hws = [ctx.upload(w) for w in ws]
     hos = [ctx.alloc(m * n * 4) for n in ns]
     try:
-        msg = api.build_message([_mm(op, ho, has[g], hw, m, k, n) for ho, g, hw, n in zip(hos, act_of, hws, ns)])
+        msg = api.build_message([_mm(op, ho, has[g], hw, m, k, n) for ho, g, hw, n, k in zip(hos, act_of, hws, ns, ks)])
         for _ in range(2):
             for ho, n in zip(hos, ns):
                 ctx.write(ho, np.full(m * n, np.nan, np.float32))
             assert ctx.process_message(msg) == 0
             assert api.message_request_states(msg) == [0] * len(ns), ctx.last_error()
             assert ctx.last_message_submissions() == 1
-            for ho, g, w, n in zip(hos, act_of, ws, ns):
+            for ho, g, w, n, k in zip(hos, act_of, ws, ns, ks):
                 got = ctx.read(ho, np.float32, m * n).reshape(m, n)
                 assert np.array_equal(got, ctx.run_mat_mul(acts[g], w, m, k, n, wt)), "a request differs from its own launch"
                 want, mag = oracle.mat_mul_q8_0_act_f64(acts[g], w, m, k, n, wt)
