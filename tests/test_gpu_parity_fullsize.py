@@ -71,13 +71,14 @@ def llama_weights():
     return {(n, k): wl.make_q4_0_weights(rng, n, k) for n, k in {(n, k) for _, n, k in wl.LLAMA7B_LAYER}}
 
 
-@pytest.mark.parametrize("m", [1, 8])
+@pytest.mark.parametrize("m", [1, 2, 3, 8])
 def test_llama7b_layer_message_at_full_size(ctx, oracle, llama_weights, m):
     # config 1: q/k/v/o 4096x4096, gate/up 11008x4096, down 4096x11008, seven requests in one message
     rng = wl.rng_for(1, 100 + m)
     acts = {g: oracle.quantize_q8_0(wl.make_activations(rng, m, k)) for g, k in {0: 4096, 1: 4096, 2: 4096, 3: 11008}.items()}
-    # one row: the seven requests are one launch; eight rows: the six k = 4096 projections share one, down is alone
-    run_layer_message(ctx, oracle, wl.LLAMA7B_LAYER, llama_weights, acts, m, Q4, launches=1 if m == 1 else 2)
+    # up to three rows the seven requests are one launch; eight rows: the six k = 4096 projections share one, down is
+    # alone
+    run_layer_message(ctx, oracle, wl.LLAMA7B_LAYER, llama_weights, acts, m, Q4, launches=1 if m <= 3 else 2)
 
 
 @pytest.mark.parametrize("n,k", [(11008, 4096), (4096, 11008)])
@@ -103,7 +104,7 @@ def test_prefill_gemm_m512_at_full_size(ctx, oracle, llama_weights, n, k):
     assert np.array_equal(ctx.run_mat_mul(x, w, m, k, n, Q4, act_is_f32=True), got)
 
 
-@pytest.mark.parametrize("m", [1, 128])
+@pytest.mark.parametrize("m", [1, 2, 128])
 def test_qwen2_q8_0_block_message_at_full_size(ctx, oracle, m):
     # config 4: RMSNorm (1536, eps 1e-6, weight N(1, 0.1)) -> Q8_0 -> Q8_0-weight matmuls 1536x1536 (q, o), 256x1536
     # (k, v), 8960x1536 (gate, up), 1536x8960 (down)
@@ -117,5 +118,5 @@ def test_qwen2_q8_0_block_message_at_full_size(ctx, oracle, m):
     assert np.array_equal(fused, oracle.quantize_q8_0(normed))  # the chain on the GPU's own normalized rows: bit-exact
     acts = {0: fused, 1: oracle.quantize_q8_0(wl.make_activations(rng, m, 1536)),
             2: oracle.quantize_q8_0(wl.make_activations(rng, m, 1536)), 3: oracle.quantize_q8_0(wl.make_activations(rng, m, 8960))}
-    act_rows = None if m == 1 else np.array([0, 1, 31, 32, 63, 64, 100, 126, 127])
+    act_rows = None if m <= 8 else np.array([0, 1, 31, 32, 63, 64, 100, 126, 127])
     run_layer_message(ctx, oracle, wl.QWEN2_1P5B_LAYER, weights, acts, m, Q8, act_rows, launches=1)
