@@ -21,6 +21,8 @@
 #include "device_utils.h"
 #include "kernels.h"
 
+#include <algorithm>
+
 namespace htpops {
 
 namespace {
@@ -537,26 +539,35 @@ hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *
   FragMembers grp;
   unsigned    total = 0;
   TileConfig  cfg   = { 0, 0 };
+  // Workgroups start in block order: the members whose waves have the most blocks to walk go first, so that the launch
+  // ends on short waves (members are independent of each other, their order is free).
+  int order[kGemmGroupMax];
   for (int i = 0; i < count; ++i) {
+    order[i] = i;
+  }
+  auto walk = [&](int i) { return ks[i] <= 0 || ns[i] <= 0 ? 0 : ks[i] / 32 / tile_config(m, ns[i], ks[i]).ksplit; };
+  std::stable_sort(order, order + count, [&](int a, int b) { return walk(a) > walk(b); });
+  for (int slot = 0; slot < count; ++slot) {
+    const int i = order[slot];
     if (ks[i] <= 0 || ks[i] % 32 != 0 || ns[i] <= 0) {
       return hipErrorInvalidValue;
     }
     const TileConfig c = tile_config(m, ns[i], ks[i]);
-    if (i > 0 && (c.unit != cfg.unit || (c.unit != 1 && c.ksplit != cfg.ksplit))) {
+    if (slot > 0 && (c.unit != cfg.unit || (c.unit != 1 && c.ksplit != cfg.ksplit))) {
       return hipErrorNotSupported;  // every member runs in the configuration it would get alone
     }
     cfg               = c;
     const int nblk = ks[i] / 32, n_tiles = (ns[i] + 31) / 32;
-    grp.m[i].a_frag   = static_cast<const uint4 *>(act_fragments[i]);
-    grp.m[i].a_scale  = scales_of(act_fragments[i], (size_t) m_tiles, (size_t) nblk);
-    grp.m[i].b_frag   = static_cast<const uint4 *>(weight_fragments[i]);
-    grp.m[i].b_scale  = scales_of(weight_fragments[i], (size_t) n_tiles, (size_t) nblk);
-    grp.m[i].out      = outs[i];
-    grp.m[i].n        = ns[i];
-    grp.m[i].nblk     = nblk;
-    grp.m[i].n_tiles  = n_tiles;
-    grp.m[i].ksplit   = c.ksplit;
-    grp.m[i].wg_begin = total;
+    grp.m[slot].a_frag   = static_cast<const uint4 *>(act_fragments[i]);
+    grp.m[slot].a_scale  = scales_of(act_fragments[i], (size_t) m_tiles, (size_t) nblk);
+    grp.m[slot].b_frag   = static_cast<const uint4 *>(weight_fragments[i]);
+    grp.m[slot].b_scale  = scales_of(weight_fragments[i], (size_t) n_tiles, (size_t) nblk);
+    grp.m[slot].out      = outs[i];
+    grp.m[slot].n        = ns[i];
+    grp.m[slot].nblk     = nblk;
+    grp.m[slot].n_tiles  = n_tiles;
+    grp.m[slot].ksplit   = c.ksplit;
+    grp.m[slot].wg_begin = total;
     total += member_workgroups(m_tiles, n_tiles, cfg);
   }
   grp.count = count;
