@@ -166,15 +166,16 @@ def main():
 
     def time_layers(m, steps, warmup):
         msgs = [layer_message(l, m) for l in range(LAYERS)]
+        handles = [ctx.message_handle(msg) for msg in msgs]
         # steps are enqueued without waiting in between (several messages in flight on the in-order stream);
         # completion of every message is published after the timed region
         for s in range(warmup):
-            ctx.enqueue_message(msgs[s % LAYERS])
+            ctx.enqueue_message_handle(handles[s % LAYERS])
         ctx.synchronize()
         t0 = time.perf_counter()
         ctx.timer_start()
         for s in range(steps):
-            ctx.enqueue_message(msgs[s % LAYERS])
+            ctx.enqueue_message_handle(handles[s % LAYERS])
         ev_ms = ctx.timer_stop_ms()
         ctx.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3

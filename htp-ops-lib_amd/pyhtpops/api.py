@@ -267,6 +267,15 @@ class Context:
         buf = (ctypes.c_char * len(msg)).from_buffer(msg)
         return self.lib.htpops_enqueue_message(self._ctx, ctypes.cast(buf, ctypes.c_void_p), len(msg))
 
+    def message_handle(self, msg):
+        """(address, length) of a message buffer for enqueue_message_handle: a driver loop that submits the same
+        messages again and again pays the buffer lookup once. `msg` must stay alive as long as the handle is used."""
+        buf = (ctypes.c_char * len(msg)).from_buffer(msg)
+        return ctypes.cast(buf, ctypes.c_void_p), len(msg)
+
+    def enqueue_message_handle(self, handle):
+        return self.lib.htpops_enqueue_message(self._ctx, handle[0], handle[1])
+
     def finish_message(self, msg):
         buf = (ctypes.c_char * len(msg)).from_buffer(msg)
         return self.lib.htpops_finish_message(self._ctx, ctypes.cast(buf, ctypes.c_void_p))
