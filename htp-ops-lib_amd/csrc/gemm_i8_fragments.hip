@@ -22,6 +22,7 @@
 #include "kernels.h"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace htpops {
 
@@ -227,21 +228,29 @@ struct FragMembers {
 
 // KSPLIT_T = 0: the split is the member's own (1, 2 or 4), so that members with short and long K share a launch.
 template <int KSPLIT_T, int UM, int UN>
-__global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembers grp, int m, int m_tiles) {
+struct RedSlots {
+  static constexpr int kValue = KSPLIT_T ? (kGiWaves / KSPLIT_T) * (KSPLIT_T - 1) : kGiWaves - 1;
+};
+
+__device__ __forceinline__ const FragMember &member_of_workgroup(const FragMembers &grp) {
+  int mi = 0;
+  for (int i = 1; i < grp.count; ++i) {
+    mi = blockIdx.x >= grp.m[i].wg_begin ? i : mi;
+  }
+  return grp.m[mi];
+}
+
+// one workgroup's share of a member; `red`: RedSlots x (UM UN) x 16 x 64 floats of LDS
+template <int KSPLIT_T, int UM, int UN>
+__device__ __forceinline__ void fragments_workgroup(const FragMember &mem, int m, int m_tiles, float *red_lds) {
   // fragment sets in flight per wave: small tiles run one wave per SIMD and must cover the memory latency alone
   constexpr int kGiDepth = UM == 1 ? GI_DEPTH_U1 : GI_DEPTH_U2;
-  constexpr int kRedSlots = KSPLIT_T ? (kGiWaves / KSPLIT_T) * (KSPLIT_T - 1) : kGiWaves - 1;
-  __shared__ float red[kRedSlots][UM * UN][16][64];  // partial accumulators of the waves with ks > 0
+  float (*red)[UM * UN][16][64] = reinterpret_cast<float (*)[UM * UN][16][64]>(red_lds);  // partial accumulators of the waves with ks > 0
 
   // the wave index (and everything derived from it) is made scalar so that fragment addresses are scalar base +
   // per-lane offset and cost no vector instructions in the loop
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 31, h = lane >> 5;
-  int       mi = 0;
-  for (int i = 1; i < grp.count; ++i) {
-    mi = blockIdx.x >= grp.m[i].wg_begin ? i : mi;
-  }
-  const FragMember &mem     = grp.m[mi];
   const int         KSPLIT  = KSPLIT_T ? KSPLIT_T : mem.ksplit;
   const int         TILES   = kGiWaves / KSPLIT;
   const int         ks = wave % KSPLIT, tw = wave / KSPLIT;
@@ -410,6 +419,170 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
   }
 }
 
+template <int KSPLIT_T, int UM, int UN>
+__global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembers grp, int m, int m_tiles) {
+  __shared__ float red[RedSlots<KSPLIT_T, UM, UN>::kValue * UM * UN * 16 * 64];
+  fragments_workgroup<KSPLIT_T, UM, UN>(member_of_workgroup(grp), m, m_tiles, red);
+}
+
+// ---- 32 x 32 tiles with the activation fragments shared through LDS ----------------------------------------------
+// With 32 x 32 tiles a wave fetches 2.3 KB of operands per block through the vector-memory path and holds four
+// blocks of them in registers: too few bytes in flight to cover the latency of L2 (a wave spends ~950 clocks per
+// block on the Qwen2 shapes at 128 rows). Where the four waves of a workgroup take four neighbouring column tiles of
+// ONE row tile (members whose K is not split), they read the same activation fragments: those now arrive once per
+// workgroup, by DMA into a ring of LDS stages of four blocks, and the registers they leave free hold eight blocks
+// of weight fragments in flight instead of four. Members whose K is split over the waves (long K) keep the plain
+// body above, in the same launch.
+constexpr int kShBlocks = 4;                              // blocks per stage
+constexpr int kShStages = 3;
+constexpr int kShStage  = kShBlocks * (1024 + 256);       // fragments, then the scale rows
+constexpr int kShLds    = kShStages * kShStage > RedSlots<0, 1, 1>::kValue * 16 * 64 * 4 ?
+                              kShStages * kShStage : RedSlots<0, 1, 1>::kValue * 16 * 64 * 4;
+
+__device__ __forceinline__ bool shares_activations(const FragMember &mem) {
+  return mem.ksplit == 1 && mem.nblk % kShBlocks == 0 && mem.nblk >= 2 * kShBlocks;
+}
+
+__global__ __launch_bounds__(kGiThreads, 4) void gemm_i8_fragments_small_kernel(FragMembers grp, int m, int m_tiles) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[kShLds];
+  const FragMember &mem = member_of_workgroup(grp);
+  if (!shares_activations(mem)) {
+    fragments_workgroup<0, 1, 1>(mem, m, m_tiles, reinterpret_cast<float *>(lds));
+    return;
+  }
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c = lane & 31, h = lane >> 5;
+  const int n = mem.n, nblk = mem.nblk, n_tiles = mem.n_tiles;
+  const unsigned wg = blockIdx.x - mem.wg_begin;
+  const int gy = m_tiles, gx = (n_tiles + kGiWaves - 1) / kGiWaves;  // (as in the plain body with one tile per wave)
+  const int xcd = wg & 7, slot = wg >> 3;
+  const int by = slot % gy, bx = (slot / gy) * 8 + xcd;
+  if (bx >= gx) {
+    return;  // whole workgroup
+  }
+  const int  mt = by, nt = bx * kGiWaves + wave;
+  const bool tile_ok = nt < n_tiles;
+  const int  stages = nblk / kShBlocks;
+
+  // -- activation side: stage s = blocks 4 s .. 4 s + 3 of row tile mt, 4 KiB of fragments and 1 KiB of scale rows, both
+  // contiguous in memory; wave w moves fragment KiB w, wave 0 the scale rows as well --
+  const uint32_t ring0 = (uint32_t) (uintptr_t) lds;
+  const uint8_t *a_src  = reinterpret_cast<const uint8_t *>(mem.a_frag) + ((size_t) mt * nblk) * 1024 + wave * 1024;
+  const uint8_t *sa_src = reinterpret_cast<const uint8_t *>(mem.a_scale) + ((size_t) mt * nblk) * 256;
+  const uint32_t lane16 = lane * 16;
+  auto dma16 = [&](const uint8_t *base, uint32_t dst) {
+    asm volatile("s_mov_b32 m0, %2\n s_nop 0\n global_load_lds_dwordx4 %0, %1" ::"v"(lane16), "s"(base), "s"(dst) : "memory");
+  };
+  auto issue_stage = [&](int s) {  // (stages past the end re-read the last one; nobody reads them)
+    const int      sc = min(s, stages - 1);
+    const uint32_t so = ring0 + (uint32_t) (s % kShStages) * kShStage;
+    dma16(a_src + (size_t) sc * (kShBlocks * 1024), so + wave * 1024);
+    if (wave == 0) {
+      dma16(sa_src + (size_t) sc * (kShBlocks * 256), so + kShBlocks * 1024);
+    }
+  };
+  const int mine = wave == 0 ? 2 : 1;  // transfers of this wave per stage
+
+  // -- weight side: eight blocks in registers (two stages), block q of stage s in slot (s % 2) * 4 + q --
+  auto resource = [](const void *base) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int) 0xffffffffu, 0x00020000);
+  };
+  const size_t           ntc = (size_t) min(nt, n_tiles - 1);
+  __amdgpu_buffer_rsrc_t rb  = resource(mem.b_frag + ntc * nblk * 64);
+  __amdgpu_buffer_rsrc_t rsb = resource(mem.b_scale + ntc * nblk * 32);
+  const int c4 = c * 4;
+  uint4    bq[2 * kShBlocks];
+  uint32_t dwq[2 * kShBlocks];
+  auto load_b = [&](int slot_, int kb_raw) {
+    const int kb = min(kb_raw, nblk - 1);  // (blocks past the end repeat the last one; they are never used)
+    bq[slot_]  = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int) lane16, kb * 1024, 0));
+    dwq[slot_] = __builtin_amdgcn_raw_buffer_load_b32(rsb, c4, kb * 128, 0);
+  };
+
+  // prologue: order of vector-memory operations = DMA(0), B(0), DMA(1), B(1); from then on DMA(s + 2) at the start of
+  // stage s and B(s + 2) block by block during it
+  issue_stage(0);
+#pragma unroll
+  for (int q = 0; q < kShBlocks; ++q) {
+    load_b(q, q);
+  }
+  issue_stage(1);
+#pragma unroll
+  for (int q = 0; q < kShBlocks; ++q) {
+    load_b(kShBlocks + q, kShBlocks + q);
+  }
+
+  v16f acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    acc[r] = 0.0f;
+  }
+  const v16f zf = { 0 };
+  const v16i zi = { 0 };
+  typedef __attribute__((address_space(3))) const uint8_t *lds_ptr;
+  const uint32_t a_rd = ring0 + lane16, sa_rd = ring0 + kShBlocks * 1024 + lane * 4;
+
+  auto stage = [&](auto parity_tag, int s) {
+    constexpr int P = decltype(parity_tag)::value;  // s % 2: which half of the weight registers
+    // This wave's transfers of stage s have landed: everything it issued after them -- the weight loads of stage
+    // s + 1, the transfers of stage s + 1 and the weight loads of ... -- may stay in flight. Counted from the order
+    // above: B(s) [4 x 2], DMA(s + 1) [mine], B(s + 1) [4 x 2] follow DMA(s).
+    if (mine == 2) {
+      __builtin_amdgcn_s_waitcnt(0x0F70 | ((8 + 2 + 8) & 15) | (((8 + 2 + 8) >> 4) << 14));
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70 | ((8 + 1 + 8) & 15) | (((8 + 1 + 8) >> 4) << 14));
+    }
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    const uint32_t so = (uint32_t) (s % kShStages) * kShStage;
+    v4i      af[kShBlocks];
+    uint32_t da[kShBlocks];
+#pragma unroll
+    for (int q = 0; q < kShBlocks; ++q) {
+      af[q] = *reinterpret_cast<__attribute__((address_space(3))) const v4i *>((lds_ptr) (uintptr_t) (a_rd + so) + q * 1024);
+      da[q] = *reinterpret_cast<__attribute__((address_space(3))) const uint32_t *>((lds_ptr) (uintptr_t) (sa_rd + so) + q * 256);
+    }
+    // everybody has left stage s - 1: its LDS stage takes stage s + 2
+    issue_stage(s + 2);
+    // One unit at a time (the empty asm statements pin that order, so that one unit's results are in registers at a
+    // time): with four waves per SIMD it is the other waves that fill the pipes meanwhile.
+#pragma unroll
+    for (int q = 0; q < kShBlocks; ++q) {
+      const v4i a4 = af[q];
+      const v4i b4 = { (int) bq[P * kShBlocks + q].x, (int) bq[P * kShBlocks + q].y, (int) bq[P * kShBlocks + q].z,
+                       (int) bq[P * kShBlocks + q].w };
+      v16i        sum = __builtin_amdgcn_mfma_i32_32x32x32_i8(a4, b4, zi, 0, 0, 0);
+      const uint2 ua = make_uint2(da[q], 0u), ub = make_uint2(dwq[P * kShBlocks + q], 0u);
+      v16f        scl = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(v4h, ua), __builtin_bit_cast(v4h, ub), zf, 0, 0, 0);
+      asm volatile("" : "+v"(sum), "+v"(scl));
+      // both instructions of block q have read its slot: the slot takes its block of stage s + 2
+      load_b(P * kShBlocks + q, (s + 2) * kShBlocks + q);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc[r] = __builtin_fmaf((float) sum[r], scl[r], acc[r]);
+      }
+      asm volatile("" : "+v"(acc));
+    }
+  };
+  for (int s = 0; s < stages; s += 2) {
+    stage(std::integral_constant<int, 0>(), s);
+    if (s + 1 < stages) {
+      stage(std::integral_constant<int, 1>(), s + 1);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // (transfers of stages past the end must have landed before LDS is released)
+  if (tile_ok) {
+    const int col = nt * 32 + c;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int row = mt * 32 + 8 * (r >> 2) + 4 * h + (r & 3);
+      if (row < m && col < n) {
+        mem.out[(size_t) row * n + col] = acc[r];
+      }
+    }
+  }
+}
+
 size_t round256(size_t x) {
   return (x + 255) & ~(size_t) 255;
 }
@@ -572,7 +745,7 @@ hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *
   }
   grp.count = count;
   if (cfg.unit == 1) {
-    hipLaunchKernelGGL((gemm_i8_fragments_kernel<0, 1, kSmallUN>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
+    hipLaunchKernelGGL(gemm_i8_fragments_small_kernel, dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
   } else if (cfg.ksplit == 4) {
     hipLaunchKernelGGL((gemm_i8_fragments_kernel<4, 2, 2>), dim3(total), dim3(kGiThreads), 0, stream, grp, m, m_tiles);
   } else {
