@@ -219,6 +219,7 @@ struct FragMember {
   float          *out;
   int             n, nblk, n_tiles;
   int             ksplit;  // waves that share a tile's K (used by the instantiation that takes it at run time)
+  int             share;   // small tiles: which operand the workgroup shares through LDS (kShare*)
   unsigned        wg_begin;
 };
 struct FragMembers {
@@ -425,50 +426,53 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
   fragments_workgroup<KSPLIT_T, UM, UN>(member_of_workgroup(grp), m, m_tiles, red);
 }
 
-// ---- 32 x 32 tiles with the activation fragments shared through LDS ----------------------------------------------
+// ---- 32 x 32 tiles with one operand shared through LDS ------------------------------------------------------------
 // With 32 x 32 tiles a wave fetches 2.3 KB of operands per block through the vector-memory path and holds four
-// blocks of them in registers: too few bytes in flight to cover the latency of L2 (a wave spends ~950 clocks per
-// block on the Qwen2 shapes at 128 rows). Where the four waves of a workgroup take four neighbouring column tiles of
-// ONE row tile (members whose K is not split), they read the same activation fragments: those now arrive once per
-// workgroup, by DMA into a ring of LDS stages of four blocks, and the registers they leave free hold eight blocks
-// of weight fragments in flight instead of four. Members whose K is split over the waves (long K) keep the plain
-// body above, in the same launch.
+// blocks of them in registers: too few bytes in flight to cover the latency (a wave spends ~950 clocks per block on
+// the Qwen2 shapes at 128 rows). For members whose K is not split over the waves, the four waves of a workgroup
+// therefore share one operand: it arrives once per workgroup, by DMA into a ring of LDS stages of four blocks, and the
+// registers it leaves free hold eight blocks of the other operand in flight instead of four.
+//   kShareWeights      the waves are the four row tiles of ONE column tile (row counts that are whole groups of four
+//                      row tiles, e.g. 128): the weight fragments -- the stream that comes from HBM -- go through LDS,
+//                      once per column tile and launch
+//   kShareActivations  the waves are four neighbouring column tiles of ONE row tile: the activation fragments go
+//                      through LDS
+// Members whose K is split over the waves (long K) keep the plain body above, in the same launch.
 constexpr int kShBlocks = 4;                              // blocks per stage
 constexpr int kShStages = 3;
-constexpr int kShStage  = kShBlocks * (1024 + 256);       // fragments, then the scale rows
+constexpr int kShStage  = kShBlocks * (1024 + 256);       // fragments, then the scale rows (256 or 128 bytes a block)
 constexpr int kShLds    = kShStages * kShStage > RedSlots<0, 1, 1>::kValue * 16 * 64 * 4 ?
                               kShStages * kShStage : RedSlots<0, 1, 1>::kValue * 16 * 64 * 4;
+enum { kSharePlain = 0, kShareActivations = 1, kShareWeights = 2 };
 
-__device__ __forceinline__ bool shares_activations(const FragMember &mem) {
-  return mem.ksplit == 1 && mem.nblk % kShBlocks == 0 && mem.nblk >= 2 * kShBlocks;
-}
-
-__global__ __launch_bounds__(kGiThreads, 4) void gemm_i8_fragments_small_kernel(FragMembers grp, int m, int m_tiles) {
-  __shared__ __attribute__((aligned(1024))) uint8_t lds[kShLds];
-  const FragMember &mem = member_of_workgroup(grp);
-  if (!shares_activations(mem)) {
-    fragments_workgroup<0, 1, 1>(mem, m, m_tiles, reinterpret_cast<float *>(lds));
-    return;
-  }
+template <bool SHARE_W>
+__device__ __forceinline__ void shared_operand_workgroup(const FragMember &mem, int m, int m_tiles, uint8_t *lds) {
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 31, h = lane >> 5;
   const int n = mem.n, nblk = mem.nblk, n_tiles = mem.n_tiles;
   const unsigned wg = blockIdx.x - mem.wg_begin;
-  const int gy = m_tiles, gx = (n_tiles + kGiWaves - 1) / kGiWaves;  // (as in the plain body with one tile per wave)
+  // grid of the member: gy groups along m, gx along n (padded to 8 for the XCDs), as member_workgroups lays it out
+  const int gy = SHARE_W ? m_tiles / kGiWaves : m_tiles;
+  const int gx = SHARE_W ? n_tiles : (n_tiles + kGiWaves - 1) / kGiWaves;
   const int xcd = wg & 7, slot = wg >> 3;
   const int by = slot % gy, bx = (slot / gy) * 8 + xcd;
   if (bx >= gx) {
     return;  // whole workgroup
   }
-  const int  mt = by, nt = bx * kGiWaves + wave;
-  const bool tile_ok = nt < n_tiles;
+  const int  mt = SHARE_W ? by * kGiWaves + wave : by;
+  const int  nt = SHARE_W ? bx : bx * kGiWaves + wave;
+  const bool tile_ok = nt < n_tiles;  // (mt < m_tiles by construction)
   const int  stages = nblk / kShBlocks;
+  const size_t ntc = (size_t) min(nt, n_tiles - 1);
 
-  // -- activation side: stage s = blocks 4 s .. 4 s + 3 of row tile mt, 4 KiB of fragments and 1 KiB of scale rows, both
+  // -- the shared operand: stage s = blocks 4 s .. 4 s + 3 of its tile, 4 KiB of fragments and the scale rows, both
   // contiguous in memory; wave w moves fragment KiB w, wave 0 the scale rows as well --
+  constexpr int  kScaleRow = SHARE_W ? 128 : 256;  // bytes of scales per block
   const uint32_t ring0 = (uint32_t) (uintptr_t) lds;
-  const uint8_t *a_src  = reinterpret_cast<const uint8_t *>(mem.a_frag) + ((size_t) mt * nblk) * 1024 + wave * 1024;
-  const uint8_t *sa_src = reinterpret_cast<const uint8_t *>(mem.a_scale) + ((size_t) mt * nblk) * 256;
+  const uint8_t *sh_src = SHARE_W ? reinterpret_cast<const uint8_t *>(mem.b_frag) + (ntc * nblk) * 1024 + wave * 1024 :
+                                    reinterpret_cast<const uint8_t *>(mem.a_frag) + ((size_t) mt * nblk) * 1024 + wave * 1024;
+  const uint8_t *sc_src = SHARE_W ? reinterpret_cast<const uint8_t *>(mem.b_scale) + (ntc * nblk) * 128 :
+                                    reinterpret_cast<const uint8_t *>(mem.a_scale) + ((size_t) mt * nblk) * 256;
   const uint32_t lane16 = lane * 16;
   auto dma16 = [&](const uint8_t *base, uint32_t dst) {
     asm volatile("s_mov_b32 m0, %2\n s_nop 0\n global_load_lds_dwordx4 %0, %1" ::"v"(lane16), "s"(base), "s"(dst) : "memory");
@@ -476,40 +480,41 @@ __global__ __launch_bounds__(kGiThreads, 4) void gemm_i8_fragments_small_kernel(
   auto issue_stage = [&](int s) {  // (stages past the end re-read the last one; nobody reads them)
     const int      sc = min(s, stages - 1);
     const uint32_t so = ring0 + (uint32_t) (s % kShStages) * kShStage;
-    dma16(a_src + (size_t) sc * (kShBlocks * 1024), so + wave * 1024);
+    dma16(sh_src + (size_t) sc * (kShBlocks * 1024), so + wave * 1024);
     if (wave == 0) {
-      dma16(sa_src + (size_t) sc * (kShBlocks * 256), so + kShBlocks * 1024);
+      if (!SHARE_W || lane < 32) {  // 4 x 128 bytes of weight scales are half a transfer
+        dma16(sc_src + (size_t) sc * (kShBlocks * kScaleRow), so + kShBlocks * 1024);
+      }
     }
   };
   const int mine = wave == 0 ? 2 : 1;  // transfers of this wave per stage
 
-  // -- weight side: eight blocks in registers (two stages), block q of stage s in slot (s % 2) * 4 + q --
+  // -- the wave's own operand: eight blocks in registers (two stages), block q of stage s in slot (s % 2) * 4 + q --
   auto resource = [](const void *base) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int) 0xffffffffu, 0x00020000);
   };
-  const size_t           ntc = (size_t) min(nt, n_tiles - 1);
-  __amdgpu_buffer_rsrc_t rb  = resource(mem.b_frag + ntc * nblk * 64);
-  __amdgpu_buffer_rsrc_t rsb = resource(mem.b_scale + ntc * nblk * 32);
-  const int c4 = c * 4;
-  uint4    bq[2 * kShBlocks];
-  uint32_t dwq[2 * kShBlocks];
-  auto load_b = [&](int slot_, int kb_raw) {
+  __amdgpu_buffer_rsrc_t ro  = SHARE_W ? resource(mem.a_frag + (size_t) mt * nblk * 64) : resource(mem.b_frag + ntc * nblk * 64);
+  __amdgpu_buffer_rsrc_t rso = SHARE_W ? resource(mem.a_scale + (size_t) mt * nblk * 64) : resource(mem.b_scale + ntc * nblk * 32);
+  const int own_scale_off = SHARE_W ? lane * 4 : c * 4;
+  uint4     oq[2 * kShBlocks];
+  uint32_t  dq[2 * kShBlocks];
+  auto load_own = [&](int slot_, int kb_raw) {
     const int kb = min(kb_raw, nblk - 1);  // (blocks past the end repeat the last one; they are never used)
-    bq[slot_]  = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rb, (int) lane16, kb * 1024, 0));
-    dwq[slot_] = __builtin_amdgcn_raw_buffer_load_b32(rsb, c4, kb * 128, 0);
+    oq[slot_] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ro, (int) lane16, kb * 1024, 0));
+    dq[slot_] = __builtin_amdgcn_raw_buffer_load_b32(rso, own_scale_off, kb * (SHARE_W ? 256 : 128), 0);
   };
 
-  // prologue: order of vector-memory operations = DMA(0), B(0), DMA(1), B(1); from then on DMA(s + 2) at the start of
-  // stage s and B(s + 2) block by block during it
+  // prologue: order of vector-memory operations = DMA(0), own(0), DMA(1), own(1); from then on DMA(s + 2) at the start
+  // of stage s and own(s + 2) block by block during it
   issue_stage(0);
 #pragma unroll
   for (int q = 0; q < kShBlocks; ++q) {
-    load_b(q, q);
+    load_own(q, q);
   }
   issue_stage(1);
 #pragma unroll
   for (int q = 0; q < kShBlocks; ++q) {
-    load_b(kShBlocks + q, kShBlocks + q);
+    load_own(kShBlocks + q, kShBlocks + q);
   }
 
   v16f acc;
@@ -520,13 +525,12 @@ __global__ __launch_bounds__(kGiThreads, 4) void gemm_i8_fragments_small_kernel(
   const v16f zf = { 0 };
   const v16i zi = { 0 };
   typedef __attribute__((address_space(3))) const uint8_t *lds_ptr;
-  const uint32_t a_rd = ring0 + lane16, sa_rd = ring0 + kShBlocks * 1024 + lane * 4;
+  const uint32_t sh_rd = ring0 + lane16, sc_rd = ring0 + kShBlocks * 1024 + (SHARE_W ? c * 4 : lane * 4);
 
   auto stage = [&](auto parity_tag, int s) {
-    constexpr int P = decltype(parity_tag)::value;  // s % 2: which half of the weight registers
-    // This wave's transfers of stage s have landed: everything it issued after them -- the weight loads of stage
-    // s + 1, the transfers of stage s + 1 and the weight loads of ... -- may stay in flight. Counted from the order
-    // above: B(s) [4 x 2], DMA(s + 1) [mine], B(s + 1) [4 x 2] follow DMA(s).
+    constexpr int P = decltype(parity_tag)::value;  // s % 2: which half of the own registers
+    // This wave's transfers of stage s have landed; what it issued after them -- own(s) [4 x 2 loads], DMA(s + 1)
+    // [mine], own(s + 1) [4 x 2] -- may stay in flight.
     if (mine == 2) {
       __builtin_amdgcn_s_waitcnt(0x0F70 | ((8 + 2 + 8) & 15) | (((8 + 2 + 8) >> 4) << 14));
     } else {
@@ -535,12 +539,12 @@ __global__ __launch_bounds__(kGiThreads, 4) void gemm_i8_fragments_small_kernel(
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     const uint32_t so = (uint32_t) (s % kShStages) * kShStage;
-    v4i      af[kShBlocks];
-    uint32_t da[kShBlocks];
+    v4i      sf[kShBlocks];
+    uint32_t sd[kShBlocks];
 #pragma unroll
     for (int q = 0; q < kShBlocks; ++q) {
-      af[q] = *reinterpret_cast<__attribute__((address_space(3))) const v4i *>((lds_ptr) (uintptr_t) (a_rd + so) + q * 1024);
-      da[q] = *reinterpret_cast<__attribute__((address_space(3))) const uint32_t *>((lds_ptr) (uintptr_t) (sa_rd + so) + q * 256);
+      sf[q] = *reinterpret_cast<__attribute__((address_space(3))) const v4i *>((lds_ptr) (uintptr_t) (sh_rd + so) + q * 1024);
+      sd[q] = *reinterpret_cast<__attribute__((address_space(3))) const uint32_t *>((lds_ptr) (uintptr_t) (sc_rd + so) + q * kScaleRow);
     }
     // everybody has left stage s - 1: its LDS stage takes stage s + 2
     issue_stage(s + 2);
@@ -548,15 +552,21 @@ __global__ __launch_bounds__(kGiThreads, 4) void gemm_i8_fragments_small_kernel(
     // time): with four waves per SIMD it is the other waves that fill the pipes meanwhile.
 #pragma unroll
     for (int q = 0; q < kShBlocks; ++q) {
-      const v4i a4 = af[q];
-      const v4i b4 = { (int) bq[P * kShBlocks + q].x, (int) bq[P * kShBlocks + q].y, (int) bq[P * kShBlocks + q].z,
-                       (int) bq[P * kShBlocks + q].w };
-      v16i        sum = __builtin_amdgcn_mfma_i32_32x32x32_i8(a4, b4, zi, 0, 0, 0);
-      const uint2 ua = make_uint2(da[q], 0u), ub = make_uint2(dwq[P * kShBlocks + q], 0u);
-      v16f        scl = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(v4h, ua), __builtin_bit_cast(v4h, ub), zf, 0, 0, 0);
+      const v4i o4 = { (int) oq[P * kShBlocks + q].x, (int) oq[P * kShBlocks + q].y, (int) oq[P * kShBlocks + q].z,
+                       (int) oq[P * kShBlocks + q].w };
+      const uint2 uo = make_uint2(dq[P * kShBlocks + q], 0u), us = make_uint2(sd[q], 0u);
+      v16i        sum;
+      v16f        scl;
+      if (SHARE_W) {  // A operand: activations (own), B operand: weights (shared)
+        sum = __builtin_amdgcn_mfma_i32_32x32x32_i8(o4, sf[q], zi, 0, 0, 0);
+        scl = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(v4h, uo), __builtin_bit_cast(v4h, us), zf, 0, 0, 0);
+      } else {
+        sum = __builtin_amdgcn_mfma_i32_32x32x32_i8(sf[q], o4, zi, 0, 0, 0);
+        scl = __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(v4h, us), __builtin_bit_cast(v4h, uo), zf, 0, 0, 0);
+      }
       asm volatile("" : "+v"(sum), "+v"(scl));
       // both instructions of block q have read its slot: the slot takes its block of stage s + 2
-      load_b(P * kShBlocks + q, (s + 2) * kShBlocks + q);
+      load_own(P * kShBlocks + q, (s + 2) * kShBlocks + q);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         acc[r] = __builtin_fmaf((float) sum[r], scl[r], acc[r]);
@@ -580,6 +590,18 @@ __global__ __launch_bounds__(kGiThreads, 4) void gemm_i8_fragments_small_kernel(
         mem.out[(size_t) row * n + col] = acc[r];
       }
     }
+  }
+}
+
+__global__ __launch_bounds__(kGiThreads, 4) void gemm_i8_fragments_small_kernel(FragMembers grp, int m, int m_tiles) {
+  __shared__ __attribute__((aligned(1024))) uint8_t lds[kShLds];
+  const FragMember &mem = member_of_workgroup(grp);
+  if (mem.share == kShareWeights) {
+    shared_operand_workgroup<true>(mem, m, m_tiles, lds);
+  } else if (mem.share == kShareActivations) {
+    shared_operand_workgroup<false>(mem, m, m_tiles, lds);
+  } else {
+    fragments_workgroup<0, 1, 1>(mem, m, m_tiles, reinterpret_cast<float *>(lds));
   }
 }
 
@@ -647,7 +669,19 @@ TileConfig tile_config(int m, int n, int k) {
 // the Qwen2-like block at m = 128: these launches want waves more than they want bytes saved.
 constexpr int kSmallUN = 1;
 
-unsigned member_workgroups(int m_tiles, int n_tiles, TileConfig cfg) {
+// small tiles: which operand the four waves of a workgroup share (see shared_operand_workgroup)
+int small_tile_share(int m_tiles, int nblk, TileConfig cfg) {
+  if (cfg.unit != 1 || cfg.ksplit != 1 || nblk % kShBlocks != 0 || nblk < 2 * kShBlocks) {
+    return kSharePlain;
+  }
+  // (measured on the Qwen2 block at 128 rows: weights shared 39.6 us, activations shared 40.2 us, neither 43.9 us)
+  return m_tiles % kGiWaves == 0 ? kShareWeights : kShareActivations;
+}
+
+unsigned member_workgroups(int m_tiles, int n_tiles, int nblk, TileConfig cfg) {
+  if (small_tile_share(m_tiles, nblk, cfg) == kShareWeights) {
+    return (unsigned) ((n_tiles + 7) / 8 * 8 * (m_tiles / kGiWaves));
+  }
   const unsigned tiles_per_wg = kGiWaves / cfg.ksplit;
   const unsigned un = cfg.unit == 1 ? kSmallUN : cfg.unit;
   const unsigned gy = (unsigned) ((m_tiles + cfg.unit - 1) / cfg.unit);
@@ -741,7 +775,8 @@ hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *
     grp.m[slot].n_tiles  = n_tiles;
     grp.m[slot].ksplit   = c.ksplit;
     grp.m[slot].wg_begin = total;
-    total += member_workgroups(m_tiles, n_tiles, cfg);
+    grp.m[slot].share    = small_tile_share(m_tiles, nblk, c);
+    total += member_workgroups(m_tiles, n_tiles, nblk, cfg);
   }
   grp.count = count;
   if (cfg.unit == 1) {
