@@ -220,6 +220,9 @@ struct FragMember {
   int             n, nblk, n_tiles;
   int             ksplit;  // waves that share a tile's K (used by the instantiation that takes it at run time)
   int             share;   // small tiles: which operand the workgroup shares through LDS (kShare*)
+  int             kparts;  // kShareWeights: workgroups that share a tile's K (partial tiles meet in `exchange`)
+  float          *exchange;
+  unsigned       *tickets;  // one zeroed counter per (tile, wave) of this member, left zeroed
   unsigned        wg_begin;
 };
 struct FragMembers {
@@ -437,7 +440,10 @@ __global__ __launch_bounds__(kGiThreads) void gemm_i8_fragments_kernel(FragMembe
 //                      once per column tile and launch
 //   kShareActivations  the waves are four neighbouring column tiles of ONE row tile: the activation fragments go
 //                      through LDS
-// Members whose K is split over the waves (long K) keep the plain body above, in the same launch.
+// Long K (which the plain body splits over the four waves of a workgroup) is split over `kparts` WORKGROUPS in the
+// kShareWeights arrangement: every wave leaves its partial tile in `exchange` (device-scope stores) and takes a
+// ticket; the wave that comes last adds all parts in part order and stores the tile, so the result does not depend
+// on who that was and nobody waits for anybody. Other members with split K keep the plain body, in the same launch.
 constexpr int kShBlocks = 4;                              // blocks per stage
 constexpr int kShStages = 3;
 constexpr int kShStage  = kShBlocks * (1024 + 256);       // fragments, then the scale rows (256 or 128 bytes a block)
@@ -454,7 +460,8 @@ __device__ __forceinline__ void shared_operand_workgroup(const FragMember &mem, 
   // grid of the member: gy groups along m, gx along n (padded to 8 for the XCDs), as member_workgroups lays it out
   const int gy = SHARE_W ? m_tiles / kGiWaves : m_tiles;
   const int gx = SHARE_W ? n_tiles : (n_tiles + kGiWaves - 1) / kGiWaves;
-  const int xcd = wg & 7, slot = wg >> 3;
+  const int kparts = SHARE_W ? mem.kparts : 1;
+  const int xcd = wg & 7, slot = (int) (wg >> 3) / kparts, kpart = (int) (wg >> 3) % kparts;
   const int by = slot % gy, bx = (slot / gy) * 8 + xcd;
   if (bx >= gx) {
     return;  // whole workgroup
@@ -462,7 +469,10 @@ __device__ __forceinline__ void shared_operand_workgroup(const FragMember &mem, 
   const int  mt = SHARE_W ? by * kGiWaves + wave : by;
   const int  nt = SHARE_W ? bx : bx * kGiWaves + wave;
   const bool tile_ok = nt < n_tiles;  // (mt < m_tiles by construction)
-  const int  stages = nblk / kShBlocks;
+  // stages of this workgroup's part of K: [stage0, stage0 + stages)
+  const int  all_stages = nblk / kShBlocks;
+  const int  stage0 = (int) ((long) kpart * all_stages / kparts);
+  const int  stages = (int) ((long) (kpart + 1) * all_stages / kparts) - stage0;
   const size_t ntc = (size_t) min(nt, n_tiles - 1);
 
   // -- the shared operand: stage s = blocks 4 s .. 4 s + 3 of its tile, 4 KiB of fragments and the scale rows, both
@@ -478,7 +488,7 @@ __device__ __forceinline__ void shared_operand_workgroup(const FragMember &mem, 
     asm volatile("s_mov_b32 m0, %2\n s_nop 0\n global_load_lds_dwordx4 %0, %1" ::"v"(lane16), "s"(base), "s"(dst) : "memory");
   };
   auto issue_stage = [&](int s) {  // (stages past the end re-read the last one; nobody reads them)
-    const int      sc = min(s, stages - 1);
+    const int      sc = stage0 + min(s, stages - 1);
     const uint32_t so = ring0 + (uint32_t) (s % kShStages) * kShStage;
     dma16(sh_src + (size_t) sc * (kShBlocks * 1024), so + wave * 1024);
     if (wave == 0) {
@@ -499,7 +509,7 @@ __device__ __forceinline__ void shared_operand_workgroup(const FragMember &mem, 
   uint4     oq[2 * kShBlocks];
   uint32_t  dq[2 * kShBlocks];
   auto load_own = [&](int slot_, int kb_raw) {
-    const int kb = min(kb_raw, nblk - 1);  // (blocks past the end repeat the last one; they are never used)
+    const int kb = min(stage0 * kShBlocks + kb_raw, nblk - 1);  // (blocks past the end repeat the last one; they are never used)
     oq[slot_] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(ro, (int) lane16, kb * 1024, 0));
     dq[slot_] = __builtin_amdgcn_raw_buffer_load_b32(rso, own_scale_off, kb * (SHARE_W ? 256 : 128), 0);
   };
@@ -581,6 +591,36 @@ __device__ __forceinline__ void shared_operand_workgroup(const FragMember &mem, 
     }
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);  // (transfers of stages past the end must have landed before LDS is released)
+  if (SHARE_W && kparts > 1) {
+    const size_t tile_slot = ((size_t) bx * gy + by) * kGiWaves + wave;  // (column tile, row group, wave)
+    float       *parts     = mem.exchange + tile_slot * kparts * 1024;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      __hip_atomic_store(&parts[kpart * 1024 + r * 64 + lane], acc[r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the stores are acknowledged before the ticket is taken
+    unsigned ticket = 0;
+    if (lane == 0) {
+      ticket = __hip_atomic_fetch_add(&mem.tickets[tile_slot], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    ticket = __builtin_amdgcn_readfirstlane(ticket);
+    if (ticket != (unsigned) (kparts - 1)) {
+      return;  // the wave that comes last finishes the tile
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      acc[r] = 0.0f;
+    }
+    for (int p = 0; p < kparts; ++p) {  // all parts, this wave's own included, in part order
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        acc[r] += __hip_atomic_load(&parts[p * 1024 + r * 64 + lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    if (lane == 0) {
+      __hip_atomic_store(&mem.tickets[tile_slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    }
+  }
   if (tile_ok) {
     const int col = nt * 32 + c;
 #pragma unroll
@@ -669,18 +709,28 @@ TileConfig tile_config(int m, int n, int k) {
 // the Qwen2-like block at m = 128: these launches want waves more than they want bytes saved.
 constexpr int kSmallUN = 1;
 
-// small tiles: which operand the four waves of a workgroup share (see shared_operand_workgroup)
-int small_tile_share(int m_tiles, int nblk, TileConfig cfg) {
-  if (cfg.unit != 1 || cfg.ksplit != 1 || nblk % kShBlocks != 0 || nblk < 2 * kShBlocks) {
-    return kSharePlain;
+// small tiles: which operand the four waves of a workgroup share (see shared_operand_workgroup) and, with the weights
+// shared, over how many workgroups K is split (`split_k`: the caller has scratch for the partial tiles)
+struct SmallTilePlan {
+  int share, kparts;
+};
+SmallTilePlan small_tile_plan(int m_tiles, int nblk, TileConfig cfg, bool split_k) {
+  if (cfg.unit != 1 || nblk % kShBlocks != 0 || nblk < 2 * kShBlocks) {
+    return { kSharePlain, 1 };
+  }
+  const bool row_groups = m_tiles % kGiWaves == 0;
+  if (cfg.ksplit != 1) {
+    // a wave should walk some 48 blocks (as the plain body's split of K aims at)
+    // (measured on the Qwen2 block at 128 rows, k = 8960: 24 / 32 / 40 / 48 / 64 blocks per part 38.7 / 38.6 / 35.3 / 35.8 / 37.0 us)
+    return row_groups && split_k ? SmallTilePlan{ kShareWeights, std::min(8, nblk / 48) } : SmallTilePlan{ kSharePlain, 1 };
   }
   // (measured on the Qwen2 block at 128 rows: weights shared 39.6 us, activations shared 40.2 us, neither 43.9 us)
-  return m_tiles % kGiWaves == 0 ? kShareWeights : kShareActivations;
+  return { row_groups ? kShareWeights : kShareActivations, 1 };
 }
 
-unsigned member_workgroups(int m_tiles, int n_tiles, int nblk, TileConfig cfg) {
-  if (small_tile_share(m_tiles, nblk, cfg) == kShareWeights) {
-    return (unsigned) ((n_tiles + 7) / 8 * 8 * (m_tiles / kGiWaves));
+unsigned member_workgroups(int m_tiles, int n_tiles, TileConfig cfg, SmallTilePlan plan) {
+  if (plan.share == kShareWeights) {
+    return (unsigned) ((n_tiles + 7) / 8 * 8 * (m_tiles / kGiWaves) * plan.kparts);
   }
   const unsigned tiles_per_wg = kGiWaves / cfg.ksplit;
   const unsigned un = cfg.unit == 1 ? kSmallUN : cfg.unit;
@@ -736,12 +786,21 @@ hipError_t launch_act_to_i8_fragments_group(hipStream_t stream, int count, void 
   return hipGetLastError();
 }
 
+size_t gemm_i8_fragments_exchange_bytes(int m, int n, int k) {
+  const int           m_tiles = (m + 31) / 32, n_tiles = (n + 31) / 32, nblk = k / 32;
+  const SmallTilePlan plan    = small_tile_plan(m_tiles, nblk, tile_config(m, n, k), true);
+  return plan.kparts > 1 ? (size_t) ((n_tiles + 7) / 8 * 8) * m_tiles * plan.kparts * 1024 * sizeof(float) : 0;
+}
+
 hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *const *outs,
                                           const void *const *act_fragments, const void *const *weight_fragments,
-                                          const int *ns, const int *ks, int m) {
+                                          const int *ns, const int *ks, int m, void *exchange, size_t exchange_bytes,
+                                          unsigned *tickets, int ticket_slots) {
   if (count < 1 || count > kGemmGroupMax || m <= 0) {
     return hipErrorInvalidValue;
   }
+  size_t exchange_used = 0;
+  int    tickets_used  = 0;
   const int   m_tiles = (m + 31) / 32;
   FragMembers grp;
   unsigned    total = 0;
@@ -775,8 +834,22 @@ hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *
     grp.m[slot].n_tiles  = n_tiles;
     grp.m[slot].ksplit   = c.ksplit;
     grp.m[slot].wg_begin = total;
-    grp.m[slot].share    = small_tile_share(m_tiles, nblk, c);
-    total += member_workgroups(m_tiles, n_tiles, nblk, cfg);
+    // K split over workgroups while the caller's scratch for partial tiles and its ticket counters last
+    const size_t  xbytes  = gemm_i8_fragments_exchange_bytes(m, ns[i], ks[i]);
+    const int     xslots  = (n_tiles + 7) / 8 * 8 * m_tiles;
+    const bool    split_k = exchange && tickets && xbytes > 0 && exchange_used + xbytes <= exchange_bytes &&
+                         tickets_used + xslots <= ticket_slots;
+    SmallTilePlan plan    = small_tile_plan(m_tiles, nblk, c, split_k);
+    grp.m[slot].share    = plan.share;
+    grp.m[slot].kparts   = plan.kparts;
+    grp.m[slot].exchange = nullptr;
+    grp.m[slot].tickets  = nullptr;
+    if (plan.kparts > 1) {
+      grp.m[slot].exchange = reinterpret_cast<float *>(static_cast<uint8_t *>(exchange) + exchange_used);
+      grp.m[slot].tickets  = tickets + tickets_used;
+      exchange_used += xbytes, tickets_used += xslots;
+    }
+    total += member_workgroups(m_tiles, n_tiles, cfg, plan);
   }
   grp.count = count;
   if (cfg.unit == 1) {
@@ -790,7 +863,8 @@ hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *
 }
 
 hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_fragments,
-                                    int m, int k, int n, void *act_fragments, bool act_fragments_ready) {
+                                    int m, int k, int n, void *act_fragments, bool act_fragments_ready, void *exchange,
+                                    size_t exchange_bytes, unsigned *tickets, int ticket_slots) {
   if (k % 32 != 0 || m <= 0 || n <= 0) {
     return hipErrorInvalidValue;
   }
@@ -800,7 +874,8 @@ hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *
     }
   }
   const void *af = act_fragments;
-  return launch_gemm_i8_fragments_group(stream, 1, &out, &af, &weight_fragments, &n, &k, m);
+  return launch_gemm_i8_fragments_group(stream, 1, &out, &af, &weight_fragments, &n, &k, m, exchange, exchange_bytes, tickets,
+                                        ticket_slots);
 }
 
 }  // namespace htpops

@@ -521,7 +521,8 @@ MatMulPlan plan_mat_mul(htpops_context *ctx, const void *weight, bool act_aligne
   p.act_bytes    = (htpops::gemm_i8_act_fragment_bytes(m, k) + 255) & ~(size_t) 255;
   p.weight_bytes = (htpops::gemm_i8_weight_fragment_bytes(k, n) + 255) & ~(size_t) 255;
   lookup_copy(kFragKindRowLayout + wt);
-  p.ws_bytes = p.act_bytes + ((p.cached || p.cacheable) ? 0 : p.weight_bytes);
+  p.ws_bytes = p.act_bytes + ((p.cached || p.cacheable) ? 0 : p.weight_bytes) +
+               ((htpops::gemm_i8_fragments_exchange_bytes(m, n, k) + 255) & ~(size_t) 255);
   return p;
 }
 
@@ -601,7 +602,11 @@ int run_mat_mul(htpops_context *ctx, MatMulPlan &plan, float *dst, const void *a
   if (plan.kind == kPlanLdsFp6) {
     HTPOPS_HIP(ctx, htpops::launch_gemm_fp6_lds(ctx->stream, dst, act, frags, m, k, n, ws, ready));
   } else {
-    HTPOPS_HIP(ctx, htpops::launch_gemm_i8_fragments(ctx->stream, dst, act, frags, m, k, n, ws, ready));
+    // (scratch for partial tiles at the end of this matmul's share of the workspace)
+    const size_t xbytes = htpops::gemm_i8_fragments_exchange_bytes(m, n, k);
+    HTPOPS_HIP(ctx, htpops::launch_gemm_i8_fragments(ctx->stream, dst, act, frags, m, k, n, ws, ready,
+                                                     ws + plan.ws_bytes - ((xbytes + 255) & ~(size_t) 255), xbytes,
+                                                     ctx->tickets, kTicketSlots));
   }
   if (keep) {
     af.src = act, af.src_bytes = q8_0_bytes((size_t) m, (size_t) k), af.m = m, af.k = k, af.kind = (int) plan.kind;
@@ -1197,7 +1202,11 @@ int run_fragment_group(htpops_context *ctx, GemvBatch &b) {
     }
     act_of[i] = j;
   }
-  if (int r = ensure_workspace(ctx, total)) {
+  size_t xbytes = 0;  // scratch for the partial tiles of members whose K is split over workgroups, behind the activations
+  for (int i = 0; i < b.count; ++i) {
+    xbytes += htpops::gemm_i8_fragments_exchange_bytes(b.m, b.n[i], b.k[i]);
+  }
+  if (int r = ensure_workspace(ctx, total + xbytes)) {
     return r;
   }
   ctx->act_fragments.src = nullptr;
@@ -1211,7 +1220,8 @@ int run_fragment_group(htpops_context *ctx, GemvBatch &b) {
     af[i] = act_dst[act_of[i]];
   }
   HTPOPS_HIP(ctx, htpops::launch_act_to_i8_fragments_group(ctx->stream, n_acts, act_dst, acts, act_k, b.m));
-  HTPOPS_HIP(ctx, htpops::launch_gemm_i8_fragments_group(ctx->stream, b.count, b.out, af, wf, b.n, b.k, b.m));
+  HTPOPS_HIP(ctx, htpops::launch_gemm_i8_fragments_group(ctx->stream, b.count, b.out, af, wf, b.n, b.k, b.m, ws + total, xbytes,
+                                                         ctx->tickets, kTicketSlots));
   return HTPOPS_OK;
 }
 

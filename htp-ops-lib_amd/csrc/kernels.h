@@ -82,20 +82,25 @@ size_t     gemm_i8_weight_fragment_bytes(int k, int n);
 size_t     gemm_i8_act_fragment_bytes(int m, int k);
 hipError_t launch_weights_to_i8_fragments(hipStream_t stream, void *dst, const void *weight, int k, int n,
                                           WeightType wt);
+// `exchange` (gemm_i8_fragments_exchange_bytes; may be 0) and `tickets` (zeroed counters, left zeroed): scratch for shapes
+// whose K is split over workgroups. Without them those shapes run unsplit: correct, slower, and rounded differently.
+size_t     gemm_i8_fragments_exchange_bytes(int m, int n, int k);
 hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_fragments,
-                                    int m, int k, int n, void *act_fragments, bool act_fragments_ready);
+                                    int m, int k, int n, void *act_fragments, bool act_fragments_ready, void *exchange,
+                                    size_t exchange_bytes, unsigned *tickets, int ticket_slots);
 // The same for up to kGemmGroupMax matmuls of one row count m in one launch each for the conversions and the products:
 // member i multiplies the converted activations act_fragments[i] (gemm_i8_act_fragment_bytes(m, ks[i]) each; members
 // that read the same rows may share one) by weight_fragments[i]. Every member must be `groupable` (the tile
 // configuration it gets depends on (m, n) alone, and a launch has one), else hipErrorNotSupported; a member's result
-// is bit for bit what its own launch gives.
+// is bit for bit what its own launch gives, provided `exchange` holds the sum of the members' exchange bytes.
 constexpr int kGemmGroupMax = 8;
 bool       gemm_i8_fragments_groupable(int m, int n);
 hipError_t launch_act_to_i8_fragments_group(hipStream_t stream, int count, void *const *act_fragments,
                                             const void *const *acts_q8_0, const int *ks, int m);
 hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *const *outs,
                                           const void *const *act_fragments, const void *const *weight_fragments,
-                                          const int *ns, const int *ks, int m);
+                                          const int *ns, const int *ks, int m, void *exchange, size_t exchange_bytes,
+                                          unsigned *tickets, int ticket_slots);
 // picks between the one-row and the small-batch kernel by m (any m; many rows are better served by the fragment path)
 size_t     mat_mul_workspace_bytes(int m, int k, int n);
 hipError_t launch_mat_mul_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
