@@ -340,10 +340,23 @@ struct GemvMembers {
   int        count;
 };
 
+// The fused form of the launch: the activation row of EVERY member is the RMS-normalized, Q8_0-quantized image of one
+// fp32 row (the decode chain norm -> quantize -> projections as one launch). Each workgroup makes that image for itself
+// in LDS -- the first 256 threads repeat the fused RMSNorm + Q8_0 kernel's arithmetic thread for thread, so the bytes
+// are the ones that kernel writes -- and the first workgroup of the launch also writes it to `q_out`, where the
+// message asked for it.
+struct GemvNorm {
+  const float *src;     // fp32 [k]
+  const float *weight;  // fp32 [k] or nullptr
+  float        eps;
+  uint8_t     *q_out;   // block_q8_0 [k / 32]
+};
+
 // lanes per row x pairs per lane x waves per row
 enum { kShapeG16 = 0, kShapeG32 = 1, kShapeG64 = 2, kShapeG64x2 = 3, kShapeG64x2S2 = 4 };
 
 constexpr int kSharedActMaxPairs = 192;  // longest activation row the kernel stages (k = 12288)
+constexpr int kFusedNormMaxBlocks = 1024;  // most workgroups for which making the activation row in each of them pays
 constexpr int kRedDwords         = 16;   // LDS words in front of the staged row: partial sums of rows split over waves
 
 // One workgroup of WAVES waves. SEG = 1: wave `wave` computes rows row0 .. row0 + SLOTS * R - 1, SLOTS = 64 / G rows at
@@ -351,8 +364,8 @@ constexpr int kRedDwords         = 16;   // LDS words in front of the staged row
 // meet in LDS and are added in a fixed order (first half + second half) -- measured on MI355X, a wave that requests
 // more than about 4.6 KB of the stream at once (three pairs per lane, the k = 11008 rows on one wave) streams 10-25 %
 // slower than two waves with half of it each.
-template <int WT, int G, int ITERS, int R, int SEG, int WAVES>
-__device__ __forceinline__ void gemv_row_sets(const GemvMember &mem, int wg, uint32_t *lds) {
+template <int WT, int G, int ITERS, int R, int SEG, int WAVES, bool FUSED>
+__device__ __forceinline__ void gemv_row_sets(const GemvMember &mem, int wg, uint32_t *lds, const GemvNorm &norm) {
   static_assert(SEG == 1 || (G == kWave && R == 1 && WAVES % SEG == 0), "split rows: one row per wave pair");
   constexpr int PD      = Pair<WT>::kDwords;
   constexpr int SLOTS   = kWave / G;
@@ -383,9 +396,39 @@ __device__ __forceinline__ void gemv_row_sets(const GemvMember &mem, int wg, uin
   // about 4 % of a decoder layer's stream. Threads beyond the row inside such a wave re-read its last pair.
   uint32_t   araw[kActPairDwords];
   const bool stager = wave * kWave < pairs;
-  if (stager) {
+  if (!FUSED && stager) {
     const int my_pair = min((int) threadIdx.x, pairs - 1);
     load_dwords<kActPairDwords>(araw, act + (size_t) my_pair * kActPairDwords);
+  }
+  // fused form: this thread's slices of the fp32 row (8 floats each, slice = thread / 4 + 64 b is a quant block's
+  // quarter `thread % 4`), requested before the weights for the same reason
+  constexpr int BPT = FUSED ? (2 * TS + 63) / 64 : 1;
+  // (the norm weights too, instead of behind the sum of squares)
+  static_assert(!FUSED || BPT <= 2, "the fused form is for rows of up to 64 pairs");
+  float          xv[BPT][8], gv[BPT][8];
+  const int      nb = 2 * pairs, part = threadIdx.x & 3;
+  if (FUSED && threadIdx.x < 256) {
+#pragma unroll
+    for (int b = 0; b < BPT; ++b) {
+      const int blk = ((int) threadIdx.x >> 2) + b * 64;
+      if (blk < nb) {
+        const float4 *xp = reinterpret_cast<const float4 *>(norm.src + blk * kQK + part * 8);
+        const float4  a0 = xp[0], a1 = xp[1];
+        xv[b][0] = a0.x, xv[b][1] = a0.y, xv[b][2] = a0.z, xv[b][3] = a0.w;
+        xv[b][4] = a1.x, xv[b][5] = a1.y, xv[b][6] = a1.z, xv[b][7] = a1.w;
+        if (norm.weight) {
+          const float4 *wp = reinterpret_cast<const float4 *>(norm.weight + blk * kQK + part * 8);
+          const float4  w0 = wp[0], w1 = wp[1];
+          gv[b][0] = w0.x, gv[b][1] = w0.y, gv[b][2] = w0.z, gv[b][3] = w0.w;
+          gv[b][4] = w1.x, gv[b][5] = w1.y, gv[b][6] = w1.z, gv[b][7] = w1.w;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          xv[b][i] = 0.0f;
+        }
+      }
+    }
   }
 
   // Branch-free weight loads (so that the compiler can count them and wait per use): lanes without work read a
@@ -401,6 +444,89 @@ __device__ __forceinline__ void gemv_row_sets(const GemvMember &mem, int wg, uin
     }
   }
 
+  if (FUSED) {
+    // RMSNorm + Q8_0 of the row into an LDS image of its block_q8_0 bytes, in the arithmetic and the order of sums of
+    // rms_norm_quantize_kernel (256 threads, slices as above; the other waves add zeros)
+    float   *red = reinterpret_cast<float *>(lds);
+    uint8_t *img = reinterpret_cast<uint8_t *>(tab + TS * Prepared<WT>::kEntries);
+    float    ss  = 0.0f;
+    if (threadIdx.x < 256) {
+#pragma unroll
+      for (int b = 0; b < BPT; ++b) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          ss = __fmaf_rn(xv[b][i], xv[b][i], ss);
+        }
+      }
+    }
+    ss = group_sum<kWave>(ss);
+    if (lane == 0 && wave < 4) {
+      red[wave] = ss;
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // LDS only: the weight loads stay in flight
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    const float sum   = ((red[0] + red[1]) + red[2]) + red[3];
+    const float mean  = sum / (float) (nb * kQK);
+    const float scale = 1.0f / sqrtf(mean + norm.eps);
+    if (threadIdx.x < 256) {
+#pragma unroll
+      for (int b = 0; b < BPT; ++b) {
+        const int blk  = ((int) threadIdx.x >> 2) + b * 64;
+        float     amax = 0.0f;
+        float     y[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          y[i] = xv[b][i] * scale;
+        }
+        if (norm.weight && blk < nb) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            y[i] *= gv[b][i];
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          amax = fmaxf(amax, fabsf(y[i]));
+        }
+        amax           = group_max<4>(amax);
+        const float d  = amax / 127.0f;
+        const float id = (d != 0.0f) ? 1.0f / d : 0.0f;
+        if (blk < nb) {
+          uint16_t      *o16 = reinterpret_cast<uint16_t *>(img + (size_t) blk * 34);
+          uint16_t      *g16 = reinterpret_cast<uint16_t *>(norm.q_out + (size_t) blk * 34);
+          const bool     pub = blockIdx.x == 0;  // the first workgroup of the launch writes the row where it was asked for
+          const uint16_t dh  = __half_as_ushort(__float2half_rn(d));
+          if (part == 0) {
+            o16[0] = dh;
+            if (pub) {
+              g16[0] = dh;
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int      q0 = (int) roundf(y[2 * i] * id), q1 = (int) roundf(y[2 * i + 1] * id);
+            const uint16_t qq = (uint16_t) ((q0 & 0xff) | ((q1 & 0xff) << 8));
+            o16[1 + part * 4 + i] = qq;
+            if (pub) {
+              g16[1 + part * 4 + i] = qq;
+            }
+          }
+        }
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // LDS only: the weight loads stay in flight
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (stager) {
+      const int       my_pair = min((int) threadIdx.x, pairs - 1);
+      const uint32_t *ip      = reinterpret_cast<const uint32_t *>(img) + (size_t) my_pair * kActPairDwords;
+#pragma unroll
+      for (int i = 0; i < kActPairDwords; ++i) {
+        araw[i] = ip[i];
+      }
+    }
+  }
   if (stager) {
     ActPair<WT> ap;
     prepare(ap, araw);
@@ -455,9 +581,9 @@ __device__ __forceinline__ void gemv_row_sets(const GemvMember &mem, int wg, uin
 // The first workgroup of members 1..7 travels as plain leading arguments (INT_MAX for members that do not exist), the
 // first words of the argument block: a wave knows its member after one scalar load and fetches that member's record with
 // a second one, instead of walking the table in memory.
-template <int WT, bool LONG, int THREADS>
-__global__ __launch_bounds__(THREADS) void gemv_members_kernel(int b1, int b2, int b3, int b4, int b5, int b6, int b7,
-                                                               GemvMembers grp) {
+template <int WT, bool LONG, int THREADS, bool FUSED>
+__device__ __forceinline__ void gemv_members_body(int b1, int b2, int b3, int b4, int b5, int b6, int b7,
+                                                  const GemvMembers &grp, const GemvNorm &norm) {
   static_assert(kGemvGroupMax == 8, "one leading argument per member after the first");
   extern __shared__ __attribute__((aligned(16))) uint32_t gemv_lds[];
   constexpr int W   = THREADS / kWave;
@@ -467,17 +593,17 @@ __global__ __launch_bounds__(THREADS) void gemv_members_kernel(int b1, int b2, i
   const int         wg  = (int) blockIdx.x - mem.block0;
   const int         sel = mem.shape * 2 + (mem.r - 1);
   switch (sel) {
-    case kShapeG16 * 2 + 0: gemv_row_sets<WT, 16, 1, 1, 1, W>(mem, wg, gemv_lds); break;
-    case kShapeG16 * 2 + 1: gemv_row_sets<WT, 16, 1, 2, 1, W>(mem, wg, gemv_lds); break;
-    case kShapeG32 * 2 + 0: gemv_row_sets<WT, 32, 1, 1, 1, W>(mem, wg, gemv_lds); break;
-    case kShapeG32 * 2 + 1: gemv_row_sets<WT, 32, 1, 2, 1, W>(mem, wg, gemv_lds); break;
-    case kShapeG64 * 2 + 0: gemv_row_sets<WT, 64, 1, 1, 1, W>(mem, wg, gemv_lds); break;
-    case kShapeG64 * 2 + 1: gemv_row_sets<WT, 64, 1, 2, 1, W>(mem, wg, gemv_lds); break;
+    case kShapeG16 * 2 + 0: gemv_row_sets<WT, 16, 1, 1, 1, W, FUSED>(mem, wg, gemv_lds, norm); break;
+    case kShapeG16 * 2 + 1: gemv_row_sets<WT, 16, 1, 2, 1, W, FUSED>(mem, wg, gemv_lds, norm); break;
+    case kShapeG32 * 2 + 0: gemv_row_sets<WT, 32, 1, 1, 1, W, FUSED>(mem, wg, gemv_lds, norm); break;
+    case kShapeG32 * 2 + 1: gemv_row_sets<WT, 32, 1, 2, 1, W, FUSED>(mem, wg, gemv_lds, norm); break;
+    case kShapeG64 * 2 + 0: gemv_row_sets<WT, 64, 1, 1, 1, W, FUSED>(mem, wg, gemv_lds, norm); break;
+    case kShapeG64 * 2 + 1: gemv_row_sets<WT, 64, 1, 2, 1, W, FUSED>(mem, wg, gemv_lds, norm); break;
     default:
-      if (LONG) {
+      if constexpr (LONG) {
         switch (sel) {
-          case kShapeG64x2 * 2 + 0: gemv_row_sets<WT, 64, 2, 1, 1, W>(mem, wg, gemv_lds); break;
-          case kShapeG64x2S2 * 2 + 0: gemv_row_sets<WT, 64, 2, 1, 2, W>(mem, wg, gemv_lds); break;
+          case kShapeG64x2 * 2 + 0: gemv_row_sets<WT, 64, 2, 1, 1, W, FUSED>(mem, wg, gemv_lds, norm); break;
+          case kShapeG64x2S2 * 2 + 0: gemv_row_sets<WT, 64, 2, 1, 2, W, FUSED>(mem, wg, gemv_lds, norm); break;
           default: break;
         }
       }
@@ -485,9 +611,21 @@ __global__ __launch_bounds__(THREADS) void gemv_members_kernel(int b1, int b2, i
   }
 }
 
-// Fills shape, r and block0 of every member and launches.
+template <int WT, bool LONG, int THREADS>
+__global__ __launch_bounds__(THREADS) void gemv_members_kernel(int b1, int b2, int b3, int b4, int b5, int b6, int b7,
+                                                               GemvMembers grp) {
+  gemv_members_body<WT, LONG, THREADS, false>(b1, b2, b3, b4, b5, b6, b7, grp, GemvNorm{});
+}
+
+template <int WT, bool LONG, int THREADS>
+__global__ __launch_bounds__(THREADS) void gemv_members_norm_kernel(int b1, int b2, int b3, int b4, int b5, int b6, int b7,
+                                                                    GemvMembers grp, GemvNorm norm) {
+  gemv_members_body<WT, LONG, THREADS, true>(b1, b2, b3, b4, b5, b6, b7, grp, norm);
+}
+
+// Fills shape, r and block0 of every member and launches; with `norm`, the fused form (see GemvNorm).
 template <int WT>
-hipError_t launch_gemv_members(hipStream_t stream, GemvMembers &grp) {
+hipError_t launch_gemv_members(hipStream_t stream, GemvMembers &grp, const GemvNorm *norm = nullptr) {
   // measured on MI355X: short-lived waves (one row set each) stream best; only very wide launches of short rows
   // (gate + up of a 7B layer: 22016 rows of 64 pairs) gain from two rows per lane group
   long total_short_rows = 0;
@@ -522,15 +660,23 @@ hipError_t launch_gemv_members(hipStream_t stream, GemvMembers &grp) {
       return hipErrorNotSupported;
     }
     mem.shape = p <= 16 ? kShapeG16 : p <= 32 ? kShapeG32 : p <= 64 ? kShapeG64 : p <= 128 ? kShapeG64x2 : kShapeG64x2S2;
-    mem.r     = (p <= 64 && total_short_rows >= 16384) ? 2 : 1;
+    mem.r     = (p <= 64 && (total_short_rows >= 16384 || norm)) ? 2 : 1;
     max_pairs = p > max_pairs ? p : max_pairs;
     any_long  = any_long || p > 64;
   }
-  const int threads = place(512, false) >= 1024 ? 512 : kThreads;
+  // (making the activation row is work per workgroup: the fused form takes the fewest, largest workgroups)
+  const int threads = (norm || place(512, false) >= 1024) ? 512 : kThreads;
   const int blocks = place(threads, true);
+  // Measured on MI355X with Q4_0 weights of k = 4096: making the row costs every workgroup about as much as 8 KB of its
+  // weight stream, which beats a launch of its own (3.5-4 us behind another) up to about a thousand workgroups:
+  // n = 4096: 5.2 us against 7.0 us, 3 x 4096: 9.0 / 10.4, 2 x 11008: 16.4 / 14.5. Longer rows cost in proportion.
+  if (norm && (any_long || blocks > kFusedNormMaxBlocks)) {
+    return hipErrorNotSupported;
+  }
   // the table stride of the widest body among the members (see TS in gemv_row_sets)
   const int    table_pairs = max_pairs <= 16 ? 16 : max_pairs <= 32 ? 32 : max_pairs <= 64 ? 64 : max_pairs <= 128 ? 128 : kSharedActMaxPairs;
-  const size_t lds = (size_t) (kRedDwords + table_pairs * Prepared<WT>::kEntries) * 4;
+  const size_t lds = (size_t) (kRedDwords + table_pairs * Prepared<WT>::kEntries) * 4 +
+                     (norm ? (size_t) max_pairs * 2 * 34 + 4 : 0);  // + the LDS image of the quantized row
   const dim3   grid((unsigned) blocks);
   int b[kGemvGroupMax];
   for (int i = 1; i < kGemvGroupMax; ++i) {
@@ -538,7 +684,10 @@ hipError_t launch_gemv_members(hipStream_t stream, GemvMembers &grp) {
   }
 #define HTPOPS_GEMV_LAUNCH(LONG, T) \
   hipLaunchKernelGGL((gemv_members_kernel<WT, LONG, T>), grid, dim3(T), lds, stream, b[1], b[2], b[3], b[4], b[5], b[6], b[7], grp)
-  if (threads == 512) {
+  if (norm) {
+    hipLaunchKernelGGL((gemv_members_norm_kernel<WT, false, 512>), grid, dim3(512), lds, stream, b[1], b[2], b[3], b[4],
+                       b[5], b[6], b[7], grp, *norm);
+  } else if (threads == 512) {
     if (any_long) {
       HTPOPS_GEMV_LAUNCH(true, 512);
     } else {
@@ -781,6 +930,32 @@ hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *cons
     grp.m[i].out = outs[i], grp.m[i].n = ns[i], grp.m[i].pairs = nblk / 2;
   }
   return wt == kQ4_0 ? launch_gemv_members<kQ4_0>(stream, grp) : launch_gemv_members<kQ8_0>(stream, grp);
+}
+
+// The decode chain as one launch: every member's activation row is RMSNorm(src [* norm_weight]) quantized to Q8_0,
+// made by each workgroup for itself and also written to `q_out` (k / 32 blocks), bit for bit what
+// launch_rms_norm_quantize_q8_0 writes. k % 64 == 0, k <= 4096, 16-byte aligned src / norm_weight and few enough
+// weight rows that it pays (see launch_gemv_members), else hipErrorNotSupported and nothing is launched.
+hipError_t launch_gemv_group_rms_norm_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *const *weights,
+                                               const int *ns, int k, WeightType wt, const float *src,
+                                               const float *norm_weight, float eps, void *q_out) {
+  const int nblk = k / kQK;
+  if (count < 1 || count > kGemvGroupMax || k % (2 * kQK) != 0 || nblk / 2 > kSharedActMaxPairs ||
+      (reinterpret_cast<uintptr_t>(src) & 15) != 0 || (reinterpret_cast<uintptr_t>(norm_weight) & 15) != 0 ||
+      (reinterpret_cast<uintptr_t>(q_out) & 3) != 0) {
+    return hipErrorNotSupported;
+  }
+  GemvMembers grp = {};
+  grp.count       = count;
+  for (int i = 0; i < count; ++i) {
+    if ((reinterpret_cast<uintptr_t>(weights[i]) & 3) != 0) {
+      return hipErrorNotSupported;
+    }
+    grp.m[i].w = static_cast<const uint32_t *>(weights[i]), grp.m[i].act = static_cast<const uint32_t *>(q_out);
+    grp.m[i].out = outs[i], grp.m[i].n = ns[i], grp.m[i].pairs = nblk / 2;
+  }
+  const GemvNorm norm = { src, norm_weight, eps, static_cast<uint8_t *>(q_out) };
+  return wt == kQ4_0 ? launch_gemv_members<kQ4_0>(stream, grp, &norm) : launch_gemv_members<kQ8_0>(stream, grp, &norm);
 }
 
 bool gemv_rows_fits(int m, int k, WeightType wt) {

@@ -1160,6 +1160,17 @@ struct GemvBatch {
   const void           *act[htpops::kGemvGroupMax];
   int                   n[htpops::kGemvGroupMax];
   int                   k[htpops::kGemvGroupMax];
+  // A one-row RMSNorm + Q8_0 request that waits for the matmuls that read its row (the decode chain): when only such
+  // matmuls follow, one launch makes the row and multiplies by it; anything else runs the request first, as it came.
+  struct {
+    bool                  waiting = false;
+    struct RequestHeader *hdr     = nullptr;
+    void                 *dst     = nullptr;
+    const float          *src = nullptr, *weight = nullptr;
+    float                 eps = 0.0f;
+    int                   ne0 = 0;
+  } norm;
+  bool fused = false;  // the members read norm.dst and run in the launch that makes it
 };
 
 // The many-row members of a batch: converted weights from the cache (made now where missing), the distinct activation
@@ -1226,6 +1237,36 @@ int run_fragment_group(htpops_context *ctx, GemvBatch &b) {
 }
 
 void flush_batch(htpops_context *ctx, GemvBatch &b) {
+  if (b.norm.waiting) {
+    b.norm.waiting = false;
+    const size_t q_bytes = q8_0_bytes(1, (size_t) b.norm.ne0);
+    if (b.fused && b.count > 0) {
+      b.fused = false;
+      note_device_write(ctx, b.norm.dst, q_bytes);
+      for (int i = 0; i < b.count; ++i) {
+        note_device_write(ctx, b.out[i], (size_t) b.n[i] * 4);
+      }
+      const hipError_t e = htpops::launch_gemv_group_rms_norm_q8_0_act(ctx->stream, b.count, b.out, b.w, b.n, b.norm.ne0,
+                                                                       (htpops::WeightType) b.wt, b.norm.src,
+                                                                       b.norm.weight, b.norm.eps, b.norm.dst);
+      if (e != hipErrorNotSupported) {
+        ++ctx->message_submissions;
+        if (e != hipSuccess) {
+          const int ret = fail(ctx, HTPOPS_ERR_HIP, "rms_norm + mat_mul launch: %s", hipGetErrorString(e));
+          b.norm.hdr->state = ret;
+          for (int i = 0; i < b.count; ++i) {
+            b.hdr[i]->state = ret;
+          }
+        }
+        b.count = 0;
+        return;
+      }
+      (void) hipGetLastError();
+    }
+    b.fused = false;
+    ++ctx->message_submissions;
+    b.norm.hdr->state = op_rms_norm_quantize(ctx, b.norm.dst, b.norm.src, b.norm.weight, b.norm.eps, b.norm.ne0, 1);
+  }
   if (b.count == 0) {
     return;
   }
@@ -1316,6 +1357,29 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
   b.count = 0;
 }
 
+// true: the one-row RMSNorm + Q8_0 request now waits in the (empty) batch for the matmuls behind it; false: run it now
+bool try_defer_norm(htpops_context *ctx, const struct OpComputeRequest *req, struct RequestHeader *hdr, GemvBatch &b) {
+  const auto *p = reinterpret_cast<const RmsNormExParams *>(req->payload);
+  if (!ctx->has_device || p->ne1 != 1 || p->ne0 <= 0 || p->ne0 % 64 != 0 || p->ne0 > 4096) {
+    return false;
+  }
+  const size_t src_bytes = (size_t) p->ne0 * 4, q_bytes = q8_0_bytes(1, (size_t) p->ne0);
+  const float *w = nullptr;
+  if (p->weight.fd >= 0 && !(w = (const float *) resolve(ctx, p->weight, src_bytes))) {
+    return false;
+  }
+  const float *src = (const float *) resolve(ctx, p->src, src_bytes);
+  void        *dst = resolve(ctx, p->dst, q_bytes);
+  if (!src || !dst || !aligned(dst, 4) || !aligned(src, 16) || (w && !aligned(w, 16)) ||
+      ranges_overlap(dst, q_bytes, src, src_bytes) || (w && ranges_overlap(dst, q_bytes, w, src_bytes))) {
+    return false;  // the ordinary path reports what is wrong; a row quantized in place keeps its own launch
+  }
+  b.norm.waiting = true, b.norm.hdr = hdr, b.norm.dst = dst, b.norm.src = src, b.norm.weight = w, b.norm.eps = p->eps;
+  b.norm.ne0 = p->ne0;
+  hdr->state = HTPOPS_OK;
+  return true;
+}
+
 // true: the request is now part of the batch and its state is set; false: run it the ordinary way (after a flush)
 bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct RequestHeader *hdr, GemvBatch &b) {
   if (!ctx->has_device ||
@@ -1349,7 +1413,20 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
       return false;
     }
   }
-  bool join = b.count > 0 && b.count < htpops::kGemvGroupMax && b.wt == wt && b.m == p->m &&
+  // behind a waiting RMSNorm + Q8_0 request: only one-row matmuls over the row it makes, whose outputs leave its
+  // operands alone, can run in its launch
+  const bool reads_norm = b.norm.waiting && p->m == 1 && act == b.norm.dst && p->k == b.norm.ne0 &&
+                          !ranges_overlap(out, out_bytes, b.norm.src, (size_t) p->k * 4) &&
+                          !(b.norm.weight && ranges_overlap(out, out_bytes, b.norm.weight, (size_t) p->k * 4)) &&
+                          !ranges_overlap(w, w_bytes, b.norm.dst, act_bytes);
+  if (b.norm.waiting && b.count == 0) {
+    if (reads_norm) {
+      b.fused = true;
+    } else {
+      flush_batch(ctx, b);  // runs the waiting request by itself
+    }
+  }
+  bool join = b.count > 0 && b.count < htpops::kGemvGroupMax && b.wt == wt && b.m == p->m && (!b.fused || reads_norm) &&
               (p->m == 1 || many_rows || b.k[0] == p->k ||
                (htpops::gemv_rows_fits(p->m, p->k, (htpops::WeightType) wt) &&
                 htpops::gemv_rows_fits(b.m, b.k[0], (htpops::WeightType) wt)));
@@ -1363,7 +1440,9 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
            !ranges_overlap(b.out[i], oi, act, act_bytes);
   }
   if (!join) {
-    flush_batch(ctx, b);
+    if (b.count > 0) {
+      flush_batch(ctx, b);
+    }
     b.wt = wt, b.m = p->m;
   }
   b.hdr[b.count] = hdr, b.out[b.count] = out, b.w[b.count] = w, b.act[b.count] = act, b.n[b.count] = p->n, b.k[b.count] = p->k;
@@ -1418,7 +1497,14 @@ int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_b
           const auto *req = reinterpret_cast<const struct OpComputeRequest *>(hdr->data);
           const bool  matmul_payload =
             size >= sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest) + sizeof(MatMulParams);
-          if (!(matmul_payload && try_batch(ctx, req, hdr, batch))) {
+          const bool  norm_payload =
+            req->op == HTP_OPS_RMS_NORM_QUANTIZE_Q8_0 &&
+            size >= sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest) + sizeof(RmsNormExParams);
+          if (norm_payload) {
+            flush_batch(ctx, batch);
+          }
+          if (!(norm_payload && try_defer_norm(ctx, req, hdr, batch)) &&
+              !(matmul_payload && try_batch(ctx, req, hdr, batch))) {
             flush_batch(ctx, batch);
             ++ctx->message_submissions;
             hdr->state = htpops_execute_op(ctx, req);

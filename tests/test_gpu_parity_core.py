@@ -791,6 +791,109 @@ def test_message_groups_independent_few_row_matmuls(ctx, oracle, wt, m):
             ctx.release(h)
 
 
+def _norm_q(hq, hx, hg, k, rows, eps):
+    return (api.REQUEST_TYPE_OP_COMPUTE,
+            api.op_compute_request(api.HTP_OPS_RMS_NORM_QUANTIZE_Q8_0, api.rms_norm_ex_params((hq, 0), (hx, 0), (hg, 0), k, rows, eps)))
+
+
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+@pytest.mark.parametrize("k,wide", [(64, False), (1024, False), (1536, False), (4096, False), (4096, True), (8192, False),
+                                    (11008, False)])
+@pytest.mark.parametrize("with_weight", [True, False])
+def test_message_decode_chain_in_one_launch(ctx, oracle, wt, k, wide, with_weight):
+    # RMSNorm -> Q8_0 of one row followed by the one-row matmuls that read it (q/k/v or gate/up of a decoder layer) is one
+    # launch: every workgroup makes the row for itself. The Q8_0 row written must be the bytes of the op run alone, and
+    # every product the bits of its own launch over that row. Rows longer than 4096 and launches of more than about a
+    # thousand workgroups (`wide`: gate and up of a 7B layer) keep the two launches, where that is faster.
+    rng = wl.rng_for(77, wt * 100000 + k * 4 + int(with_weight) * 2 + int(wide))
+    op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
+    ns = [11008, 11008] if wide else [256, 1000, 48]
+    launches = 1 if k <= 4096 and not wide else 2
+    x = wl.make_activations(rng, 1, k)
+    g = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32) if with_weight else None
+    ws = [wl.make_weights(rng, n, k, wt) for n in ns]
+    hx, hq = ctx.upload(x), ctx.alloc(k // 32 * 34)
+    hg = ctx.upload(g) if with_weight else -1
+    hws, hos = [ctx.upload(w) for w in ws], [ctx.alloc(n * 4) for n in ns]
+    try:
+        q_alone = ctx.run_rms_norm(x, g, 1e-6, quantize=True)
+        want_q = oracle.quantize_q8_0(oracle.rms_norm(x, g if with_weight else np.ones(k, np.float32), 1e-6))
+        assert np.count_nonzero(q_alone != want_q) <= q_alone.size // 100   # (last-bit differences before rounding only)
+        msg = api.build_message([_norm_q(hq, hx, hg, k, 1, 1e-6)] + [_mm(op, ho, hq, hw, 1, k, n) for ho, hw, n in zip(hos, hws, ns)])
+        for _ in range(2):
+            ctx.write(hq, np.full(k // 32 * 34, 0xA5, np.uint8))
+            for ho, n in zip(hos, ns):
+                ctx.write(ho, np.full(n, np.nan, np.float32))
+            assert ctx.process_message(msg) == 0
+            assert api.message_request_states(msg) == [0] * (1 + len(ns)), ctx.last_error()
+            assert ctx.last_message_submissions() == launches
+            assert np.array_equal(ctx.read(hq, np.uint8, k // 32 * 34), q_alone[0]), "the row differs from the op run alone"
+            for ho, w, n in zip(hos, ws, ns):
+                got = ctx.read(ho, np.float32, n)
+                assert np.array_equal(got, ctx.run_mat_mul(q_alone, w, 1, k, n, wt)[0]), "a request differs from its own launch"
+                want, mag = oracle.mat_mul_q8_0_act_f64(q_alone, w, 1, k, n, wt)
+                assert np.all(np.abs(got - want[0]) <= MATMUL_RTOL * mag[0])
+    finally:
+        for h in [hx, hq] + hws + hos + ([hg] if with_weight else []):
+            ctx.release(h)
+
+
+def test_message_decode_chain_keeps_its_own_launch_when_it_must(ctx, oracle):
+    # The RMSNorm -> Q8_0 request runs by itself, in order, when what follows cannot share its launch: a matmul over another
+    # row, a matmul whose output lands on the request's input, several rows, the end of the message; and matmuls that
+    # read the new row after a request that could not join still see it.
+    wt, op = wl.GGML_TYPE_Q8_0, api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
+    rng = wl.rng_for(78, 0)
+    k, n = 1024, 256
+    x = wl.make_activations(rng, 2, k)
+    g = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    w, w2 = wl.make_weights(rng, n, k, wt), wl.make_weights(rng, n, k, wt)
+    other = oracle.quantize_q8_0(wl.make_activations(rng, 1, k))
+    hx, hg, hw, hw2, hother = ctx.upload(x), ctx.upload(g), ctx.upload(w), ctx.upload(w2), ctx.upload(other)
+    hq, ho, ho2 = ctx.alloc(2 * (k // 32) * 34), ctx.alloc(2 * n * 4), ctx.alloc(n * 4)
+    hxo = ctx.alloc(k * 4)                                     # a row that a matmul overwrites (n = 256 of its floats)
+    try:
+        q1 = ctx.run_rms_norm(x[:1], g, 1e-6, quantize=True)
+        q2 = ctx.run_rms_norm(x, g, 1e-6, quantize=True)
+
+        def run(reqs, submissions):
+            ctx.write(hq, np.full(2 * (k // 32) * 34, 0xA5, np.uint8))
+            ctx.write(hxo, x[0])
+            msg = api.build_message(reqs)
+            assert ctx.process_message(msg) == 0
+            assert api.message_request_states(msg) == [0] * len(reqs), ctx.last_error()
+            assert ctx.last_message_submissions() == submissions
+
+        # another row first, then the new one: the norm by itself, then the two matmuls together
+        run([_norm_q(hq, hx, hg, k, 1, 1e-6), _mm(op, ho2, hother, hw2, 1, k, n), _mm(op, ho, hq, hw, 1, k, n)], 2)
+        assert np.array_equal(ctx.read(hq, np.uint8, k // 32 * 34), q1[0])
+        assert np.array_equal(ctx.read(ho, np.float32, n), ctx.run_mat_mul(q1, w, 1, k, n, wt)[0])
+        assert np.array_equal(ctx.read(ho2, np.float32, n), ctx.run_mat_mul(other, w2, 1, k, n, wt)[0])
+        # the new row, then a request over another row: the first two share a launch, the third has its own
+        run([_norm_q(hq, hx, hg, k, 1, 1e-6), _mm(op, ho, hq, hw, 1, k, n), _mm(op, ho2, hother, hw2, 1, k, n)], 2)
+        assert np.array_equal(ctx.read(ho, np.float32, n), ctx.run_mat_mul(q1, w, 1, k, n, wt)[0])
+        assert np.array_equal(ctx.read(ho2, np.float32, n), ctx.run_mat_mul(other, w2, 1, k, n, wt)[0])
+        # the matmul writes over the row that the norm reads: norm first, then the matmul
+        run([_norm_q(hq, hxo, hg, k, 1, 1e-6), _mm(op, hxo, hq, hw, 1, k, n)], 2)
+        assert np.array_equal(ctx.read(hq, np.uint8, k // 32 * 34), q1[0])
+        assert np.array_equal(ctx.read(hxo, np.float32, n), ctx.run_mat_mul(q1, w, 1, k, n, wt)[0])
+        # two rows: the ordinary two launches
+        run([_norm_q(hq, hx, hg, k, 2, 1e-6), _mm(op, ho, hq, hw, 2, k, n)], 2)
+        assert np.array_equal(ctx.read(hq, np.uint8, 2 * (k // 32) * 34), q2.reshape(-1))
+        assert np.array_equal(ctx.read(ho, np.float32, 2 * n).reshape(2, n), ctx.run_mat_mul(q2, w, 2, k, n, wt))
+        # nothing behind it
+        run([_norm_q(hq, hx, hg, k, 1, 1e-6)], 1)
+        assert np.array_equal(ctx.read(hq, np.uint8, k // 32 * 34), q1[0])
+        # two chains in one message: each is one launch
+        run([_norm_q(hq, hx, hg, k, 1, 1e-6), _mm(op, ho, hq, hw, 1, k, n),
+             _norm_q(hq, hx, hg, k, 1, 1e-6), _mm(op, ho2, hq, hw2, 1, k, n)], 2)
+        assert np.array_equal(ctx.read(ho, np.float32, n), ctx.run_mat_mul(q1, w, 1, k, n, wt)[0])
+        assert np.array_equal(ctx.read(ho2, np.float32, n), ctx.run_mat_mul(q1, w2, 1, k, n, wt)[0])
+    finally:
+        for h in (hx, hg, hw, hw2, hother, hq, ho, ho2, hxo):
+            ctx.release(h)
+
+
 def test_message_keeps_dependent_gemvs_in_order(ctx, oracle):
     # Requests with a data dependency must not share a launch. (1) read-after-write: request 1's fp32 output bytes are
     # request 2's Q8_0 activation row (unit scales and small integers make those bytes finite Q8_0 blocks);
