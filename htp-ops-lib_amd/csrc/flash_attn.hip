@@ -16,7 +16,8 @@
 //    no rescaling. Under `causal`, KV blocks above the diagonal are skipped and the longest query blocks start first.
 //  * decode (qo_len == 1, head_dim 64 or 128): bandwidth bound. The KV range is split across workgroups (n_kv_heads
 //    alone would leave the GPU idle); 16 lanes share a key (16 bytes of K and V each), all heads of the GQA group are
-//    scored against the same K/V registers, and a second tiny kernel merges the per-split (max, sum, O) partials.
+//    scored against the same K/V registers, and a second tiny kernel merges the per-split (max, sum, O) partials in
+//    one trip to memory.
 //  * any other even head_dim up to 256 (the reference's flash_attn_sp_hdim.c domain): a plain kernel without MFMA.
 #include "device_utils.h"
 #include "kernels.h"
@@ -431,24 +432,31 @@ __device__ __forceinline__ float key_group_sum(float v) {
 }
 
 // partial record per (head, split): m, l, then D floats of un-normalised O.
-// A workgroup owns SPLIT consecutive keys of one KV head. LPK = D / 8 lanes share a key (16 bytes of K and of
-// V each); every K and V load of the wave is issued before the first use, the scores of all GH heads are formed
-// against the same registers, and the per-slot (max, sum, O) partials are merged through LDS.
-template <int D, int GH, bool QO_F32, int SPLIT>
-__global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *__restrict__ part,
-                                                                        const void *__restrict__ q_ptr,
-                                                                        const _Float16 *__restrict__ k_ptr,
-                                                                        const _Float16 *__restrict__ v_ptr,
-                                                                        const _Float16 *__restrict__ mask, int kv_len,
-                                                                        int n_heads, int n_kv_heads, int head0_in_group,
-                                                                        int n_splits) {
+// A workgroup of THREADS threads owns SPLIT consecutive keys of one KV head. LPK = D / 8 lanes share a key (16 bytes of
+// K and of V each); every K and V load of the wave is issued before the first use and the scores of all GH heads are
+// formed against the same registers. The workgroup agrees on one maximum per head (lane exchange inside the wave, LDS
+// between the waves) BEFORE the exponentials, so the per-slot sums and O columns only have to be added up.
+// Measured on MI355X (32 query / 8 KV heads of 128, kv_len 4096, cold K/V): a call is 11.3-11.5 us of which about 9 us
+// are the two dependent launches themselves (the same call reading an eighth of the keys: 9.0 us; without the score
+// and P V arithmetic: 10.7 us); 512 threads per workgroup change nothing. Merging inside this launch -- records
+// written through, a ticket per KV head, the last workgroup merges -- is slower (18-19 us, 47 us at kv_len 16384):
+// the 32 to 128 ticket updates of one counter from all over the chip are served one after the other.
+template <int D, int GH, bool QO_F32, int SPLIT, int THREADS>
+__global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__restrict__ part,
+                                                                    const void *__restrict__ q_ptr,
+                                                                    const _Float16 *__restrict__ k_ptr,
+                                                                    const _Float16 *__restrict__ v_ptr,
+                                                                    const _Float16 *__restrict__ mask, int kv_len,
+                                                                    int n_heads, int n_kv_heads, int head0_in_group,
+                                                                    int n_splits) {
   constexpr int LPK    = D / 8;        // lanes per key (8 halfs = 16 bytes each)
   constexpr int KPW    = kWave / LPK;  // keys per wave per pass
-  constexpr int WAVES  = kDecThreads / kWave;
+  constexpr int WAVES  = THREADS / kWave;
   constexpr int SLOTS  = WAVES * KPW;  // independent partial streams in the workgroup
   constexpr int PASSES = SPLIT / SLOTS;
-  static_assert(SPLIT % SLOTS == 0, "whole passes");
-  __shared__ float red_m[SLOTS][GH], red_l[SLOTS][GH], red_o[SLOTS][GH][D];
+  static_assert(SPLIT % SLOTS == 0 && PASSES >= 1, "whole passes");
+  extern __shared__ float dec_lds[];  // red_o[SLOTS][GH][D], red_l[SLOTS][GH], red_m[WAVES][GH]
+  float *red_o = dec_lds, *red_l = dec_lds + SLOTS * GH * D, *red_m = red_l + SLOTS * GH;
 
   const int group = n_heads / n_kv_heads;
   const int h_kv  = blockIdx.y;
@@ -483,10 +491,10 @@ __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *_
     const int    hg   = min(head0_in_group + g, group - 1);
     const size_t base = (size_t) (h_kv * group + hg) * D + sub * 8;
     if (QO_F32) {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        q[g][e] = reinterpret_cast<const float *>(q_ptr)[base + e] * scale;
-      }
+      const float4 *qp = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(q_ptr) + base);
+      const float4  q0 = qp[0], q1 = qp[1];
+      q[g][0] = q0.x * scale, q[g][1] = q0.y * scale, q[g][2] = q0.z * scale, q[g][3] = q0.w * scale;
+      q[g][4] = q1.x * scale, q[g][5] = q1.y * scale, q[g][6] = q1.z * scale, q[g][7] = q1.w * scale;
     } else {
       const v8h qv = *reinterpret_cast<const v8h *>(reinterpret_cast<const _Float16 *>(q_ptr) + base);
 #pragma unroll
@@ -528,11 +536,29 @@ __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *_
       m_loc[g] = fmaxf(m_loc[g], s);
     }
   }
-  float o[GH][8], l_loc[GH];
+  // one maximum per head for the whole workgroup: over the wave's key slots, then over the waves
 #pragma unroll
   for (int g = 0; g < GH; ++g) {
-    const float m_safe = (m_loc[g] == -INFINITY) ? 0.0f : m_loc[g];
-    l_loc[g]           = 0.0f;
+#pragma unroll
+    for (int off = LPK; off < kWave; off <<= 1) {
+      m_loc[g] = fmaxf(m_loc[g], __shfl_xor(m_loc[g], off, kWave));
+    }
+    if (lane == 0) {
+      red_m[wave * GH + g] = m_loc[g];
+    }
+  }
+  __syncthreads();
+  float o[GH][8];
+#pragma unroll
+  for (int g = 0; g < GH; ++g) {
+    float m_all = red_m[g];
+#pragma unroll
+    for (int w = 1; w < WAVES; ++w) {
+      m_all = fmaxf(m_all, red_m[w * GH + g]);
+    }
+    m_loc[g]           = m_all;
+    const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
+    float       l_loc  = 0.0f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       o[g][e] = 0.0f;
@@ -540,112 +566,90 @@ __global__ __launch_bounds__(kDecThreads) void flash_attn_decode_kernel(float *_
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       const float pr = fast_exp2(sc[p][g] - m_safe);
-      l_loc[g] += pr;
+      l_loc += pr;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         o[g][e] += pr * (float) vreg[p][e];
       }
     }
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      red_o[slot][g][sub * 8 + e] = o[g][e];
-    }
+    float4 *dst = reinterpret_cast<float4 *>(red_o + ((size_t) slot * GH + g) * D + sub * 8);
+    dst[0]      = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
+    dst[1]      = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
     if (sub == 0) {
-      red_m[slot][g] = m_loc[g], red_l[slot][g] = l_loc[g];
+      red_l[slot * GH + g] = l_loc;
     }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < GH * D; i += kDecThreads) {
+  // add the slots up: two neighbouring columns per thread
+  for (int i = threadIdx.x * 2; i < GH * D; i += THREADS * 2) {
     const int g = i / D, d = i % D;
     if (head0_in_group + g >= group) {
       continue;
     }
-    float m_all = -INFINITY;
+    float v0 = 0.0f, v1 = 0.0f, l = 0.0f;
 #pragma unroll
     for (int w = 0; w < SLOTS; ++w) {
-      m_all = fmaxf(m_all, red_m[w][g]);
-    }
-    const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
-    float       l = 0.0f, v = 0.0f;
-#pragma unroll
-    for (int w = 0; w < SLOTS; ++w) {
-      const float f = fast_exp2(red_m[w][g] - m_safe);
-      l += red_l[w][g] * f;
-      v += red_o[w][g][d] * f;
+      const float2 x = *reinterpret_cast<const float2 *>(red_o + ((size_t) w * GH + g) * D + d);
+      v0 += x.x, v1 += x.y;
     }
     const int head = h_kv * group + head0_in_group + g;
     float    *rec  = part + ((size_t) head * n_splits + split) * (D + 2);
     if (d == 0) {
-      rec[0] = m_all, rec[1] = l;
+#pragma unroll
+      for (int w = 0; w < SLOTS; ++w) {
+        l += red_l[w * GH + g];
+      }
+      float m_all = red_m[g];
+#pragma unroll
+      for (int w = 1; w < WAVES; ++w) {
+        m_all = fmaxf(m_all, red_m[w * GH + g]);
+      }
+      *reinterpret_cast<float2 *>(rec) = make_float2(m_all, l);
     }
-    rec[2 + d] = v;
+    *reinterpret_cast<float2 *>(rec + 2 + d) = make_float2(v0, v1);
   }
 }
+
+// One workgroup per head, one thread per output column. Splits are taken 64 at a time with every load of a chunk -- the
+// (max, sum) pair of split `lane` and this thread's column of all 64 records -- requested before the first use, so a
+// chunk costs one trip to memory (kv_len up to 8192 at 128 keys per split: the whole merge is one trip). Each
+// wave works the rescale factors out for itself (lane s holds that of split s, read back with v_readlane), so there
+// is neither LDS nor a barrier; chunks are folded into a running (max, sum, column) like KV blocks are.
+constexpr int kMergeChunk = 64;
 
 template <int D, bool QO_F32>
 __global__ __launch_bounds__(D) void flash_attn_decode_merge_kernel(void *__restrict__ o_ptr,
                                                                     const float *__restrict__ part, int n_splits) {
-  // phase 1: the (max, sum) heads of all splits are fetched in parallel and turned into rescale factors in LDS;
-  // phase 2: every thread sums its column with independent loads.
-  extern __shared__ float merge_f[];  // [n_splits] factors, then [1] total
-  __shared__ float        merge_red[2][D / kWave > 0 ? D / kWave : 1];
-  const int    head = blockIdx.x, d = threadIdx.x;
+  const int    head = blockIdx.x, d = threadIdx.x, lane = threadIdx.x & (kWave - 1);
   const float *rec0 = part + (size_t) head * n_splits * (D + 2);
-  float        m_loc = -INFINITY;
-  for (int s = d; s < n_splits; s += D) {
-    m_loc = fmaxf(m_loc, rec0[(size_t) s * (D + 2)]);
-  }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    m_loc = fmaxf(m_loc, __shfl_xor(m_loc, off));
-  }
-  if ((d & 63) == 0) {
-    merge_red[0][d >> 6] = m_loc;
-  }
-  __syncthreads();
-  float m_all = merge_red[0][0];
-#pragma unroll
-  for (int w = 1; w < D / kWave; ++w) {
-    m_all = fmaxf(m_all, merge_red[0][w]);
-  }
-  const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
-  float       l_loc  = 0.0f;
-  for (int s = d; s < n_splits; s += D) {
-    const float *rec = rec0 + (size_t) s * (D + 2);
-    const float  f   = fast_exp2(rec[0] - m_safe);
-    merge_f[s]       = f;
-    l_loc += rec[1] * f;
-  }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    l_loc += __shfl_xor(l_loc, off);
-  }
-  if ((d & 63) == 0) {
-    merge_red[1][d >> 6] = l_loc;
-  }
-  __syncthreads();
-  float l = 0.0f;
-#pragma unroll
-  for (int w = 0; w < D / kWave; ++w) {
-    l += merge_red[1][w];
-  }
-  float v = 0.0f;
-  int   s = 0;
-  for (; s + 8 <= n_splits; s += 8) {
-    float x[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      x[u] = rec0[(size_t) (s + u) * (D + 2) + 2 + d];
+  float        m_run = -INFINITY, l_run = 0.0f, v_run = 0.0f;
+  for (int s0 = 0; s0 < n_splits; s0 += kMergeChunk) {
+    const int  left = n_splits - s0;  // >= 1
+    const bool mine = lane < kMergeChunk && lane < left;
+    float      m_s = -INFINITY, l_s = 0.0f;
+    if (mine) {
+      const float2 ml = *reinterpret_cast<const float2 *>(rec0 + (size_t) (s0 + lane) * (D + 2));
+      m_s = ml.x, l_s = ml.y;
     }
+    float x[kMergeChunk];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      v += x[u] * merge_f[s + u];
+    for (int u = 0; u < kMergeChunk; ++u) {
+      x[u] = u < left ? rec0[(size_t) (s0 + u) * (D + 2) + 2 + d] : 0.0f;
     }
+    const float m_new  = fmaxf(m_run, group_max<kWave>(m_s));
+    const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
+    const float keep   = fast_exp2(m_run - m_safe);  // 0 for the first chunk
+    const float f      = fast_exp2(m_s - m_safe);    // 0 in lanes without a split
+    l_run              = l_run * keep + group_sum<kWave>(l_s * f);
+    float v            = 0.0f;
+#pragma unroll
+    for (int u = 0; u < kMergeChunk; ++u) {
+      v += x[u] * __int_as_float(__builtin_amdgcn_readlane(__float_as_int(f), u));
+    }
+    v_run = v_run * keep + v;
+    m_run = m_new;
   }
-  for (; s < n_splits; ++s) {
-    v += rec0[(size_t) s * (D + 2) + 2 + d] * merge_f[s];
-  }
-  const float out = v * (1.0f / l);
+  const float out = v_run * (1.0f / l_run);
   if (QO_F32) {
     reinterpret_cast<float *>(o_ptr)[(size_t) head * D + d] = out;
   } else {
@@ -828,6 +832,25 @@ hipError_t launch_prefill(hipStream_t stream, void *o, const void *q, const void
   return hipGetLastError();
 }
 
+template <int D, int GH, bool QO_F32, int SPLIT, int THREADS>
+hipError_t launch_decode_pass(hipStream_t stream, dim3 grid, float *workspace, const void *q, const void *k, const void *v,
+                              const void *mask, int kv_len, int n_heads, int n_kv_heads, int h0, int n_splits) {
+  constexpr int    kSlots = (THREADS / kWave) * (kWave / (D / 8));
+  constexpr size_t kLds   = ((size_t) kSlots * GH * D + (size_t) kSlots * GH + (size_t) (THREADS / kWave) * GH) * sizeof(float);
+  static_assert(kLds <= 160 * 1024, "LDS of one compute unit");
+  auto *kernel = flash_attn_decode_kernel<D, GH, QO_F32, SPLIT, THREADS>;
+  if (kLds > 64 * 1024) {
+    static const hipError_t raised =
+      hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int) kLds);
+    if (raised != hipSuccess) {
+      return raised;
+    }
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(THREADS), kLds, stream, workspace, q, (const _Float16 *) k, (const _Float16 *) v,
+                     (const _Float16 *) mask, kv_len, n_heads, n_kv_heads, h0, n_splits);
+  return hipGetLastError();
+}
+
 template <int D, bool QO_F32>
 hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void *k, const void *v, const void *mask,
                          int kv_len, int n_heads, int n_kv_heads, float *workspace) {
@@ -839,20 +862,15 @@ hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void 
   const int  n_splits = (kv_len + split - 1) / split;
   const dim3 grid((unsigned) n_splits, (unsigned) n_kv_heads);
   for (int h0 = 0; h0 < group; h0 += kDecMaxGroup) {
-    const int gh = group - h0;
-#define HTPOPS_DECODE(GH)                                                                                          \
-  if (short_kv) {                                                                                                  \
-    hipLaunchKernelGGL((flash_attn_decode_kernel<D, GH, QO_F32, kDecSplitShort>), grid, dim3(kDecThreads), 0,      \
-                       stream, workspace, q, (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask,  \
-                       kv_len, n_heads, n_kv_heads, h0, n_splits);                                                 \
-  } else {                                                                                                         \
-    hipLaunchKernelGGL((flash_attn_decode_kernel<D, GH, QO_F32, kDecSplit>), grid, dim3(kDecThreads), 0, stream,   \
-                       workspace, q, (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, kv_len,  \
-                       n_heads, n_kv_heads, h0, n_splits);                                                         \
-  }
-    if (gh >= 8) {
-      HTPOPS_DECODE(8);
-    } else if (gh > 4) {
+    const int  gh = group - h0;
+    hipError_t e;
+#define HTPOPS_DECODE(GH)                                                                                              \
+  e = short_kv ? launch_decode_pass<D, GH, QO_F32, kDecSplitShort, kDecThreads>(stream, grid, workspace, q, k, v, mask, \
+                                                                               kv_len, n_heads, n_kv_heads, h0,        \
+                                                                               n_splits) :                             \
+                 launch_decode_pass<D, GH, QO_F32, kDecSplit, kDecThreads>(stream, grid, workspace, q, k, v, mask,  \
+                                                                              kv_len, n_heads, n_kv_heads, h0, n_splits)
+    if (gh > 4) {
       HTPOPS_DECODE(8);
     } else if (gh > 2) {
       HTPOPS_DECODE(4);
@@ -862,9 +880,12 @@ hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void 
       HTPOPS_DECODE(1);
     }
 #undef HTPOPS_DECODE
+    if (e != hipSuccess) {
+      return e;
+    }
   }
-  hipLaunchKernelGGL((flash_attn_decode_merge_kernel<D, QO_F32>), dim3((unsigned) n_heads), dim3(D),
-                     (size_t) n_splits * sizeof(float), stream, o, workspace, n_splits);
+  hipLaunchKernelGGL((flash_attn_decode_merge_kernel<D, QO_F32>), dim3((unsigned) n_heads), dim3(D), 0, stream, o,
+                     workspace, n_splits);
   return hipGetLastError();
 }
 
