@@ -894,6 +894,69 @@ def test_message_decode_chain_keeps_its_own_launch_when_it_must(ctx, oracle):
             ctx.release(h)
 
 
+@pytest.mark.parametrize("seed", range(60))
+def test_message_batching_equals_one_request_at_a_time(ctx, seed):
+    # Random programs over a small pool of buffers, so that requests read what earlier ones wrote, overwrite what earlier
+    # ones read, and write the same bytes twice: RMSNorm -> Q8_0 (op 13), Q8_0 quantization (op 14) and matmuls of 1, 2
+    # and 8 rows whose outputs feed later norms -- or land on Q8_0 rows that later matmuls read as they are (whatever
+    # those bytes mean as blocks: both walks must agree on every byte, NaNs included). The walk of ONE message (which
+    # shares launches where it may) must leave every buffer exactly as one message per request does, where nothing can
+    # share.
+    rng = wl.rng_for(79, seed)
+    k = n = (256, 512, 1024)[seed % 3]        # outputs are as long as inputs, so that they can be normalized again
+    rows = 8
+    wt = wl.GGML_TYPE_Q4_0 if seed % 2 == 0 else wl.GGML_TYPE_Q8_0
+    op_mm = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
+    q_row = k // 32 * 34
+    f_init = [wl.make_activations(rng, rows, k) for _ in range(4)]
+    q_init = [np.zeros(rows * q_row, np.uint8) for _ in range(2)]   # (zero scales and values: finite whatever reads them)
+    ws = [wl.make_weights(rng, n, k, wt) for _ in range(4)]
+    g = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    hf, hq = [ctx.upload(x) for x in f_init], [ctx.upload(x) for x in q_init]
+    hw, hg = [ctx.upload(w) for w in ws], ctx.upload(g)
+    try:
+        reqs = []
+        for _ in range(16):
+            kind = rng.integers(0, 10)
+            m = int(rng.choice([1, 1, 1, 1, 2, 8]))
+            row = int(rng.integers(0, rows - m + 1))          # requests work on rows row .. row + m - 1 of their buffers
+            f, q = int(rng.integers(0, len(hf))), int(rng.integers(0, len(hq)))
+            if kind < 3:
+                weight = (hg, 0) if rng.integers(0, 2) else (-1, 0)
+                reqs.append((api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
+                    api.HTP_OPS_RMS_NORM_QUANTIZE_Q8_0,
+                    api.rms_norm_ex_params((hq[q], row * q_row), (hf[f], row * k * 4), weight, k, m, 1e-6))))
+            elif kind < 4:
+                reqs.append((api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
+                    api.HTP_OPS_QUANTIZE_Q8_0, api.rms_norm_params((hq[q], row * q_row), (hf[f], row * k * 4), k, m))))
+            else:
+                # the output rows start wherever they fit: m x n floats somewhere in the fp32 buffer
+                out_row = int(rng.integers(0, rows - m + 1))
+                if m <= 2 and rng.integers(0, 5) < 2:    # m x n floats over the Q8_0 rows of another (or the same) buffer
+                    ho, out_off = hq[int(rng.integers(0, len(hq)))], 4 * int(rng.integers(0, (rows * q_row - m * n * 4) // 4 + 1))
+                else:
+                    ho, out_off = hf[f], out_row * n * 4
+                reqs.append(_mm(op_mm, ho, hq[q], hw[int(rng.integers(0, len(hw)))], m, k, n,
+                                out_off=out_off, act_off=row * q_row))
+
+        def run(messages):
+            for h, x in zip(hf + hq, f_init + q_init):
+                ctx.write(h, x)
+            for msg in messages:
+                assert ctx.process_message(msg) == 0
+                assert all(st == 0 for st in api.message_request_states(msg)), ctx.last_error()
+            return [ctx.read(h, np.uint8, ctx.size(h)) for h in hf + hq]
+
+        one_by_one = run([api.build_message([r]) for r in reqs])
+        together = run([api.build_message(reqs)])
+        assert ctx.last_message_submissions() <= len(reqs)
+        for i, (a, b) in enumerate(zip(one_by_one, together)):
+            assert np.array_equal(a, b), "buffer %d differs between the two walks" % i
+    finally:
+        for h in hf + hq + hw + [hg]:
+            ctx.release(h)
+
+
 def test_message_keeps_dependent_gemvs_in_order(ctx, oracle):
     # Requests with a data dependency must not share a launch. (1) read-after-write: request 1's fp32 output bytes are
     # request 2's Q8_0 activation row (unit scales and small integers make those bytes finite Q8_0 blocks);
