@@ -246,10 +246,27 @@ __global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(
       for (int r = 0; r < 16; ++r) {
         st[kt][r] = -m_ref;
       }
+    }
+    // the two key tiles advance side by side (independent accumulators), and the fragments of step s + 1 are
+    // requested before the products of step s
+    {
+      v8h kf[2][2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+        kf[0][kt] = *reinterpret_cast<const v8h *>(&sm.k[32 * kt + col][8 * half]);
+      }
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
-        const v8h kf = *reinterpret_cast<const v8h *>(&sm.k[32 * kt + col][16 * s + 8 * half]);
-        st[kt]       = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], st[kt], 0, 0, 0);
+        if (s + 1 < KSTEPS) {
+#pragma unroll
+          for (int kt = 0; kt < 2; ++kt) {
+            kf[(s + 1) & 1][kt] = *reinterpret_cast<const v8h *>(&sm.k[32 * kt + col][16 * (s + 1) + 8 * half]);
+          }
+        }
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+          st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s & 1][kt], qf[s], st[kt], 0, 0, 0);
+        }
       }
     }
 
@@ -312,17 +329,17 @@ __global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(
       l_run *= alpha;
       m_run = move ? m_ref + mx : m_run;
     }
-    float psum = 0.0f;
+    float psum[4] = { 0.0f, 0.0f, 0.0f, 0.0f };  // (four chains: an addition waits for the one before it in its chain)
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float p = fast_exp2(st[kt][r]);
         st[kt][r]     = p;
-        psum += p;
+        psum[r & 3] += p;
       }
     }
-    l_run += psum;
+    l_run += (psum[0] + psum[1]) + (psum[2] + psum[3]);
 
     // ---- O^T += V^T P^T ----
     // MFMA (kt, u) covers keys 32 kt + 16 u + {4 half + 0..3, 8 + 4 half + 0..3}: exactly registers 8 u .. 8 u + 7
