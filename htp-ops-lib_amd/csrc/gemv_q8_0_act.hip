@@ -332,7 +332,7 @@ struct GemvMember {
   int             pairs;   // block pairs per row (k / 64)
   int             block0;  // first workgroup of this member
   int             shape;   // kShape* below: lanes per row and pairs per lane
-  int             r;       // row sets per wave (1 or 2)
+  int             r;       // row sets per wave (1 or 2; 4 only in the launch that makes its activation row)
 };
 
 struct GemvMembers {
@@ -591,6 +591,12 @@ __device__ __forceinline__ void gemv_members_body(int b1, int b2, int b3, int b4
   const int     mi  = bid >= b7 ? 7 : bid >= b6 ? 6 : bid >= b5 ? 5 : bid >= b4 ? 4 : bid >= b3 ? 3 : bid >= b2 ? 2 : bid >= b1 ? 1 : 0;
   const GemvMember &mem = grp.m[mi];
   const int         wg  = (int) blockIdx.x - mem.block0;
+  if constexpr (FUSED) {
+    if (mem.r == 4) {  // (rows of 33..64 pairs only: see the launcher)
+      gemv_row_sets<WT, 64, 1, 4, 1, W, FUSED>(mem, wg, gemv_lds, norm);
+      return;
+    }
+  }
   const int         sel = mem.shape * 2 + (mem.r - 1);
   switch (sel) {
     case kShapeG16 * 2 + 0: gemv_row_sets<WT, 16, 1, 1, 1, W, FUSED>(mem, wg, gemv_lds, norm); break;
@@ -661,6 +667,9 @@ hipError_t launch_gemv_members(hipStream_t stream, GemvMembers &grp, const GemvN
     }
     mem.shape = p <= 16 ? kShapeG16 : p <= 32 ? kShapeG32 : p <= 64 ? kShapeG64 : p <= 128 ? kShapeG64x2 : kShapeG64x2S2;
     mem.r     = (p <= 64 && (total_short_rows >= 16384 || norm)) ? 2 : 1;
+    if (norm && p > 32 && p <= 64 && total_short_rows > kFusedNormMaxBlocks * 16) {
+      mem.r = 4;  // gate and up of a 7B layer: 32 rows per workgroup halve the number of times the row is made
+    }
     max_pairs = p > max_pairs ? p : max_pairs;
     any_long  = any_long || p > 64;
   }
@@ -669,7 +678,8 @@ hipError_t launch_gemv_members(hipStream_t stream, GemvMembers &grp, const GemvN
   const int blocks = place(threads, true);
   // Measured on MI355X with Q4_0 weights of k = 4096: making the row costs every workgroup about as much as 8 KB of its
   // weight stream, which beats a launch of its own (3.5-4 us behind another) up to about a thousand workgroups:
-  // n = 4096: 5.2 us against 7.0 us, 3 x 4096: 9.0 / 10.4, 2 x 11008: 16.4 / 14.5. Longer rows cost in proportion.
+  // n = 4096: 5.2 us against 7.0 us, 3 x 4096: 9.0 / 10.4, 2 x 11008: 16.4 / 14.5 with 16 rows per workgroup, 14.2 with
+  // 32 (and 16.0 with 64: too few workgroups). Longer rows cost in proportion.
   if (norm && (any_long || blocks > kFusedNormMaxBlocks)) {
     return hipErrorNotSupported;
   }

@@ -797,18 +797,18 @@ def _norm_q(hq, hx, hg, k, rows, eps):
 
 
 @pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
-@pytest.mark.parametrize("k,wide", [(64, False), (1024, False), (1536, False), (4096, False), (4096, True), (8192, False),
-                                    (11008, False)])
+@pytest.mark.parametrize("k,wide", [(64, 0), (1024, 0), (1536, 0), (4096, 0), (4096, 2), (4096, 4), (8192, 0), (11008, 0)])
 @pytest.mark.parametrize("with_weight", [True, False])
 def test_message_decode_chain_in_one_launch(ctx, oracle, wt, k, wide, with_weight):
     # RMSNorm -> Q8_0 of one row followed by the one-row matmuls that read it (q/k/v or gate/up of a decoder layer) is one
     # launch: every workgroup makes the row for itself. The Q8_0 row written must be the bytes of the op run alone, and
-    # every product the bits of its own launch over that row. Rows longer than 4096 and launches of more than about a
-    # thousand workgroups (`wide`: gate and up of a 7B layer) keep the two launches, where that is faster.
-    rng = wl.rng_for(77, wt * 100000 + k * 4 + int(with_weight) * 2 + int(wide))
+    # every product the bits of its own launch over that row (`wide` = 2: gate and up of a 7B layer, 32 weight rows per
+    # workgroup instead of 16). Rows longer than 4096 and launches that would still need more than about a thousand
+    # workgroups (`wide` = 4 matrices of 11008 rows) keep the two launches, where that is faster.
+    rng = wl.rng_for(77, wt * 100000 + k * 8 + int(with_weight) * 4 + wide // 2)
     op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
-    ns = [11008, 11008] if wide else [256, 1000, 48]
-    launches = 1 if k <= 4096 and not wide else 2
+    ns = [11008] * wide if wide else [256, 1000, 48]
+    launches = 1 if k <= 4096 and wide < 4 else 2
     x = wl.make_activations(rng, 1, k)
     g = (1.0 + 0.1 * rng.standard_normal(k)).astype(np.float32) if with_weight else None
     ws = [wl.make_weights(rng, n, k, wt) for n in ns]
