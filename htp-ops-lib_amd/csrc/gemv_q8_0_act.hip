@@ -344,12 +344,14 @@ struct GemvMembers {
 // fp32 row (the decode chain norm -> quantize -> projections as one launch). Each workgroup makes that image for itself
 // in LDS -- the first 256 threads repeat the fused RMSNorm + Q8_0 kernel's arithmetic thread for thread, so the bytes
 // are the ones that kernel writes -- and the first workgroup of the launch also writes it to `q_out`, where the
-// message asked for it.
+// message asked for it. Without `normalize` the row is quantized as it is: the bytes of the Q8_0 quantizer (the same
+// block arithmetic), for projections behind a plain quantization (attention output -> Q8_0 -> o projection).
 struct GemvNorm {
   const float *src;     // fp32 [k]
   const float *weight;  // fp32 [k] or nullptr
   float        eps;
   uint8_t     *q_out;   // block_q8_0 [k / 32]
+  int          normalize;
 };
 
 // lanes per row x pairs per lane x waves per row
@@ -468,7 +470,7 @@ __device__ __forceinline__ void gemv_row_sets(const GemvMember &mem, int wg, uin
     asm volatile("" ::: "memory");
     const float sum   = ((red[0] + red[1]) + red[2]) + red[3];
     const float mean  = sum / (float) (nb * kQK);
-    const float scale = 1.0f / sqrtf(mean + norm.eps);
+    const float scale = norm.normalize ? 1.0f / sqrtf(mean + norm.eps) : 1.0f;  // (x * 1.0f is x)
     if (threadIdx.x < 256) {
 #pragma unroll
       for (int b = 0; b < BPT; ++b) {
@@ -944,11 +946,11 @@ hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *cons
 
 // The decode chain as one launch: every member's activation row is RMSNorm(src [* norm_weight]) quantized to Q8_0,
 // made by each workgroup for itself and also written to `q_out` (k / 32 blocks), bit for bit what
-// launch_rms_norm_quantize_q8_0 writes. k % 64 == 0, k <= 4096, 16-byte aligned src / norm_weight and few enough
+// launch_rms_norm_quantize_q8_0 writes (`normalize` false: src quantized as it is, what launch_quantize_q8_0 writes). k % 64 == 0, k <= 4096, 16-byte aligned src / norm_weight and few enough
 // weight rows that it pays (see launch_gemv_members), else hipErrorNotSupported and nothing is launched.
 hipError_t launch_gemv_group_rms_norm_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *const *weights,
                                                const int *ns, int k, WeightType wt, const float *src,
-                                               const float *norm_weight, float eps, void *q_out) {
+                                               const float *norm_weight, float eps, void *q_out, bool normalize) {
   const int nblk = k / kQK;
   if (count < 1 || count > kGemvGroupMax || k % (2 * kQK) != 0 || nblk / 2 > kSharedActMaxPairs ||
       (reinterpret_cast<uintptr_t>(src) & 15) != 0 || (reinterpret_cast<uintptr_t>(norm_weight) & 15) != 0 ||
@@ -964,7 +966,7 @@ hipError_t launch_gemv_group_rms_norm_q8_0_act(hipStream_t stream, int count, fl
     grp.m[i].w = static_cast<const uint32_t *>(weights[i]), grp.m[i].act = static_cast<const uint32_t *>(q_out);
     grp.m[i].out = outs[i], grp.m[i].n = ns[i], grp.m[i].pairs = nblk / 2;
   }
-  const GemvNorm norm = { src, norm_weight, eps, static_cast<uint8_t *>(q_out) };
+  const GemvNorm norm = { src, normalize ? norm_weight : nullptr, eps, static_cast<uint8_t *>(q_out), normalize ? 1 : 0 };
   return wt == kQ4_0 ? launch_gemv_members<kQ4_0>(stream, grp, &norm) : launch_gemv_members<kQ8_0>(stream, grp, &norm);
 }
 

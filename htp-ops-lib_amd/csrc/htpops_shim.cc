@@ -1160,10 +1160,12 @@ struct GemvBatch {
   const void           *act[htpops::kGemvGroupMax];
   int                   n[htpops::kGemvGroupMax];
   int                   k[htpops::kGemvGroupMax];
-  // A one-row RMSNorm + Q8_0 request that waits for the matmuls that read its row (the decode chain): when only such
-  // matmuls follow, one launch makes the row and multiplies by it; anything else runs the request first, as it came.
+  // A one-row RMSNorm + Q8_0 (or plain Q8_0 quantization) request that waits for the matmuls that read its row (the
+  // decode chain): when only such matmuls follow, one launch makes the row and multiplies by it; anything else runs
+  // the request first, as it came.
   struct {
     bool                  waiting = false;
+    bool                  normalize = true;  // false: the request is a plain quantization
     struct RequestHeader *hdr     = nullptr;
     void                 *dst     = nullptr;
     const float          *src = nullptr, *weight = nullptr;
@@ -1248,7 +1250,8 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
       }
       const hipError_t e = htpops::launch_gemv_group_rms_norm_q8_0_act(ctx->stream, b.count, b.out, b.w, b.n, b.norm.ne0,
                                                                        (htpops::WeightType) b.wt, b.norm.src,
-                                                                       b.norm.weight, b.norm.eps, b.norm.dst);
+                                                                       b.norm.weight, b.norm.eps, b.norm.dst,
+                                                                       b.norm.normalize);
       if (e != hipErrorNotSupported) {
         ++ctx->message_submissions;
         if (e != hipSuccess) {
@@ -1265,7 +1268,9 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
     }
     b.fused = false;
     ++ctx->message_submissions;
-    b.norm.hdr->state = op_rms_norm_quantize(ctx, b.norm.dst, b.norm.src, b.norm.weight, b.norm.eps, b.norm.ne0, 1);
+    b.norm.hdr->state = b.norm.normalize ?
+                          op_rms_norm_quantize(ctx, b.norm.dst, b.norm.src, b.norm.weight, b.norm.eps, b.norm.ne0, 1) :
+                          op_quantize(ctx, b.norm.dst, b.norm.src, b.norm.ne0, 1);
   }
   if (b.count == 0) {
     return;
@@ -1357,25 +1362,29 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
   b.count = 0;
 }
 
-// true: the one-row RMSNorm + Q8_0 request now waits in the (empty) batch for the matmuls behind it; false: run it now
+// true: the one-row RMSNorm + Q8_0 (op 13) or Q8_0 quantization (op 14) request now waits in the (empty) batch for the
+// matmuls behind it; false: run it now
 bool try_defer_norm(htpops_context *ctx, const struct OpComputeRequest *req, struct RequestHeader *hdr, GemvBatch &b) {
-  const auto *p = reinterpret_cast<const RmsNormExParams *>(req->payload);
-  if (!ctx->has_device || p->ne1 != 1 || p->ne0 <= 0 || p->ne0 % 64 != 0 || p->ne0 > 4096) {
+  const bool   normalize = req->op == HTP_OPS_RMS_NORM_QUANTIZE_Q8_0;
+  const auto  *p  = reinterpret_cast<const RmsNormExParams *>(req->payload);
+  const auto  *pq = reinterpret_cast<const RmsNormF32Params *>(req->payload);  // (dst, src, ne0, ne1: the same head)
+  const int    ne0 = normalize ? p->ne0 : pq->ne0, ne1 = normalize ? p->ne1 : pq->ne1;
+  if (!ctx->has_device || ne1 != 1 || ne0 <= 0 || ne0 % 64 != 0 || ne0 > 4096) {
     return false;
   }
-  const size_t src_bytes = (size_t) p->ne0 * 4, q_bytes = q8_0_bytes(1, (size_t) p->ne0);
+  const size_t src_bytes = (size_t) ne0 * 4, q_bytes = q8_0_bytes(1, (size_t) ne0);
   const float *w = nullptr;
-  if (p->weight.fd >= 0 && !(w = (const float *) resolve(ctx, p->weight, src_bytes))) {
+  if (normalize && p->weight.fd >= 0 && !(w = (const float *) resolve(ctx, p->weight, src_bytes))) {
     return false;
   }
-  const float *src = (const float *) resolve(ctx, p->src, src_bytes);
-  void        *dst = resolve(ctx, p->dst, q_bytes);
+  const float *src = (const float *) resolve(ctx, normalize ? p->src : pq->src, src_bytes);
+  void        *dst = resolve(ctx, normalize ? p->dst : pq->dst, q_bytes);
   if (!src || !dst || !aligned(dst, 4) || !aligned(src, 16) || (w && !aligned(w, 16)) ||
       ranges_overlap(dst, q_bytes, src, src_bytes) || (w && ranges_overlap(dst, q_bytes, w, src_bytes))) {
     return false;  // the ordinary path reports what is wrong; a row quantized in place keeps its own launch
   }
-  b.norm.waiting = true, b.norm.hdr = hdr, b.norm.dst = dst, b.norm.src = src, b.norm.weight = w, b.norm.eps = p->eps;
-  b.norm.ne0 = p->ne0;
+  b.norm.waiting = true, b.norm.hdr = hdr, b.norm.dst = dst, b.norm.src = src, b.norm.weight = w;
+  b.norm.eps = normalize ? p->eps : 0.0f, b.norm.ne0 = ne0, b.norm.normalize = normalize;
   hdr->state = HTPOPS_OK;
   return true;
 }
@@ -1498,8 +1507,10 @@ int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_b
           const bool  matmul_payload =
             size >= sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest) + sizeof(MatMulParams);
           const bool  norm_payload =
-            req->op == HTP_OPS_RMS_NORM_QUANTIZE_Q8_0 &&
-            size >= sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest) + sizeof(RmsNormExParams);
+            (req->op == HTP_OPS_RMS_NORM_QUANTIZE_Q8_0 &&
+             size >= sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest) + sizeof(RmsNormExParams)) ||
+            (req->op == HTP_OPS_QUANTIZE_Q8_0 &&
+             size >= sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest) + sizeof(RmsNormF32Params));
           if (norm_payload) {
             flush_batch(ctx, batch);
           }

@@ -33,12 +33,12 @@ hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *cons
                                       const void *const *weights, const int *ns, const int *ks, WeightType wt);
 // The same launch with the activation row made inside it: RMSNorm(src [* norm_weight], eps) quantized to Q8_0 is what
 // every member multiplies by (all of one k), and it is also written to `q_out`, bit for bit what
-// launch_rms_norm_quantize_q8_0 writes. hipErrorNotSupported (nothing launched; the caller runs the two steps) unless
+// launch_rms_norm_quantize_q8_0 writes (`normalize` false: src quantized as it is, the bytes of launch_quantize_q8_0). hipErrorNotSupported (nothing launched; the caller runs the two steps) unless
 // k % 64 == 0, k <= 4096, src / norm_weight are 16-byte aligned and the rows are few enough for this to pay: every
 // workgroup makes the row for itself, which beats a launch of its own up to about a thousand workgroups of 16 rows.
 hipError_t launch_gemv_group_rms_norm_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *const *weights,
                                                const int *ns, int k, WeightType wt, const float *src,
-                                               const float *norm_weight, float eps, void *q_out);
+                                               const float *norm_weight, float eps, void *q_out, bool normalize);
 // 2 <= m <= 4 activation rows against several weight matrices in one launch: the decode kernel's stream over the
 // weights with the rows held in registers; member i reads the rows acts[i] of length ks[i] (k % 64 == 0, k <= 12288,
 // 4-byte aligned buffers; else hipErrorNotSupported)

@@ -838,6 +838,39 @@ def test_message_decode_chain_in_one_launch(ctx, oracle, wt, k, wide, with_weigh
             ctx.release(h)
 
 
+@pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
+@pytest.mark.parametrize("k", [128, 1536, 4096, 8192])
+def test_message_quantize_then_projections_in_one_launch(ctx, oracle, wt, k):
+    # A one-row Q8_0 quantization (op 14: the attention output on its way to the o projection) followed by one-row
+    # matmuls over the row it writes runs inside their launch like the RMSNorm + Q8_0 request does: the row written is the
+    # quantizer's, bit for bit (which is the oracle's), and so are the products. Rows longer than 4096 keep two launches.
+    rng = wl.rng_for(80, wt * 100000 + k)
+    op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
+    ns = [4096, 48]
+    x = wl.make_activations(rng, 1, k)
+    ws = [wl.make_weights(rng, n, k, wt) for n in ns]
+    hx, hq = ctx.upload(x), ctx.alloc(k // 32 * 34)
+    hws, hos = [ctx.upload(w) for w in ws], [ctx.alloc(n * 4) for n in ns]
+    try:
+        want_q = oracle.quantize_q8_0(x)
+        quant = (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(api.HTP_OPS_QUANTIZE_Q8_0, api.rms_norm_params((hq, 0), (hx, 0), k, 1)))
+        msg = api.build_message([quant] + [_mm(op, ho, hq, hw, 1, k, n) for ho, hw, n in zip(hos, hws, ns)])
+        for _ in range(2):
+            ctx.write(hq, np.full(k // 32 * 34, 0xA5, np.uint8))
+            for ho, n in zip(hos, ns):
+                ctx.write(ho, np.full(n, np.nan, np.float32))
+            assert ctx.process_message(msg) == 0
+            assert api.message_request_states(msg) == [0] * (1 + len(ns)), ctx.last_error()
+            assert ctx.last_message_submissions() == (1 if k <= 4096 else 2)
+            assert np.array_equal(ctx.read(hq, np.uint8, k // 32 * 34), want_q[0]), "the row differs from the quantizer's"
+            for ho, w, n in zip(hos, ws, ns):
+                got = ctx.read(ho, np.float32, n)
+                assert np.array_equal(got, ctx.run_mat_mul(want_q, w, 1, k, n, wt)[0]), "a request differs from its own launch"
+    finally:
+        for h in [hx, hq] + hws + hos:
+            ctx.release(h)
+
+
 def test_message_decode_chain_keeps_its_own_launch_when_it_must(ctx, oracle):
     # The RMSNorm -> Q8_0 request runs by itself, in order, when what follows cannot share its launch: a matmul over another
     # row, a matmul whose output lands on the request's input, several rows, the end of the message; and matmuls that
@@ -932,10 +965,13 @@ def test_message_batching_equals_one_request_at_a_time(ctx, seed):
             else:
                 # the output rows start wherever they fit: m x n floats somewhere in the fp32 buffer
                 out_row = int(rng.integers(0, rows - m + 1))
+                ho, out_off = hf[f], out_row * n * 4
                 if m <= 2 and rng.integers(0, 5) < 2:    # m x n floats over the Q8_0 rows of another (or the same) buffer
-                    ho, out_off = hq[int(rng.integers(0, len(hq)))], 4 * int(rng.integers(0, (rows * q_row - m * n * 4) // 4 + 1))
-                else:
-                    ho, out_off = hf[f], out_row * n * 4
+                    qo, off = int(rng.integers(0, len(hq))), 4 * int(rng.integers(0, (rows * q_row - m * n * 4) // 4 + 1))
+                    # (not over the rows this very request reads: a request that overwrites its own input while its
+                    # workgroups still read it has no defined result)
+                    if qo != q or off + m * n * 4 <= row * q_row or off >= (row + m) * q_row:
+                        ho, out_off = hq[qo], off
                 reqs.append(_mm(op_mm, ho, hq[q], hw[int(rng.integers(0, len(hw)))], m, k, n,
                                 out_off=out_off, act_off=row * q_row))
 
