@@ -21,6 +21,8 @@ The same run also measures, and reports inside the JSON line:
                 and replayed (reported beside `value`, which is the ordinary message walk)
   q8_0_block    the Qwen2-1.5B-like Q8_0 block of config 4 at m = 1 and m = 128
   decode_chain_us   config 0: RMSNorm -> Q8_0 -> GEMV (4096 x 4096) for one token, submitted as one message
+  decoder_layer_one_token   the 12 requests of a Llama-7B-like layer for one token (norms, projections, attention over
+                4096 cached keys, quantizations) as one message
   elementwise   RMSNorm, the Q8_0 quantizer and the fused RMSNorm + quantizer over m x 4096 at m = 1 / 128 / 512
   attention     config 3: decode (1 x 4096, 1 x 16384) and causal prefill (2048 x 2048), 32 query / 8 KV heads of 128, fp16
   cpu_baseline  the scalar C oracle (a port of the same arithmetic) on the host cores: the headline layer, and under
@@ -486,6 +488,84 @@ def main():
         for h in [hq, ho] + hks + hvs:
             ctx.release(h)
 
+    # ------------------------------------------------------------------ a whole decoder layer for one token
+    # Every op of a Llama-7B-like layer that this backend has, in the order a decoder issues them, as ONE message:
+    # RMSNorm+Q8_0 -> q, k, v -> attention over 4096 cached keys (32 query / 8 KV heads) -> Q8_0 -> o -> RMSNorm+Q8_0 ->
+    # gate, up -> Q8_0 -> down. (The residual additions, RoPE and SiLU x up belong to the caller; k and v here are
+    # 4096 wide like the layer's weights, the cache is read with 8 KV heads.) The norms and the one-row quantizations
+    # run inside the launches of the projections behind them where that pays.
+    rng6 = wl.rng_for(6, 0)
+    kv6 = 4096
+    _, kk6, vv6 = wl.make_attention_inputs(rng6, 1, kv6, nh, nkv, hd)
+    hx6, hg6 = ctx.upload(wl.make_activations(rng6, 1, 4096)), ctx.upload(np.ones(4096, np.float32))
+    hh6 = ctx.upload(wl.make_activations(rng6, 1, 11008))
+    hq6 = {name: ctx.alloc(k // 32 * 34) for name, k in (("a", 4096), ("o", 4096), ("b", 4096), ("d", 11008))}
+    hattn6 = ctx.alloc(4096 * 4)
+    n_caches = 8
+    hk6, hv6 = [ctx.upload(kk6) for _ in range(n_caches)], [ctx.upload(vv6) for _ in range(n_caches)]
+    IDX = {name: i for i, (name, _, _) in enumerate(shapes)}
+
+    def mm6(layer, name, act):
+        _, n, k = shapes[IDX[name]]
+        return (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
+            api.HTP_OPS_MAT_MUL_Q4_0_Q8_0, api.mat_mul_params((h_out[1][IDX[name]], 0), (act, 0), (layers[layer][IDX[name]], 0), 1, k, n)))
+
+    def op6(op, payload):
+        return (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(op, payload))
+
+    def decoder_layer_requests(layer):
+        return [
+            op6(api.HTP_OPS_RMS_NORM_QUANTIZE_Q8_0, api.rms_norm_ex_params((hq6["a"], 0), (hx6, 0), (hg6, 0), 4096, 1, 1e-6)),
+            mm6(layer, "q", hq6["a"]), mm6(layer, "k", hq6["a"]), mm6(layer, "v", hq6["a"]),
+            op6(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16,
+                api.flash_attn_params((hattn6, 0), (h_out[1][IDX["q"]], 0), (hk6[layer % n_caches], 0), (hv6[layer % n_caches], 0),
+                                      (-1, 0), 1, kv6, nh, nkv, hd)),
+            op6(api.HTP_OPS_QUANTIZE_Q8_0, api.rms_norm_params((hq6["o"], 0), (hattn6, 0), 4096, 1)),
+            mm6(layer, "o", hq6["o"]),
+            op6(api.HTP_OPS_RMS_NORM_QUANTIZE_Q8_0, api.rms_norm_ex_params((hq6["b"], 0), (h_out[1][IDX["o"]], 0), (hg6, 0), 4096, 1, 1e-6)),
+            mm6(layer, "gate", hq6["b"]), mm6(layer, "up", hq6["b"]),
+            op6(api.HTP_OPS_QUANTIZE_Q8_0, api.rms_norm_params((hq6["d"], 0), (hh6, 0), 11008, 1)),
+            mm6(layer, "down", hq6["d"])]
+
+    msgs6 = [api.build_message(decoder_layer_requests(l)) for l in range(LAYERS)]
+    assert ctx.process_message(msgs6[0]) == 0
+    check_states(msgs6[0])
+    launches6 = ctx.last_message_submissions() + 1   # (the attention request is two launches: splits, then their merge)
+    handles6 = [ctx.message_handle(msg) for msg in msgs6]
+    for s_ in range(2 * LAYERS):
+        ctx.enqueue_message_handle(handles6[s_ % LAYERS])
+    ctx.synchronize()
+    ctx.timer_start()
+    for s_ in range(200):
+        ctx.enqueue_message_handle(handles6[s_ % LAYERS])
+    layer6_us = ctx.timer_stop_ms() * 1e3 / 200
+    ctx.synchronize()
+    for msg in msgs6:
+        ctx.finish_message(msg)
+        check_states(msg)
+    # the same requests one message each: nothing shares a launch (12 requests, 13 launches)
+    singles6 = [[api.build_message([r]) for r in decoder_layer_requests(l)] for l in range(LAYERS)]
+    single_handles6 = [[ctx.message_handle(msg) for msg in grp] for grp in singles6]
+    for grp in single_handles6:
+        for h in grp:
+            ctx.enqueue_message_handle(h)
+    ctx.synchronize()
+    ctx.timer_start()
+    for s_ in range(100):
+        for h in single_handles6[s_ % LAYERS]:
+            ctx.enqueue_message_handle(h)
+    layer6_single_us = ctx.timer_stop_ms() * 1e3 / 100
+    ctx.synchronize()
+    for grp in singles6:
+        for msg in grp:
+            ctx.finish_message(msg)
+            check_states(msg)
+    layer6_bytes = layer_bytes[1] + 2 * kv6 * nkv * hd * 2
+    log("decoder layer for one token (12 requests, %d launches): %.2f us, %.0f GB/s of weights and KV cache; one message per request: %.2f us" % (
+        launches6, layer6_us, layer6_bytes / layer6_us / 1e3, layer6_single_us))
+    for h in [hx6, hg6, hh6, hattn6] + list(hq6.values()) + hk6 + hv6:
+        ctx.release(h)
+
     # ------------------------------------------------------------------ device ceilings
     read_layer_us = ctx.measure_read_us(layer_bytes[1] // 16 * 16, LAYERS, 10)
     read_down_us = ctx.measure_read_us(wl.matmul_algorithmic_bytes(1, 11008, 4096, Q4) // 16 * 16, 24, 10)
@@ -608,6 +688,9 @@ def main():
         "recorded_message_us_per_step": None if args.skip_recorded else
         {"m1": round(rec_step[1] * 1e3, 2), "m8": round(rec_step[8] * 1e3, 2)},
         "decode_chain_us": round(chain_us, 2),
+        "decoder_layer_one_token": {"us": round(layer6_us, 2), "requests": 12, "launches": launches6, "kv_len": kv6,
+                                    "bytes": layer6_bytes, "GBps": round(layer6_bytes / layer6_us / 1e3, 1),
+                                    "us_one_message_per_request": round(layer6_single_us, 2)},
         "elementwise": elementwise,
         "attention": attention,
         "q8_0_block": [q8_block[1], q8_block[128]],
