@@ -304,8 +304,33 @@ def main():
         first_us = ctx.timer_stop_ms() * 1e3
         ctx.release(h_fresh)
         hw = layers[0][4] if (n, k) == (11008, 4096) else layers[0][6]
-        us = time_single(n, k, m, Q4, [hw] * 8, ha, ho, 5, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)  # 8 launches per message share the re-tiled activations
+        us = time_single(n, k, m, Q4, [hw] * 8, ha, ho, 10, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)  # 8 launches per message share the re-tiled activations
         us_alone = time_single(n, k, m, Q4, [hw], ha, ho, 20, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)  # re-tiling + one launch
+        # independent matmuls over the same rows (q/k/v, gate/up of a prefill chunk: distinct weights, distinct outputs)
+        # share a launch: three and eight per message
+        idx = 4 if (n, k) == (11008, 4096) else 6
+        hos_g = [ho] + [ctx.alloc(m * n * 4) for _ in range(7)]
+        grouped = {}
+        for g_n in (3, 8):
+            reqs_g = [(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
+                api.HTP_OPS_MAT_MUL_Q4_0_Q8_0, api.mat_mul_params((hos_g[i], 0), (ha, 0), (layers[i][idx], 0), m, k, n)))
+                for i in range(g_n)]
+            msg_g = api.build_message(reqs_g)
+            for _ in range(3):
+                ctx.enqueue_message(msg_g)
+            ctx.synchronize()
+            ctx.timer_start()
+            for _ in range(80 // g_n):   # (about 80 matmuls back to back in every variant: the clock settles with the load)
+                ctx.enqueue_message(msg_g)
+            grouped[g_n] = ctx.timer_stop_ms() * 1e3 / (80 // g_n * g_n)
+            ctx.finish_message(msg_g)
+            check_states(msg_g)
+            launches_g = ctx.last_message_submissions()
+            assert launches_g == 1, "independent many-row matmuls over the same rows are expected to share a launch"
+            assert np.array_equal(ctx.read(hos_g[g_n - 1], np.float32, m * n),
+                                  ctx.read(ho, np.float32, m * n)), "a grouped matmul differs from the first of its group"
+        for h in hos_g[1:]:
+            ctx.release(h)
         got = ctx.read(ho, np.float32, m * n).reshape(m, n)
         rows_m = [0, 257, 511]
         cols = np.unique(np.linspace(0, n - 1, 64).astype(int))
@@ -314,13 +339,16 @@ def main():
         tops = 2.0 * m * n * k / us / 1e6
         prefill.append({"m": m, "n": n, "k": k, "us": round(us, 2), "tera_ops": round(tops, 1),
                         "frac_of_int8_nominal": round(tops / INT8_PEAK_TOPS, 4),
+                        "us_per_matmul_3_in_one_message": round(grouped[3], 2),
+                        "us_per_matmul_8_in_one_message": round(grouped[8], 2),
+                        "tera_ops_8_in_one_message": round(2.0 * m * n * k / grouped[8] / 1e6, 1),
                         "us_with_activation_retiling": round(us_alone, 2),
                         "activation_retiling_us": round(max(0.0, us_alone - us) * 8 / 7, 2),
                         "first_use_us_incl_weight_conversion": round(first_us, 1),
                         "converted_weight_copy_bytes": n * k,
                         "algorithmic_bytes": wl.matmul_algorithmic_bytes(m, k, n, Q4)})
-        log("prefill GEMM m=512 n=%d k=%d: %.1f us  %.1f Tops (%.1f%% of 5 Pop/s); alone with re-tiling %.1f us; first use %.0f us" % (
-            n, k, us, tops, tops / 50, us_alone, first_us))
+        log("prefill GEMM m=512 n=%d k=%d: %.1f us  %.1f Tops (%.1f%% of 5 Pop/s); 3 / 8 independent ones in a message: %.1f / %.1f us each; alone with re-tiling %.1f us; first use %.0f us" % (
+            n, k, us, tops, tops / 50, grouped[3], grouped[8], us_alone, first_us))
         ctx.release(ha), ctx.release(ho)
 
     # ------------------------------------------------------------------ decode chain (config 0)

@@ -212,12 +212,25 @@ struct Shape {
   static constexpr int kPerWave  = (kDma + kWaves - 1) / kWaves;      // transfers of the waves that issue the most
 };
 
+// The matmuls of one launch: the same activation rows against several weight matrices (q/k/v, gate/up of a prefill
+// chunk). blockIdx.y is the member; workgroups past a member's own tiles leave at once. One grid for all of them keeps
+// every compute unit fed to the end: a launch of its own ends with compute units idle while the last workgroups finish
+// (512 x 11008 x 4096: 65 us alone, 60 / 52 / 50 us per matmul with 2 / 4 / 8 in a launch).
+struct Fp6Members {
+  float         *out[kGemmGroupMax];
+  const uint8_t *w_tiles[kGemmGroupMax];
+  int            n[kGemmGroupMax];
+  int            tiles_n[kGemmGroupMax];
+};
+
 template <int NT, int NS, int KS>
-__global__ __launch_bounds__(Shape<NT>::kWaves *kWave *KS) void gemm_fp6_lds_kernel(float *__restrict__ out,
+__global__ __launch_bounds__(Shape<NT>::kWaves *kWave *KS) void gemm_fp6_lds_kernel(Fp6Members grp,
                                                                                    const uint8_t *__restrict__ a_tiles,
                                                                                    const uint8_t *__restrict__ a_scales,
-                                                                                   const uint8_t *__restrict__ w_tiles, int m,
-                                                                                   int n, int pairs, int tiles_m, int tiles_n) {
+                                                                                   int m, int pairs, int tiles_m) {
+  float *__restrict__ out           = grp.out[blockIdx.y];
+  const uint8_t *__restrict__ w_tiles = grp.w_tiles[blockIdx.y];
+  const int n = grp.n[blockIdx.y], tiles_n = grp.tiles_n[blockIdx.y];
   using S = Shape<NT>;
   constexpr int kStage = S::kStage, kRing = NS * S::kStage, kOffSa = S::kOffSa;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
@@ -456,14 +469,22 @@ __global__ __launch_bounds__(Shape<NT>::kWaves *kWave *KS) void gemm_fp6_lds_ker
   }
 }
 
+// (count members: outs, w_tiles and ns of the matmuls that take this instance)
 template <int NT, int NS, int KS>
-hipError_t launch_instance(hipStream_t stream, float *out, const uint8_t *a_tiles, const uint8_t *a_scales,
-                           const uint8_t *w_tiles, int m, int n, int pairs) {
+hipError_t launch_instance(hipStream_t stream, int count, float *const *outs, const uint8_t *a_tiles, const uint8_t *a_scales,
+                           const uint8_t *const *w_tiles, int m, const int *ns, int pairs) {
   using S = Shape<NT>;
-  const int    tiles_m = (m + kBM - 1) / kBM, tiles_n = (n + 32 * NT - 1) / (32 * NT);
+  const int    tiles_m = (m + kBM - 1) / kBM;
   const size_t lds     = (size_t) KS * NS * S::kStage;
   static_assert((size_t) KS * NS * S::kStage <= 160 * 1024, "the rings fit LDS");
-  const dim3   grid((unsigned) (((tiles_n + 7) / 8) * 8 * tiles_m));
+  Fp6Members grp = {};
+  int        widest = 0;
+  for (int i = 0; i < count; ++i) {
+    grp.out[i] = outs[i], grp.w_tiles[i] = w_tiles[i], grp.n[i] = ns[i];
+    grp.tiles_n[i] = (ns[i] + 32 * NT - 1) / (32 * NT);
+    widest         = std::max(widest, grp.tiles_n[i]);
+  }
+  const dim3   grid((unsigned) (((widest + 7) / 8) * 8 * tiles_m), (unsigned) count);
   auto         kernel  = gemm_fp6_lds_kernel<NT, NS, KS>;
   static bool  raised  = false;
   if (!raised) {
@@ -473,8 +494,7 @@ hipError_t launch_instance(hipStream_t stream, float *out, const uint8_t *a_tile
     }
     raised = true;
   }
-  hipLaunchKernelGGL(kernel, grid, dim3(S::kWaves * kWave * KS), lds, stream, out, a_tiles, a_scales, w_tiles, m, n, pairs,
-                     tiles_m, tiles_n);
+  hipLaunchKernelGGL(kernel, grid, dim3(S::kWaves * kWave * KS), lds, stream, grp, a_tiles, a_scales, m, pairs, tiles_m);
   return hipGetLastError();
 }
 
@@ -497,8 +517,11 @@ constexpr int kWdPerWave = (kWdDma + kWdWaves - 1) / kWdWaves;
 constexpr int kWdMinTiles = 512;  // 128 x 128 output tiles from which this kernel is used
 
 __global__ __launch_bounds__(kWdWaves *kWave, 2) void gemm_fp6_lds_wide_kernel(
-    float *__restrict__ out, const uint8_t *__restrict__ a_tiles, const uint8_t *__restrict__ a_scales,
-    const uint8_t *__restrict__ w_tiles, int m, int n, int pairs, int tiles_m, int tiles_n) {
+    Fp6Members grp, const uint8_t *__restrict__ a_tiles, const uint8_t *__restrict__ a_scales, int m, int pairs,
+    int tiles_m) {
+  float *__restrict__ out           = grp.out[blockIdx.y];
+  const uint8_t *__restrict__ w_tiles = grp.w_tiles[blockIdx.y];
+  const int n = grp.n[blockIdx.y], tiles_n = grp.tiles_n[blockIdx.y];
   constexpr int NS = kWdStages, kStage = kWdStage;
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const int lane = threadIdx.x & 63;
@@ -675,11 +698,17 @@ __global__ __launch_bounds__(kWdWaves *kWave, 2) void gemm_fp6_lds_wide_kernel(
   }
 }
 
-hipError_t launch_wide(hipStream_t stream, float *out, const uint8_t *a_tiles, const uint8_t *a_scales, const uint8_t *w_tiles,
-                       int m, int n, int pairs) {
-  const int    tiles_m = (m + 127) / 128, tiles_n = (n + 127) / 128;
+hipError_t launch_wide(hipStream_t stream, int count, float *const *outs, const uint8_t *a_tiles, const uint8_t *a_scales,
+                       const uint8_t *const *w_tiles, int m, const int *ns, int pairs) {
+  const int    tiles_m = (m + 127) / 128;
   const size_t lds     = (size_t) kWdStages * kWdStage;
-  const dim3   grid((unsigned) (((tiles_n + 7) / 8) * 8 * tiles_m));
+  Fp6Members   grp     = {};
+  int          widest  = 0;
+  for (int i = 0; i < count; ++i) {
+    grp.out[i] = outs[i], grp.w_tiles[i] = w_tiles[i], grp.n[i] = ns[i], grp.tiles_n[i] = (ns[i] + 127) / 128;
+    widest = std::max(widest, grp.tiles_n[i]);
+  }
+  const dim3   grid((unsigned) (((widest + 7) / 8) * 8 * tiles_m), (unsigned) count);
   static bool  raised  = false;
   if (!raised) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_fp6_lds_wide_kernel),
@@ -689,8 +718,8 @@ hipError_t launch_wide(hipStream_t stream, float *out, const uint8_t *a_tiles, c
     }
     raised = true;
   }
-  hipLaunchKernelGGL(gemm_fp6_lds_wide_kernel, grid, dim3(kWdWaves * kWave), lds, stream, out, a_tiles, a_scales, w_tiles, m,
-                     n, pairs, tiles_m, tiles_n);
+  hipLaunchKernelGGL(gemm_fp6_lds_wide_kernel, grid, dim3(kWdWaves * kWave), lds, stream, grp, a_tiles, a_scales, m, pairs,
+                     tiles_m);
   return hipGetLastError();
 }
 
@@ -726,10 +755,16 @@ hipError_t launch_q4_0_to_fp6_tiles(hipStream_t stream, void *dst, const void *w
   return hipGetLastError();
 }
 
-hipError_t launch_gemm_fp6_lds(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_tiles, int m, int k,
-                               int n, void *act_tiles, bool act_tiles_ready) {
-  if (!gemm_fp6_lds_fits(m, k, n) || (reinterpret_cast<uintptr_t>(act_q8_0) & 3) != 0) {
+hipError_t launch_gemm_fp6_lds_group(hipStream_t stream, int count, float *const *outs, const void *act_q8_0,
+                                     const void *const *weight_tiles, int m, int k, const int *ns, void *act_tiles,
+                                     bool act_tiles_ready) {
+  if (count < 1 || count > kGemmGroupMax || (reinterpret_cast<uintptr_t>(act_q8_0) & 3) != 0) {
     return hipErrorNotSupported;
+  }
+  for (int i = 0; i < count; ++i) {
+    if (!gemm_fp6_lds_fits(m, k, ns[i])) {
+      return hipErrorNotSupported;
+    }
   }
   const int pairs   = k / 64;
   const int m_tiles = (m + 31) / 32;
@@ -744,29 +779,51 @@ hipError_t launch_gemm_fp6_lds(hipStream_t stream, float *out, const void *act_q
       return e;
     }
   }
-  const uint8_t *wt      = static_cast<const uint8_t *>(weight_tiles);
+  // Which kernel a member takes depends on its own shape, as if it were launched alone:
   // 128 x 128 tiles from where they fill two workgroups per compute unit (10 % faster there: 84 against 95 us at
-  // 512 x 16384 x 4096)
-  if ((long) ((m + 127) / 128) * ((n + 127) / 128) >= kWdMinTiles) {
-    return launch_wide(stream, out, tiles, scales, wt, m, n, pairs);
-  }
-  const long     tiles64 = (long) ((m + kBM - 1) / kBM) * ((n + 63) / 64);
+  // 512 x 16384 x 4096); else
   // 128 x 64 tiles: a K group is 4 waves (one per SIMD) and one ring of three stages, and a compute unit holds three
   // rings: one group per workgroup when the tiles alone give every compute unit three workgroups, otherwise up to
   // three groups per workgroup, each with its share of K, so that the same tiles put more waves on a compute unit.
   // (128 x 96 tiles -- NT = 3, four stages, two workgroups of 6 waves per compute unit, a third fewer activation bytes
   // per unit of work -- measured slower, 84 against 64 us at 512 x 11008 x 4096: six waves do not spread evenly over
-  // four SIMDs.)
-  int ks = tiles64 >= 640 ? 1 : tiles64 >= 384 ? 2 : 3;
-  ks     = std::max(1, std::min(ks, pairs / 4));
-  switch (ks) {
-    case 1:
-      return launch_instance<2, 3, 1>(stream, out, tiles, scales, wt, m, n, pairs);
-    case 2:
-      return launch_instance<2, 3, 2>(stream, out, tiles, scales, wt, m, n, pairs);
-    default:
-      return launch_instance<2, 3, 3>(stream, out, tiles, scales, wt, m, n, pairs);
+  // four SIMDs.) Members that take the same kernel share its launch.
+  int kind[kGemmGroupMax];  // 0: 128 x 128 tiles; 1..3: K groups per workgroup of the 128 x 64 kernel
+  for (int i = 0; i < count; ++i) {
+    if ((long) ((m + 127) / 128) * ((ns[i] + 127) / 128) >= kWdMinTiles) {
+      kind[i] = 0;
+    } else {
+      const long tiles64 = (long) ((m + kBM - 1) / kBM) * ((ns[i] + 63) / 64);
+      const int  ks      = tiles64 >= 640 ? 1 : tiles64 >= 384 ? 2 : 3;
+      kind[i]            = std::max(1, std::min(ks, pairs / 4));
+    }
   }
+  for (int which = 0; which <= 3; ++which) {
+    float         *o[kGemmGroupMax];
+    const uint8_t *w[kGemmGroupMax];
+    int            n[kGemmGroupMax], c = 0;
+    for (int i = 0; i < count; ++i) {
+      if (kind[i] == which) {
+        o[c] = outs[i], w[c] = static_cast<const uint8_t *>(weight_tiles[i]), n[c++] = ns[i];
+      }
+    }
+    if (c == 0) {
+      continue;
+    }
+    const hipError_t e = which == 0 ? launch_wide(stream, c, o, tiles, scales, w, m, n, pairs) :
+                         which == 1 ? launch_instance<2, 3, 1>(stream, c, o, tiles, scales, w, m, n, pairs) :
+                         which == 2 ? launch_instance<2, 3, 2>(stream, c, o, tiles, scales, w, m, n, pairs) :
+                                      launch_instance<2, 3, 3>(stream, c, o, tiles, scales, w, m, n, pairs);
+    if (e != hipSuccess) {
+      return e;
+    }
+  }
+  return hipSuccess;
+}
+
+hipError_t launch_gemm_fp6_lds(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_tiles, int m, int k,
+                               int n, void *act_tiles, bool act_tiles_ready) {
+  return launch_gemm_fp6_lds_group(stream, 1, &out, act_q8_0, &weight_tiles, m, k, &n, act_tiles, act_tiles_ready);
 }
 
 }  // namespace htpops

@@ -1173,6 +1173,7 @@ struct GemvBatch {
     int                   ne0 = 0;
   } norm;
   bool fused = false;  // the members read norm.dst and run in the launch that makes it
+  bool fp6   = false;  // many-row members of the FP6-tile kernel (all over the same activation rows and k)
 };
 
 // The many-row members of a batch: converted weights from the cache (made now where missing), the distinct activation
@@ -1238,6 +1239,53 @@ int run_fragment_group(htpops_context *ctx, GemvBatch &b) {
   return HTPOPS_OK;
 }
 
+// The many-row members of a batch that take the FP6-tile kernel over one set of activation rows: converted weights from
+// the cache (made now where missing), the activations converted once (or found converted at the start of the
+// workspace), one launch per kernel variant for the products. Returns a status, or 1 when the members have to be run
+// one by one after all.
+int run_fp6_group(htpops_context *ctx, GemvBatch &b) {
+  const void *wf[htpops::kGemmGroupMax];
+  size_t      act_bytes = 0;
+  for (int i = 0; i < b.count; ++i) {
+    MatMulPlan plan = plan_mat_mul(ctx, b.w[i], true, b.m, b.k[i], b.n[i], b.wt);
+    if (plan.kind != kPlanLdsFp6 || !(plan.cached || plan.cacheable)) {
+      return 1;  // (a converted copy went away since the member joined: the caller runs the members one by one)
+    }
+    if (!plan.cached) {
+      void *fresh = nullptr;
+      HTPOPS_HIP(ctx, hipMalloc(&fresh, plan.weight_bytes));
+      const hipError_t e = htpops::launch_q4_0_to_fp6_tiles(ctx->stream, fresh, b.w[i], b.k[i], b.n[i]);
+      if (e != hipSuccess) {
+        (void) hipFree(fresh);
+        return fail(ctx, HTPOPS_ERR_HIP, "weight conversion: %s", hipGetErrorString(e));
+      }
+      ctx->frag_cache.push_back({ b.w[i], weight_bytes((size_t) b.n[i], (size_t) b.k[i], b.wt), plan.frag_kind, b.k[i], b.n[i], fresh });
+      plan.cached = fresh;
+    }
+    wf[i]     = plan.cached;
+    act_bytes = plan.act_bytes;
+  }
+  if (int r = ensure_workspace(ctx, act_bytes)) {
+    return r;
+  }
+  // (note_device_write for the outputs, done by the caller, has already dropped the record if a member writes into
+  // the activations)
+  const int    m = b.m, k = b.k[0];
+  const size_t a_bytes = q8_0_bytes((size_t) m, (size_t) k);
+  auto        &af      = ctx->act_fragments;
+  const bool   ready   = af.src == b.act[0] && af.m == m && af.k == k && af.kind == (int) kPlanLdsFp6;
+  bool         keep    = ready || (ctx->in_message && in_owned_buffer(ctx, b.act[0], a_bytes));
+  for (int i = 0; i < b.count; ++i) {
+    keep = keep && !ranges_overlap(b.out[i], (size_t) m * b.n[i] * 4, b.act[0], a_bytes);
+  }
+  af.src = nullptr;
+  HTPOPS_HIP(ctx, htpops::launch_gemm_fp6_lds_group(ctx->stream, b.count, b.out, b.act[0], wf, m, k, b.n, ctx->workspace, ready));
+  if (keep) {
+    af.src = b.act[0], af.src_bytes = a_bytes, af.m = m, af.k = k, af.kind = (int) kPlanLdsFp6;
+  }
+  return HTPOPS_OK;
+}
+
 void flush_batch(htpops_context *ctx, GemvBatch &b) {
   if (b.norm.waiting) {
     b.norm.waiting = false;
@@ -1284,7 +1332,7 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
     const int        k0 = b.k[0];
     hipError_t e;
     if (b.m > kBatchMaxM) {
-      ret = run_fragment_group(ctx, b);
+      ret = b.fp6 ? run_fp6_group(ctx, b) : run_fragment_group(ctx, b);
       e   = ret == 1 ? hipErrorNotSupported : hipSuccess;
       ret = ret == 1 ? HTPOPS_OK : ret;
     } else if (b.m == 1) {
@@ -1411,14 +1459,17 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
     return false;  // the ordinary path reports what is wrong, or handles the aliasing in order
   }
   const bool many_rows = p->m > kBatchMaxM;
+  bool       fp6       = false;
   if (many_rows) {
-    // only matmuls that take the fragment kernel in its small-tile configuration over a converted copy kept with the
-    // weight buffer; everything else runs on its own
-    if (!htpops::gemm_i8_fragments_groupable(p->m, p->n)) {
+    // only matmuls over a converted copy kept with the weight buffer that take the FP6-tile kernel (members of a launch
+    // read the same activation rows) or the fragment kernel in its small-tile configuration; everything else runs on
+    // its own
+    const MatMulPlan plan = plan_mat_mul(ctx, w, aligned(act, 4), p->m, p->k, p->n, wt);
+    if (!(plan.cached || plan.cacheable)) {
       return false;
     }
-    const MatMulPlan plan = plan_mat_mul(ctx, w, true, p->m, p->k, p->n, wt);
-    if (plan.kind != kPlanFragments || !(plan.cached || plan.cacheable)) {
+    fp6 = plan.kind == kPlanLdsFp6;
+    if (!fp6 && !(plan.kind == kPlanFragments && htpops::gemm_i8_fragments_groupable(p->m, p->n))) {
       return false;
     }
   }
@@ -1436,6 +1487,7 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
     }
   }
   bool join = b.count > 0 && b.count < htpops::kGemvGroupMax && b.wt == wt && b.m == p->m && (!b.fused || reads_norm) &&
+              b.fp6 == fp6 && (!fp6 || (b.act[0] == act && b.k[0] == p->k)) &&
               (p->m == 1 || many_rows || b.k[0] == p->k ||
                (htpops::gemv_rows_fits(p->m, p->k, (htpops::WeightType) wt) &&
                 htpops::gemv_rows_fits(b.m, b.k[0], (htpops::WeightType) wt)));
@@ -1452,7 +1504,7 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
     if (b.count > 0) {
       flush_batch(ctx, b);
     }
-    b.wt = wt, b.m = p->m;
+    b.wt = wt, b.m = p->m, b.fp6 = fp6;
   }
   b.hdr[b.count] = hdr, b.out[b.count] = out, b.w[b.count] = w, b.act[b.count] = act, b.n[b.count] = p->n, b.k[b.count] = p->k;
   ++b.count;

@@ -791,6 +791,39 @@ def test_message_groups_independent_few_row_matmuls(ctx, oracle, wt, m):
             ctx.release(h)
 
 
+def test_message_groups_many_row_matmuls_over_the_same_rows(ctx, oracle):
+    # Independent many-row Q4_0 matmuls over the SAME activation rows (q/k/v or gate/up of a prefill chunk) whose
+    # weights live in buffers of the context share the launch of the FP6-tile kernel (one grid keeps the compute units
+    # fed to the end). Every request must equal its own launch bit for bit; one that reads other rows starts a new launch.
+    wt, op = wl.GGML_TYPE_Q4_0, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0
+    rng = wl.rng_for(81, 0)
+    m, k = 512, 1024
+    ns = [4096, 3072, 6144, 3072]
+    act_of = [0, 0, 0, 1]
+    ws = [wl.make_weights(rng, n, k, wt) for n in ns]
+    acts = [oracle.quantize_q8_0(wl.make_activations(rng, m, k)) for _ in range(2)]
+    has, hws = [ctx.upload(a) for a in acts], [ctx.upload(w) for w in ws]
+    hos = [ctx.alloc(m * n * 4) for n in ns]
+    try:
+        msg = api.build_message([_mm(op, ho, has[g], hw, m, k, n) for ho, g, hw, n in zip(hos, act_of, hws, ns)])
+        for _ in range(2):
+            for ho, n in zip(hos, ns):
+                ctx.write(ho, np.full(m * n, np.nan, np.float32))
+            assert ctx.process_message(msg) == 0
+            assert api.message_request_states(msg) == [0] * len(ns), ctx.last_error()
+            assert ctx.last_message_submissions() == 2
+            for ho, g, w, n in zip(hos, act_of, ws, ns):
+                got = ctx.read(ho, np.float32, m * n).reshape(m, n)
+                assert np.array_equal(got, ctx.run_mat_mul(acts[g], w, m, k, n, wt)), "a request differs from its own launch"
+                rows = [0, 31, 32, 300, m - 1]
+                cols = np.unique(np.linspace(0, n - 1, 40).astype(int))
+                want, mag = oracle.mat_mul_q8_0_act_f64(acts[g][rows], w[cols], len(rows), k, len(cols), wt)
+                assert np.all(np.abs(got[np.ix_(rows, cols)] - want) <= MATMUL_RTOL * mag)
+    finally:
+        for h in has + hws + hos:
+            ctx.release(h)
+
+
 def _norm_q(hq, hx, hg, k, rows, eps):
     return (api.REQUEST_TYPE_OP_COMPUTE,
             api.op_compute_request(api.HTP_OPS_RMS_NORM_QUANTIZE_Q8_0, api.rms_norm_ex_params((hq, 0), (hx, 0), (hg, 0), k, rows, eps)))
