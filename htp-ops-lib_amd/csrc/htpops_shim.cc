@@ -1265,7 +1265,7 @@ int run_fp6_group(htpops_context *ctx, GemvBatch &b) {
     wf[i]     = plan.cached;
     act_bytes = plan.act_bytes;
   }
-  if (int r = ensure_workspace(ctx, act_bytes)) {
+  if (int r = ensure_workspace(ctx, act_bytes, true)) {  // (tiles already there for these rows stay)
     return r;
   }
   // (note_device_write for the outputs, done by the caller, has already dropped the record if a member writes into

@@ -819,6 +819,19 @@ def test_message_groups_many_row_matmuls_over_the_same_rows(ctx, oracle):
                 cols = np.unique(np.linspace(0, n - 1, 40).astype(int))
                 want, mag = oracle.mat_mul_q8_0_act_f64(acts[g][rows], w[cols], len(rows), k, len(cols), wt)
                 assert np.all(np.abs(got[np.ix_(rows, cols)] - want) <= MATMUL_RTOL * mag)
+        # ten requests over the same rows: a launch takes eight, the ninth starts another that finds the rows converted
+        more = [ctx.alloc(m * ns[1] * 4) for _ in range(10)]
+        try:
+            msg = api.build_message([_mm(op, ho, has[0], hws[1], m, k, ns[1]) for ho in more])
+            assert ctx.process_message(msg) == 0
+            assert api.message_request_states(msg) == [0] * 10, ctx.last_error()
+            assert ctx.last_message_submissions() == 2
+            want = ctx.run_mat_mul(acts[0], ws[1], m, k, ns[1], wt)
+            for ho in more:
+                assert np.array_equal(ctx.read(ho, np.float32, m * ns[1]).reshape(m, ns[1]), want)
+        finally:
+            for h in more:
+                ctx.release(h)
     finally:
         for h in has + hws + hos:
             ctx.release(h)
