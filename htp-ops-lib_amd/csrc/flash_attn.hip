@@ -488,18 +488,10 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
   const int k_begin = split * SPLIT;
   const int k_end   = min(kv_len, k_begin + SPLIT);
 
-  // all K and V of this lane, requested up front (keys of a pass are consecutive across slots)
-  v8h kreg[PASSES], vreg[PASSES];
-#pragma unroll
-  for (int p = 0; p < PASSES; ++p) {
-    const int    key = min(k_begin + p * SLOTS + slot, k_end - 1);
-    const size_t off = (size_t) key * kv_stride + (size_t) h_kv * D + sub * 8;
-    kreg[p]          = *reinterpret_cast<const v8h *>(k_ptr + off);
-    vreg[p]          = *reinterpret_cast<const v8h *>(v_ptr + off);
-  }
-
-  // q for the GH heads, this lane's 8 dims. fp32 queries are pre-scaled and multiplied in fp32; fp16 queries stay
-  // fp16 pairs for v_dot2_f32_f16 (exact products, fp32 sums) and the scale is applied to the finished score.
+  // q for the GH heads, this lane's 8 dims, requested FIRST, then all K, then all V: loads return in order, so the
+  // scores of a pass need only that pass's K to have arrived, and the exponentials only the scores. fp32 queries are
+  // pre-scaled and multiplied in fp32; fp16 queries stay fp16 pairs for v_dot2_f32_f16 (exact products, fp32 sums) and
+  // the scale is applied to the finished score.
   typedef _Float16 v2h __attribute__((ext_vector_type(2)));
   float q[GH][8];
   v2h   q2[GH][4];
@@ -519,6 +511,21 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
         q2[g][e] = (v2h){ qv[2 * e], qv[2 * e + 1] };
       }
     }
+  }
+
+  // all K and V of this lane, requested up front (keys of a pass are consecutive across slots)
+  v8h kreg[PASSES], vreg[PASSES];
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    const int    key = min(k_begin + p * SLOTS + slot, k_end - 1);
+    const size_t off = (size_t) key * kv_stride + (size_t) h_kv * D + sub * 8;
+    kreg[p]          = *reinterpret_cast<const v8h *>(k_ptr + off);
+  }
+#pragma unroll
+  for (int p = 0; p < PASSES; ++p) {
+    const int    key = min(k_begin + p * SLOTS + slot, k_end - 1);
+    const size_t off = (size_t) key * kv_stride + (size_t) h_kv * D + sub * 8;
+    vreg[p]          = *reinterpret_cast<const v8h *>(v_ptr + off);
   }
 
   float sc[PASSES][GH];
