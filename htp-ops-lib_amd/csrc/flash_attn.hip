@@ -563,10 +563,17 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
   // one maximum per head for the whole workgroup: over the wave's key slots, then over the waves
 #pragma unroll
   for (int g = 0; g < GH; ++g) {
-#pragma unroll
-    for (int off = LPK; off < kWave; off <<= 1) {
-      m_loc[g] = fmaxf(m_loc[g], __shfl_xor(m_loc[g], off, kWave));
+    // (the LPK lanes of a key hold the same score: DPP row operations over the key slots, the result in lane 63)
+    float v = m_loc[g];
+#define HTPOPS_DPP_MAX(ctrl, rows) \
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), ctrl, rows, 0xf, false)))
+    if (LPK == 8) {
+      HTPOPS_DPP_MAX(0x140, 0xf);  // row_mirror: the two keys of a 16-lane row
     }
+    HTPOPS_DPP_MAX(0x142, 0xa);  // row_bcast15 into rows 1 and 3
+    HTPOPS_DPP_MAX(0x143, 0xc);  // row_bcast31 into rows 2 and 3
+#undef HTPOPS_DPP_MAX
+    m_loc[g] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
     if (lane == 0) {
       red_m[wave * GH + g] = m_loc[g];
     }
@@ -641,6 +648,35 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
 // is neither LDS nor a barrier; chunks are folded into a running (max, sum, column) like KV blocks are.
 constexpr int kMergeChunk = 64;
 
+// maximum / sum over the 64 lanes of a wave with DPP row operations (no trip through the LDS crossbar); every lane
+// gets the result
+#define HTPOPS_DPP_STEP(op, ctrl, rows) \
+  v = op(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(ident), __float_as_int(v), ctrl, rows, 0xf, false)))
+__device__ __forceinline__ float wave_max(float v) {
+  const float ident = -INFINITY;
+  HTPOPS_DPP_STEP(fmaxf, 0xB1, 0xf);   // quad_perm [1,0,3,2]
+  HTPOPS_DPP_STEP(fmaxf, 0x4E, 0xf);   // quad_perm [2,3,0,1]
+  HTPOPS_DPP_STEP(fmaxf, 0x141, 0xf);  // row_half_mirror
+  HTPOPS_DPP_STEP(fmaxf, 0x140, 0xf);  // row_mirror: every lane of a 16-lane row holds the row's
+  HTPOPS_DPP_STEP(fmaxf, 0x142, 0xa);  // row_bcast15 into rows 1 and 3
+  HTPOPS_DPP_STEP(fmaxf, 0x143, 0xc);  // row_bcast31 into rows 2 and 3: lane 63 holds the wave's
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+__device__ __forceinline__ float wave_add(float a, float b) {
+  return a + b;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  const float ident = 0.0f;
+  HTPOPS_DPP_STEP(wave_add, 0xB1, 0xf);
+  HTPOPS_DPP_STEP(wave_add, 0x4E, 0xf);
+  HTPOPS_DPP_STEP(wave_add, 0x141, 0xf);
+  HTPOPS_DPP_STEP(wave_add, 0x140, 0xf);
+  HTPOPS_DPP_STEP(wave_add, 0x142, 0xa);
+  HTPOPS_DPP_STEP(wave_add, 0x143, 0xc);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+#undef HTPOPS_DPP_STEP
+
 template <int D, bool QO_F32>
 __global__ __launch_bounds__(D) void flash_attn_decode_merge_kernel(void *__restrict__ o_ptr,
                                                                     const float *__restrict__ part, int n_splits) {
@@ -660,11 +696,11 @@ __global__ __launch_bounds__(D) void flash_attn_decode_merge_kernel(void *__rest
     for (int u = 0; u < kMergeChunk; ++u) {
       x[u] = u < left ? rec0[(size_t) (s0 + u) * (D + 2) + 2 + d] : 0.0f;
     }
-    const float m_new  = fmaxf(m_run, group_max<kWave>(m_s));
+    const float m_new  = fmaxf(m_run, wave_max(m_s));
     const float m_safe = (m_new == -INFINITY) ? 0.0f : m_new;
     const float keep   = fast_exp2(m_run - m_safe);  // 0 for the first chunk
     const float f      = fast_exp2(m_s - m_safe);    // 0 in lanes without a split
-    l_run              = l_run * keep + group_sum<kWave>(l_s * f);
+    l_run              = l_run * keep + wave_sum(l_s * f);
     float v            = 0.0f;
 #pragma unroll
     for (int u = 0; u < kMergeChunk; ++u) {
