@@ -648,34 +648,6 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
 // is neither LDS nor a barrier; chunks are folded into a running (max, sum, column) like KV blocks are.
 constexpr int kMergeChunk = 64;
 
-// maximum / sum over the 64 lanes of a wave with DPP row operations (no trip through the LDS crossbar); every lane
-// gets the result
-#define HTPOPS_DPP_STEP(op, ctrl, rows) \
-  v = op(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(ident), __float_as_int(v), ctrl, rows, 0xf, false)))
-__device__ __forceinline__ float wave_max(float v) {
-  const float ident = -INFINITY;
-  HTPOPS_DPP_STEP(fmaxf, 0xB1, 0xf);   // quad_perm [1,0,3,2]
-  HTPOPS_DPP_STEP(fmaxf, 0x4E, 0xf);   // quad_perm [2,3,0,1]
-  HTPOPS_DPP_STEP(fmaxf, 0x141, 0xf);  // row_half_mirror
-  HTPOPS_DPP_STEP(fmaxf, 0x140, 0xf);  // row_mirror: every lane of a 16-lane row holds the row's
-  HTPOPS_DPP_STEP(fmaxf, 0x142, 0xa);  // row_bcast15 into rows 1 and 3
-  HTPOPS_DPP_STEP(fmaxf, 0x143, 0xc);  // row_bcast31 into rows 2 and 3: lane 63 holds the wave's
-  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
-}
-__device__ __forceinline__ float wave_add(float a, float b) {
-  return a + b;
-}
-__device__ __forceinline__ float wave_sum(float v) {
-  const float ident = 0.0f;
-  HTPOPS_DPP_STEP(wave_add, 0xB1, 0xf);
-  HTPOPS_DPP_STEP(wave_add, 0x4E, 0xf);
-  HTPOPS_DPP_STEP(wave_add, 0x141, 0xf);
-  HTPOPS_DPP_STEP(wave_add, 0x140, 0xf);
-  HTPOPS_DPP_STEP(wave_add, 0x142, 0xa);
-  HTPOPS_DPP_STEP(wave_add, 0x143, 0xc);
-  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
-}
-#undef HTPOPS_DPP_STEP
 
 template <int D, bool QO_F32>
 __global__ __launch_bounds__(D) void flash_attn_decode_merge_kernel(void *__restrict__ o_ptr,

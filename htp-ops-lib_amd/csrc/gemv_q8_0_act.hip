@@ -461,7 +461,7 @@ __device__ __forceinline__ void gemv_row_sets(const GemvMember &mem, int wg, uin
         }
       }
     }
-    ss = group_sum<kWave>(ss);
+    ss = wave_sum(ss);
     if (lane == 0 && wave < 4) {
       red[wave] = ss;
     }
@@ -491,7 +491,7 @@ __device__ __forceinline__ void gemv_row_sets(const GemvMember &mem, int wg, uin
         for (int i = 0; i < 8; ++i) {
           amax = fmaxf(amax, fabsf(y[i]));
         }
-        amax           = group_max<4>(amax);
+        amax           = quad_max(amax);
         const float d  = amax / 127.0f;
         const float id = (d != 0.0f) ? 1.0f / d : 0.0f;
         if (blk < nb) {

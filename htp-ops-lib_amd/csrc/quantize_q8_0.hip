@@ -55,7 +55,7 @@ __global__ __launch_bounds__(kThreads) void quantize_q8_0_kernel(uint8_t *__rest
   for (int i = 0; i < 8; ++i) {
     amax = fmaxf(amax, fabsf(x[i]));
   }
-  amax = group_max<4>(amax);
+  amax = quad_max(amax);
 
   const float d  = amax / 127.0f;
   const float id = (d != 0.0f) ? 1.0f / d : 0.0f;

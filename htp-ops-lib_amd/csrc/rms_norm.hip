@@ -16,7 +16,7 @@ constexpr int kThreads = 256;
 constexpr int kWaves   = kThreads / kWave;
 
 __device__ __forceinline__ float block_sum(float v, float *lds) {
-  v = group_sum<kWave>(v);
+  v = wave_sum(v);
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   if (lane == 0) {
     lds[wave] = v;
@@ -43,7 +43,10 @@ __global__ __launch_bounds__(kThreads) void rms_norm_reg_kernel(float *__restric
   float       *y   = dst + row * ne0;
   const int    n8  = ne0 / 8;
 
-  float v[PAIRS][8];
+  // (short rows fetch their norm weights together with the row instead of behind the sum of squares: one trip to
+  // memory less in a kernel that is a chain of such trips; longer rows would pay for that with registers)
+  constexpr bool kEarly = PAIRS <= 2;
+  float v[PAIRS][8], gw[kEarly ? PAIRS : 1][8];
   float ss = 0.0f;
 #pragma unroll
   for (int b = 0; b < PAIRS; ++b) {
@@ -53,6 +56,12 @@ __global__ __launch_bounds__(kThreads) void rms_norm_reg_kernel(float *__restric
       const float4  a0 = p[0], a1 = p[1];
       v[b][0] = a0.x, v[b][1] = a0.y, v[b][2] = a0.z, v[b][3] = a0.w;
       v[b][4] = a1.x, v[b][5] = a1.y, v[b][6] = a1.z, v[b][7] = a1.w;
+      if (kEarly && weight) {
+        const float4 *wp = reinterpret_cast<const float4 *>(weight + idx * 8);
+        const float4  w0 = wp[0], w1 = wp[1];
+        float        *g  = gw[kEarly ? b : 0];
+        g[0] = w0.x, g[1] = w0.y, g[2] = w0.z, g[3] = w0.w, g[4] = w1.x, g[5] = w1.y, g[6] = w1.z, g[7] = w1.w;
+      }
     } else {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -76,7 +85,12 @@ __global__ __launch_bounds__(kThreads) void rms_norm_reg_kernel(float *__restric
       for (int i = 0; i < 8; ++i) {
         o[i] = v[b][i] * scale;
       }
-      if (weight) {
+      if (weight && kEarly) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          o[i] *= gw[kEarly ? b : 0][i];
+        }
+      } else if (weight) {
         const float4 *wp = reinterpret_cast<const float4 *>(weight + idx * 8);
         const float4  w0 = wp[0], w1 = wp[1];
         o[0] *= w0.x, o[1] *= w0.y, o[2] *= w0.z, o[3] *= w0.w;
@@ -128,9 +142,10 @@ __global__ __launch_bounds__(kThreads) void rms_norm_quantize_kernel(uint8_t *__
   uint8_t     *out = dst + row * (size_t) nb * 34;
 
   // slice s = thread + b * kThreads holds floats 8 s .. 8 s + 7: a quad of lanes covers one quant block
-  const int part = threadIdx.x & 3;
-  float     v[BPT][8];
-  float     ss = 0.0f;
+  const int      part   = threadIdx.x & 3;
+  constexpr bool kEarly = BPT <= 2;  // (norm weights of short rows together with the row, see rms_norm_reg_kernel)
+  float          v[BPT][8], gw[kEarly ? BPT : 1][8];
+  float          ss = 0.0f;
 #pragma unroll
   for (int b = 0; b < BPT; ++b) {
     const int blk = (threadIdx.x >> 2) + b * (kThreads / 4);
@@ -139,6 +154,12 @@ __global__ __launch_bounds__(kThreads) void rms_norm_quantize_kernel(uint8_t *__
       const float4  a0 = p[0], a1 = p[1];
       v[b][0] = a0.x, v[b][1] = a0.y, v[b][2] = a0.z, v[b][3] = a0.w;
       v[b][4] = a1.x, v[b][5] = a1.y, v[b][6] = a1.z, v[b][7] = a1.w;
+      if (kEarly && weight) {
+        const float4 *wp = reinterpret_cast<const float4 *>(weight + blk * kQK + part * 8);
+        const float4  w0 = wp[0], w1 = wp[1];
+        float        *g  = gw[kEarly ? b : 0];
+        g[0] = w0.x, g[1] = w0.y, g[2] = w0.z, g[3] = w0.w, g[4] = w1.x, g[5] = w1.y, g[6] = w1.z, g[7] = w1.w;
+      }
     } else {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
@@ -163,7 +184,12 @@ __global__ __launch_bounds__(kThreads) void rms_norm_quantize_kernel(uint8_t *__
     for (int i = 0; i < 8; ++i) {
       y[i] = v[b][i] * scale;
     }
-    if (weight && blk < nb) {
+    if (weight && blk < nb && kEarly) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        y[i] *= gw[kEarly ? b : 0][i];
+      }
+    } else if (weight && blk < nb) {
       const float4 *wp = reinterpret_cast<const float4 *>(weight + blk * kQK + part * 8);
       const float4  w0 = wp[0], w1 = wp[1];
       y[0] *= w0.x, y[1] *= w0.y, y[2] *= w0.z, y[3] *= w0.w;
@@ -173,7 +199,7 @@ __global__ __launch_bounds__(kThreads) void rms_norm_quantize_kernel(uint8_t *__
     for (int i = 0; i < 8; ++i) {
       amax = fmaxf(amax, fabsf(y[i]));
     }
-    amax           = group_max<4>(amax);
+    amax           = quad_max(amax);
     const float d  = amax / 127.0f;
     const float id = (d != 0.0f) ? 1.0f / d : 0.0f;
     if (blk < nb) {
