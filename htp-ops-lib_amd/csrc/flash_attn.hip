@@ -617,7 +617,7 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
     if (head0_in_group + g >= group) {
       continue;
     }
-    float v0 = 0.0f, v1 = 0.0f, l = 0.0f;
+    float v0 = 0.0f, v1 = 0.0f;
 #pragma unroll
     for (int w = 0; w < SLOTS; ++w) {
       const float2 x = *reinterpret_cast<const float2 *>(red_o + ((size_t) w * GH + g) * D + d);
@@ -625,19 +625,19 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
     }
     const int head = h_kv * group + head0_in_group + g;
     float    *rec  = part + ((size_t) head * n_splits + split) * (D + 2);
-    if (d == 0) {
-#pragma unroll
-      for (int w = 0; w < SLOTS; ++w) {
-        l += red_l[w * GH + g];
-      }
-      float m_all = red_m[g];
-#pragma unroll
-      for (int w = 1; w < WAVES; ++w) {
-        m_all = fmaxf(m_all, red_m[w * GH + g]);
-      }
-      *reinterpret_cast<float2 *>(rec) = make_float2(m_all, l);
-    }
     *reinterpret_cast<float2 *>(rec + 2 + d) = make_float2(v0, v1);
+  }
+  // (maximum, sum) of head g by wave g % WAVES: a slot's sum per lane, added up across the wave
+  static_assert(SLOTS <= kWave, "a lane per slot");
+#pragma unroll
+  for (int g = 0; g < GH; ++g) {
+    if (g % WAVES == wave && head0_in_group + g < group) {
+      const float l = wave_sum(lane < SLOTS ? red_l[lane * GH + g] : 0.0f);
+      if (lane == 0) {
+        float *rec = part + ((size_t) (h_kv * group + head0_in_group + g) * n_splits + split) * (D + 2);
+        *reinterpret_cast<float2 *>(rec) = make_float2(m_loc[g], l);
+      }
+    }
   }
 }
 
