@@ -1,5 +1,7 @@
 """GPU parity: Q8_0 quantizer (bit-exact), RMSNorm (2e-3 absolute; in practice ~1e-6), quantized matmul
 (|gpu - f64| <= 1e-5 * sum|terms|, and the same against the fp32 oracle), all through the op ABI."""
+import os
+
 import numpy as np
 import pytest
 
@@ -796,6 +798,7 @@ def test_message_groups_many_row_matmuls_over_the_same_rows(ctx, oracle):
     # weights live in buffers of the context share the launch of the FP6-tile kernel (one grid keeps the compute units
     # fed to the end). Every request must equal its own launch bit for bit; one that reads other rows starts a new launch.
     wt, op = wl.GGML_TYPE_Q4_0, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0
+    fp6 = os.environ.get("HTPOPS_GEMM_FP6", "-1") != "0"   # (switched off, every request is a launch of the int8 kernel)
     rng = wl.rng_for(81, 0)
     m, k = 512, 1024
     ns = [4096, 3072, 6144, 3072]
@@ -811,7 +814,7 @@ def test_message_groups_many_row_matmuls_over_the_same_rows(ctx, oracle):
                 ctx.write(ho, np.full(m * n, np.nan, np.float32))
             assert ctx.process_message(msg) == 0
             assert api.message_request_states(msg) == [0] * len(ns), ctx.last_error()
-            assert ctx.last_message_submissions() == 2
+            assert ctx.last_message_submissions() == (2 if fp6 else 4)
             for ho, g, w, n in zip(hos, act_of, ws, ns):
                 got = ctx.read(ho, np.float32, m * n).reshape(m, n)
                 assert np.array_equal(got, ctx.run_mat_mul(acts[g], w, m, k, n, wt)), "a request differs from its own launch"
@@ -825,7 +828,7 @@ def test_message_groups_many_row_matmuls_over_the_same_rows(ctx, oracle):
             msg = api.build_message([_mm(op, ho, has[0], hws[1], m, k, ns[1]) for ho in more])
             assert ctx.process_message(msg) == 0
             assert api.message_request_states(msg) == [0] * 10, ctx.last_error()
-            assert ctx.last_message_submissions() == 2
+            assert ctx.last_message_submissions() == (2 if fp6 else 10)
             want = ctx.run_mat_mul(acts[0], ws[1], m, k, ns[1], wt)
             for ho in more:
                 assert np.array_equal(ctx.read(ho, np.float32, m * ns[1]).reshape(m, ns[1]), want)
