@@ -651,7 +651,10 @@ constexpr int kMergeChunk = 64;
 
 template <int D, bool QO_F32>
 __global__ __launch_bounds__(D) void flash_attn_decode_merge_kernel(void *__restrict__ o_ptr,
-                                                                    const float *__restrict__ part, int n_splits) {
+                                                                    const float *__restrict__ part, int n_splits,
+                                                                    uint8_t *__restrict__ q8_out) {
+  // (q8_out, fp32 output only: the output row is also written as Q8_0 blocks, the bytes the Q8_0 quantizer makes of
+  // it; a block is 32 neighbouring columns, one half of a wave)
   const int    head = blockIdx.x, d = threadIdx.x, lane = threadIdx.x & (kWave - 1);
   const float *rec0 = part + (size_t) head * n_splits * (D + 2);
   float        m_run = -INFINITY, l_run = 0.0f, v_run = 0.0f;
@@ -684,6 +687,25 @@ __global__ __launch_bounds__(D) void flash_attn_decode_merge_kernel(void *__rest
   const float out = v_run * (1.0f / l_run);
   if (QO_F32) {
     reinterpret_cast<float *>(o_ptr)[(size_t) head * D + d] = out;
+    if (q8_out != nullptr) {
+      float amax = fabsf(out);
+#define HTPOPS_DPP_MAX(ctrl) \
+  amax = fmaxf(amax, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(amax), __float_as_int(amax), ctrl, 0xf, 0xf, false)))
+      HTPOPS_DPP_MAX(0xB1);   // quad_perm [1,0,3,2]
+      HTPOPS_DPP_MAX(0x4E);   // quad_perm [2,3,0,1]
+      HTPOPS_DPP_MAX(0x141);  // row_half_mirror
+      HTPOPS_DPP_MAX(0x140);  // row_mirror: the 16 lanes of a row
+#undef HTPOPS_DPP_MAX
+      amax            = fmaxf(amax, __shfl_xor(amax, 16, kWave));  // the two rows of the block
+      const float dq  = amax / 127.0f;
+      const float id  = (dq != 0.0f) ? 1.0f / dq : 0.0f;
+      const int   col = head * D + d;
+      uint8_t    *blk = q8_out + (size_t) (col >> 5) * 34;
+      blk[2 + (col & 31)] = (uint8_t) (int) roundf(out * id);
+      if ((col & 31) == 0) {
+        *reinterpret_cast<uint16_t *>(blk) = __half_as_ushort(__float2half_rn(dq));
+      }
+    }
   } else {
     reinterpret_cast<_Float16 *>(o_ptr)[(size_t) head * D + d] = (_Float16) out;
   }
@@ -885,7 +907,7 @@ hipError_t launch_decode_pass(hipStream_t stream, dim3 grid, float *workspace, c
 
 template <int D, bool QO_F32>
 hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void *k, const void *v, const void *mask,
-                         int kv_len, int n_heads, int n_kv_heads, float *workspace) {
+                         int kv_len, int n_heads, int n_kv_heads, float *workspace, void *q8_out) {
   const int  group    = n_heads / n_kv_heads;
   // 64-key chunks while 128-key ones would give fewer than 128 workgroups (measured at 8 KV heads: kv = 512 8.8 -> 7.1 us;
   // kv = 4096 and 16384 are 1 and 6 us slower with 64)
@@ -917,11 +939,15 @@ hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void 
     }
   }
   hipLaunchKernelGGL((flash_attn_decode_merge_kernel<D, QO_F32>), dim3((unsigned) n_heads), dim3(D), 0, stream, o,
-                     workspace, n_splits);
+                     workspace, n_splits, QO_F32 ? static_cast<uint8_t *>(q8_out) : nullptr);
   return hipGetLastError();
 }
 
 }  // namespace
+
+bool flash_attn_writes_q8_0(int qo_len, int head_dim, bool qo_is_f32) {
+  return qo_len == 1 && qo_is_f32 && (head_dim == 64 || head_dim == 128);
+}
 
 size_t flash_attn_workspace_bytes(int qo_len, int kv_len, int n_heads, int head_dim) {
   if (qo_len != 1 || (head_dim != 64 && head_dim != 128)) {
@@ -933,7 +959,7 @@ size_t flash_attn_workspace_bytes(int qo_len, int kv_len, int n_heads, int head_
 
 hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const void *k, const void *v,
                              const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
-                             bool qo_is_f32, bool causal, void *workspace) {
+                             bool qo_is_f32, bool causal, void *workspace, void *q8_out) {
   if (head_dim != 64 && head_dim != 128) {
     if (head_dim <= 0 || head_dim % 2 != 0 || head_dim > kGenMaxD || qo_len > 0x7fffffff || n_heads > 65535) {
       return hipErrorNotSupported;
@@ -954,11 +980,11 @@ hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const v
   if (qo_len == 1) {
     float *ws = static_cast<float *>(workspace);
     if (head_dim == 128) {
-      return qo_is_f32 ? launch_decode<128, true>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws) :
-                         launch_decode<128, false>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws);
+      return qo_is_f32 ? launch_decode<128, true>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws, q8_out) :
+                         launch_decode<128, false>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws, q8_out);
     }
-    return qo_is_f32 ? launch_decode<64, true>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws) :
-                       launch_decode<64, false>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws);
+    return qo_is_f32 ? launch_decode<64, true>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws, q8_out) :
+                       launch_decode<64, false>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws, q8_out);
   }
   if (head_dim == 128) {
     return qo_is_f32 ?

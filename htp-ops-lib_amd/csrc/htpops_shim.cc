@@ -57,6 +57,10 @@ struct htpops_context {
   // buffers, as a host of the reference does while its consumer thread runs (reference: src/dsp/mmap_mgr.cc:15-27 maps
   // lazily on that thread). Recursive: a message's RPCMEM_MAP request releases buffers from inside the walk.
   std::recursive_mutex mu;
+  // Set by the message walk around an attention request whose output the next request quantizes to Q8_0: where that
+  // request wants its row, and whether the attention launch wrote it.
+  void               *attn_q8_out  = nullptr;
+  bool                attn_q8_done = false;
   int                 device     = HTPOPS_DEVICE_NONE;
   bool                has_device = false;
   hipStream_t         stream     = nullptr;
@@ -754,8 +758,14 @@ int op_flash_attn(htpops_context *ctx, void *o, const void *q, const void *k, co
     note_device_write(ctx, o, o_bytes);
     ws = ctx->workspace;
   }
+  void *q8_out = nullptr;
+  if (ctx->attn_q8_out && htpops::flash_attn_writes_q8_0(qo_len, head_dim, qo_is_f32 != 0)) {
+    q8_out = ctx->attn_q8_out;
+    note_device_write(ctx, q8_out, q8_0_bytes(1, (size_t) n_heads * head_dim));
+  }
   HTPOPS_HIP(ctx, htpops::launch_flash_attn(ctx->stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads,
-                                            head_dim, qo_is_f32 != 0, causal != 0, ws));
+                                            head_dim, qo_is_f32 != 0, causal != 0, ws, q8_out));
+  ctx->attn_q8_done = q8_out != nullptr;
   return HTPOPS_OK;
 }
 
@@ -1512,6 +1522,43 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
   return true;
 }
 
+// `next` behind a one-token fp32 attention request `req`: if it is the Q8_0 quantization of exactly that attention's
+// output row into a buffer that overlaps none of the attention's operands, notes where it wants the row
+// (ctx->attn_q8_out) and returns it; nullptr otherwise.
+struct RequestHeader *attention_output_quantizer(htpops_context *ctx, const struct OpComputeRequest *req,
+                                                 struct RequestHeader *next, size_t next_size) {
+  const auto *p = reinterpret_cast<const FlashAttnParams *>(req->payload);
+  if (!ctx->has_device || next->type != REQUEST_TYPE_OP_COMPUTE ||
+      next_size < sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest) + sizeof(RmsNormF32Params)) {
+    return nullptr;
+  }
+  const auto *nreq = reinterpret_cast<const struct OpComputeRequest *>(next->data);
+  const auto *pq   = reinterpret_cast<const RmsNormF32Params *>(nreq->payload);
+  if (nreq->op != HTP_OPS_QUANTIZE_Q8_0 || p->qo_len != 1 || p->kv_len <= 0 || p->n_heads <= 0 || p->n_kv_heads <= 0 ||
+      p->head_dim <= 0 || p->n_heads > (1 << 20) || p->head_dim > 256 || pq->ne1 != 1 ||
+      pq->ne0 != p->n_heads * p->head_dim || !htpops::flash_attn_writes_q8_0(1, p->head_dim, true)) {
+    return nullptr;
+  }
+  const size_t row = (size_t) pq->ne0 * 4, q_bytes = q8_0_bytes(1, (size_t) pq->ne0);
+  const size_t kv  = (size_t) p->kv_len * p->n_kv_heads * p->head_dim * 2;
+  const void  *o = resolve(ctx, p->o, row), *src = resolve(ctx, pq->src, row);
+  void        *dst = resolve(ctx, pq->dst, q_bytes);
+  const void  *q = resolve(ctx, p->q, row), *k = resolve(ctx, p->k, kv), *v = resolve(ctx, p->v, kv);
+  if (!o || o != src || !dst || !q || !k || !v || !aligned(dst, 4) || ranges_overlap(dst, q_bytes, o, row) ||
+      ranges_overlap(dst, q_bytes, q, row) || ranges_overlap(dst, q_bytes, k, kv) || ranges_overlap(dst, q_bytes, v, kv)) {
+    return nullptr;
+  }
+  if (p->mask.fd >= 0 && lookup(ctx, p->mask.fd)) {
+    const size_t mask_bytes = ((size_t) p->kv_len + 63) / 64 * 64 * 2;
+    const void  *mask       = resolve(ctx, p->mask, mask_bytes);
+    if (mask && ranges_overlap(dst, q_bytes, mask, mask_bytes)) {
+      return nullptr;
+    }
+  }
+  ctx->attn_q8_out = dst;
+  return next;
+}
+
 // 0, or the error if the request table does not fit `msg_bytes` (0 = unknown size, offsets are trusted)
 int check_message_framing(htpops_context *ctx, const struct MessageHeader *msg, size_t msg_bytes) {
   const int n_reqs = msg->n_reqs;
@@ -1570,7 +1617,21 @@ int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_b
               !(matmul_payload && try_batch(ctx, req, hdr, batch))) {
             flush_batch(ctx, batch);
             ++ctx->message_submissions;
-            hdr->state = htpops_execute_op(ctx, req);
+            // one-token attention whose fp32 output the NEXT request quantizes to Q8_0 (on its way to the o projection):
+            // the launch that finishes the attention writes that row too, and the next request is done with it
+            struct RequestHeader *next = nullptr;
+            if (req->op == HTP_OPS_FLASH_ATTN_QO_F32_KV_F16 && i + 1 < n_reqs &&
+                size >= sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest) + sizeof(FlashAttnParams)) {
+              next = attention_output_quantizer(ctx, req, message_header_get_request_ptr(msg, i + 1),
+                                                message_header_get_request_size(msg, i + 1));
+            }
+            ctx->attn_q8_done = false;
+            hdr->state        = htpops_execute_op(ctx, req);
+            ctx->attn_q8_out  = nullptr;
+            if (next && ctx->attn_q8_done && hdr->state == HTPOPS_OK) {
+              next->state = HTPOPS_OK;
+              ++i;  // (the row is written: that request needs no launch)
+            }
           }
         }
         break;

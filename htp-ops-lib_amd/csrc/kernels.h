@@ -132,11 +132,14 @@ hipError_t launch_mat_mul_fragments(hipStream_t stream, float *out, const float 
                                     int m, int k, int n, void *act_fragments);
 
 // attention; see htpops_flash_attn_ptr. `workspace` holds split-KV partials (decode), size from
-// flash_attn_workspace_bytes.
+// flash_attn_workspace_bytes. `q8_out` (or nullptr; used only where flash_attn_writes_q8_0 says so: decode with
+// head_dim 64 / 128 and fp32 output): the output row is also written there as Q8_0 blocks, bit for bit what
+// launch_quantize_q8_0 makes of it.
 size_t     flash_attn_workspace_bytes(int qo_len, int kv_len, int n_heads, int head_dim);
 hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const void *k, const void *v,
                              const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
-                             bool qo_is_f32, bool causal, void *workspace);
+                             bool qo_is_f32, bool causal, void *workspace, void *q8_out);
+bool       flash_attn_writes_q8_0(int qo_len, int head_dim, bool qo_is_f32);
 
 // measurement helpers
 hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t bytes);

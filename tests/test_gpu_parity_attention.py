@@ -75,6 +75,42 @@ def test_prefill_with_one_and_two_key_groups(ctx, oracle, monkeypatch, groups, q
         assert np.abs(got.astype(np.float32) - want.astype(np.float32)).max() <= ATOL
 
 
+@pytest.mark.parametrize("kv,nh,nkv,d", [(300, 8, 2, 128), (4096, 32, 8, 128), (70, 4, 4, 64), (1, 4, 2, 64), (9000, 16, 2, 128)])
+def test_message_attention_then_quantization_of_its_output(ctx, oracle, kv, nh, nkv, d):
+    # One-token attention followed by the Q8_0 quantization of its output row (on its way to the o projection): the
+    # launch that finishes the attention writes the Q8_0 row too. The fp32 output is the attention's own, and the row
+    # is bit for bit the quantizer's (the oracle's) of that output. A quantization of other rows, a two-token
+    # attention and a head dim of the plain kernel keep their own launches.
+    rng = wl.rng_for(62, kv * 100 + nh)
+    q, k, v = wl.make_attention_inputs(rng, 1, kv, nh, nkv, d)
+    q32 = q.astype(np.float32)
+    ne0 = nh * d
+    hq, hk, hv = ctx.upload(q32), ctx.upload(k), ctx.upload(v)
+    ho, hq8 = ctx.alloc(ne0 * 4), ctx.alloc(ne0 // 32 * 34)
+    hother = ctx.upload(wl.make_activations(rng, 1, ne0))
+    try:
+        def op(o, payload):
+            return (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(o, payload))
+
+        attn = op(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16,
+                  api.flash_attn_params((ho, 0), (hq, 0), (hk, 0), (hv, 0), (-1, 0), 1, kv, nh, nkv, d))
+        want_o = ctx.run_flash_attn(q32, k, v, None, nh, nkv, d)
+        for src, launches in ((ho, 1), (hother, 2)):
+            ctx.write(hq8, np.full(ne0 // 32 * 34, 0xA5, np.uint8))
+            ctx.write(ho, np.full(ne0, np.nan, np.float32))
+            msg = api.build_message([attn, op(api.HTP_OPS_QUANTIZE_Q8_0, api.rms_norm_params((hq8, 0), (src, 0), ne0, 1))])
+            assert ctx.process_message(msg) == 0
+            assert api.message_request_states(msg) == [0, 0], ctx.last_error()
+            assert ctx.last_message_submissions() == launches
+            got_o = ctx.read(ho, np.float32, ne0).reshape(1, nh, d)
+            assert np.array_equal(got_o, want_o)
+            row = got_o.reshape(1, ne0) if src == ho else ctx.read(hother, np.float32, ne0).reshape(1, ne0)
+            assert np.array_equal(ctx.read(hq8, np.uint8, ne0 // 32 * 34), oracle.quantize_q8_0(row)[0])
+    finally:
+        for h in (hq, hk, hv, ho, hq8, hother):
+            ctx.release(h)
+
+
 def test_fixtures_from_the_reference_routine(ctx, golden_dir):
     files = sorted(glob.glob(os.path.join(golden_dir, "naive_flash_attn_*.npz")))
     assert len(files) >= 3
