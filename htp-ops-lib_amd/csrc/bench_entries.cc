@@ -1,0 +1,148 @@
+// Timers and calibration kernels for the bench harness (include/htpops_bench.h); nothing here is on an op's path and
+// nothing has a counterpart in the reference.
+#include "context.h"
+#include "htpops_bench.h"
+
+using namespace htpops;
+using namespace htpops::host;
+
+// ------------------------------------------------------------------------------------------------ measurement
+
+extern "C" int htpops_timer_start(htpops_context *ctx) {
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_timer_stop(htpops_context *ctx) {
+  if (!ctx) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_timer_elapsed_ms(htpops_context *ctx, float *ms) {
+  if (!ctx || !ms) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  HTPOPS_HIP(ctx, hipEventSynchronize(ctx->ev_stop));
+  HTPOPS_HIP(ctx, hipEventElapsedTime(ms, ctx->ev_start, ctx->ev_stop));
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_measure_mfma_peak(htpops_context *ctx, int kind, int iters, double *tera_ops) {
+  if (!ctx || !tera_ops || iters <= 0 || kind < 0 || kind > 2) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  hipDeviceProp_t prop;
+  HTPOPS_HIP(ctx, hipGetDeviceProperties(&prop, ctx->device));
+  const int n_blocks = prop.multiProcessorCount * 2;  // 4 waves per block -> 2 waves per SIMD
+  int      *sink     = nullptr;
+  HTPOPS_HIP(ctx, hipMalloc((void **) &sink, sizeof(int)));
+  hipError_t e = launch_mfma_loop(ctx->stream, kind, 16, sink, n_blocks);  // warm-up
+  float      ms = 0.f;
+  if (e == hipSuccess) e = hipEventRecord(ctx->ev_start, ctx->stream);
+  if (e == hipSuccess) e = launch_mfma_loop(ctx->stream, kind, iters, sink, n_blocks);
+  if (e == hipSuccess) e = hipEventRecord(ctx->ev_stop, ctx->stream);
+  if (e == hipSuccess) e = hipEventSynchronize(ctx->ev_stop);
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop);
+  (void) hipFree(sink);
+  if (e != hipSuccess) {
+    return hip_fail(ctx, e, "mfma loop");
+  }
+  const double ops_per_mfma = kind == 0 ? 2.0 * 32 * 32 * 32 : (kind == 1 ? 2.0 * 16 * 16 * 64 : 2.0 * 32 * 32 * 16);
+  const double total        = (double) n_blocks * 4 /*waves*/ * (double) iters * 4 /*chains*/ * ops_per_mfma;
+  *tera_ops                 = total / ((double) ms * 1e-3) / 1e12;
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_measure_read_us(htpops_context *ctx, size_t bytes, int buffers, int iters, double *us_per_launch) {
+  if (!ctx || !us_per_launch || iters <= 0 || buffers <= 0 || buffers > 64 || bytes < 16) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  std::vector<void *> bufs;
+  unsigned           *sink = nullptr;
+  hipError_t          e    = hipMalloc(reinterpret_cast<void **>(&sink), 256);
+  for (int b = 0; b < buffers && e == hipSuccess; ++b) {
+    void *p = nullptr;
+    e       = hipMalloc(&p, bytes);
+    if (e == hipSuccess) {
+      bufs.push_back(p);
+      e = hipMemsetAsync(p, 1, bytes, ctx->stream);
+    }
+  }
+  float ms = 0.f;
+  for (size_t b = 0; b < bufs.size() && e == hipSuccess; ++b) {
+    e = launch_read(ctx->stream, bufs[b], bytes, sink);
+  }
+  if (e == hipSuccess) e = hipEventRecord(ctx->ev_start, ctx->stream);
+  for (int i = 0; i < iters && e == hipSuccess; ++i) {
+    for (size_t b = 0; b < bufs.size() && e == hipSuccess; ++b) {
+      e = launch_read(ctx->stream, bufs[b], bytes, sink);
+    }
+  }
+  if (e == hipSuccess) e = hipEventRecord(ctx->ev_stop, ctx->stream);
+  if (e == hipSuccess) e = hipEventSynchronize(ctx->ev_stop);
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop);
+  (void) hipStreamSynchronize(ctx->stream);
+  for (void *p : bufs) {
+    (void) hipFree(p);
+  }
+  (void) hipFree(sink);
+  if (e != hipSuccess) {
+    return hip_fail(ctx, e, "read loop");
+  }
+  *us_per_launch = (double) ms * 1e3 / ((double) iters * buffers);
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_measure_copy_bandwidth(htpops_context *ctx, size_t bytes, int iters, double *gbps) {
+  if (!ctx || !gbps || iters <= 0 || bytes < 16) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  void *a = nullptr, *b = nullptr;
+  HTPOPS_HIP(ctx, hipMalloc(&a, bytes));
+  hipError_t e = hipMalloc(&b, bytes);
+  if (e != hipSuccess) {
+    (void) hipFree(a);
+    return hip_fail(ctx, e, "hipMalloc");
+  }
+  float ms = 0.f;
+  e        = hipMemsetAsync(a, 1, bytes, ctx->stream);
+  if (e == hipSuccess) e = launch_copy(ctx->stream, b, a, bytes);
+  if (e == hipSuccess) e = hipEventRecord(ctx->ev_start, ctx->stream);
+  for (int i = 0; i < iters && e == hipSuccess; ++i) {
+    e = launch_copy(ctx->stream, b, a, bytes);
+  }
+  if (e == hipSuccess) e = hipEventRecord(ctx->ev_stop, ctx->stream);
+  if (e == hipSuccess) e = hipEventSynchronize(ctx->ev_stop);
+  if (e == hipSuccess) e = hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop);
+  (void) hipFree(a);
+  (void) hipFree(b);
+  if (e != hipSuccess) {
+    return hip_fail(ctx, e, "copy loop");
+  }
+  *gbps = 2.0 * (double) (bytes / 16 * 16) * iters / ((double) ms * 1e-3) / 1e9;
+  return HTPOPS_OK;
+}

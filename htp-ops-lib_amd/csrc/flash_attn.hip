@@ -26,6 +26,14 @@ namespace htpops {
 
 namespace {
 
+// What a mask value contributes to a score. Added as it is (the reference's scalar routine,
+// src/dsp/ops/flash_attn.c:1505-1512), or, with `threshold`, selecting the key: kept (0) iff mask > -16, dropped
+// (-inf) otherwise, NaN included (the kernel the reference dispatches, src/dsp/ops/flash_attn.c:448-460).
+__device__ __forceinline__ float mask_term(_Float16 mv, bool threshold) {
+  const float f = (float) mv;
+  return threshold ? (f > -16.0f ? 0.0f : -INFINITY) : f;
+}
+
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef _Float16 v2h __attribute__((ext_vector_type(2)));
@@ -60,7 +68,8 @@ __global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(
                                                                         const _Float16 *__restrict__ v_ptr,
                                                                         const _Float16 *__restrict__ mask, int qo_len,
                                                                         int kv_len, int n_heads, int n_kv_heads,
-                                                                        int causal) {
+                                                                        int flags) {
+  const bool causal = (flags & 1) != 0, mask_threshold = (flags & 2) != 0;
   __shared__ PrefillSmem<D> sm_all[GROUPS];
   constexpr int KSTEPS = D / 16;  // MFMA k-steps over the head dimension
   constexpr int DT     = D / 32;  // 32-row tiles of O^T
@@ -282,7 +291,8 @@ __global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(
           float add[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
           if (mask) {
             const v4h mv = mreg[kt][rg];
-            add[0] = (float) mv[0], add[1] = (float) mv[1], add[2] = (float) mv[2], add[3] = (float) mv[3];
+            add[0] = mask_term(mv[0], mask_threshold), add[1] = mask_term(mv[1], mask_threshold);
+            add[2] = mask_term(mv[2], mask_threshold), add[3] = mask_term(mv[3], mask_threshold);
           }
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -465,7 +475,7 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
                                                                     const _Float16 *__restrict__ v_ptr,
                                                                     const _Float16 *__restrict__ mask, int kv_len,
                                                                     int n_heads, int n_kv_heads, int head0_in_group,
-                                                                    int n_splits) {
+                                                                    int n_splits, int mask_threshold) {
   constexpr int LPK    = D / 8;        // lanes per key (8 halfs = 16 bytes each)
   constexpr int KPW    = kWave / LPK;  // keys per wave per pass
   constexpr int WAVES  = THREADS / kWave;
@@ -538,7 +548,7 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
   for (int p = 0; p < PASSES; ++p) {
     const int  key  = k_begin + p * SLOTS + slot;
     const bool live = key < k_end;
-    const float mk  = (mask && live) ? (float) mask[key] : 0.0f;  // row 0 of the mask (qo_len == 1)
+    const float mk  = (mask && live) ? mask_term(mask[key], mask_threshold != 0) : 0.0f;  // row 0 of the mask (qo_len == 1)
 #pragma unroll
     for (int g = 0; g < GH; ++g) {
       float s = 0.0f;
@@ -728,7 +738,8 @@ __global__ __launch_bounds__(kGenThreads) void flash_attn_any_dim_kernel(void *_
                                                                          const _Float16 *__restrict__ v_ptr,
                                                                          const _Float16 *__restrict__ mask, int qo_len,
                                                                          int kv_len, int n_heads, int n_kv_heads,
-                                                                         int head_dim, int causal) {
+                                                                         int head_dim, int flags) {
+  const bool causal = (flags & 1) != 0, mask_threshold = (flags & 2) != 0;
   __shared__ v2h   q_sh[kGenMaxD / 2];
   __shared__ float part_o[4][kGenMaxD];
   __shared__ float part_ml[4][2];
@@ -779,7 +790,7 @@ __global__ __launch_bounds__(kGenThreads) void flash_attn_any_dim_kernel(void *_
       }
       s = d0 + d1;
       if (mask) {
-        s += (float) mask[(size_t) row * mask_ld + key];
+        s += mask_term(mask[(size_t) row * mask_ld + key], mask_threshold);
       }
     }
     float mx = s;
@@ -856,7 +867,7 @@ __global__ __launch_bounds__(kGenThreads) void flash_attn_any_dim_kernel(void *_
 
 template <int D, bool QO_F32>
 hipError_t launch_prefill(hipStream_t stream, void *o, const void *q, const void *k, const void *v, const void *mask,
-                          int qo_len, int kv_len, int n_heads, int n_kv_heads, bool causal) {
+                          int qo_len, int kv_len, int n_heads, int n_kv_heads, bool causal, int forced, bool mask_threshold) {
   const int group      = n_heads / n_kv_heads;
   const int gc         = group < 4 ? group : 4;
   const int qsub       = 4 / gc;
@@ -872,23 +883,23 @@ hipError_t launch_prefill(hipStream_t stream, void *o, const void *q, const void
   // 2048 x 2048 without `causal` 117 against 107 us and 4096 x 4096 causal 242 against 214 us.
   constexpr unsigned kCus = 256;
   const unsigned     wgs  = grid.x * grid.y;
-  const int          forced = env_int("HTPOPS_ATTN_KEY_GROUPS", 0);  // 1 or 2: for tests and measurements
   const bool         two  = forced ? forced == 2 : (wgs <= kCus || (causal && wgs <= 2 * kCus));
   if (two) {
     hipLaunchKernelGGL((flash_attn_prefill_kernel<D, QO_F32, 2>), grid, dim3(kPfThreads * 2), 0, stream, o, q,
                        (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, qo_len, kv_len, n_heads,
-                       n_kv_heads, causal ? 1 : 0);
+                       n_kv_heads, (causal ? 1 : 0) | (mask_threshold ? 2 : 0));
   } else {
     hipLaunchKernelGGL((flash_attn_prefill_kernel<D, QO_F32, 1>), grid, dim3(kPfThreads), 0, stream, o, q,
                        (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, qo_len, kv_len, n_heads,
-                       n_kv_heads, causal ? 1 : 0);
+                       n_kv_heads, (causal ? 1 : 0) | (mask_threshold ? 2 : 0));
   }
   return hipGetLastError();
 }
 
 template <int D, int GH, bool QO_F32, int SPLIT, int THREADS>
 hipError_t launch_decode_pass(hipStream_t stream, dim3 grid, float *workspace, const void *q, const void *k, const void *v,
-                              const void *mask, int kv_len, int n_heads, int n_kv_heads, int h0, int n_splits) {
+                              const void *mask, int kv_len, int n_heads, int n_kv_heads, int h0, int n_splits,
+                              bool mask_threshold) {
   constexpr int    kSlots = (THREADS / kWave) * (kWave / (D / 8));
   constexpr size_t kLds   = ((size_t) kSlots * GH * D + (size_t) kSlots * GH + (size_t) (THREADS / kWave) * GH) * sizeof(float);
   static_assert(kLds <= 160 * 1024, "LDS of one compute unit");
@@ -901,13 +912,13 @@ hipError_t launch_decode_pass(hipStream_t stream, dim3 grid, float *workspace, c
     }
   }
   hipLaunchKernelGGL(kernel, grid, dim3(THREADS), kLds, stream, workspace, q, (const _Float16 *) k, (const _Float16 *) v,
-                     (const _Float16 *) mask, kv_len, n_heads, n_kv_heads, h0, n_splits);
+                     (const _Float16 *) mask, kv_len, n_heads, n_kv_heads, h0, n_splits, mask_threshold ? 1 : 0);
   return hipGetLastError();
 }
 
 template <int D, bool QO_F32>
 hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void *k, const void *v, const void *mask,
-                         int kv_len, int n_heads, int n_kv_heads, float *workspace, void *q8_out) {
+                         int kv_len, int n_heads, int n_kv_heads, float *workspace, void *q8_out, bool mask_threshold) {
   const int  group    = n_heads / n_kv_heads;
   // 64-key chunks while 128-key ones would give fewer than 128 workgroups (measured at 8 KV heads: kv = 512 8.8 -> 7.1 us;
   // kv = 4096 and 16384 are 1 and 6 us slower with 64)
@@ -921,9 +932,10 @@ hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void 
 #define HTPOPS_DECODE(GH)                                                                                              \
   e = short_kv ? launch_decode_pass<D, GH, QO_F32, kDecSplitShort, kDecThreads>(stream, grid, workspace, q, k, v, mask, \
                                                                                kv_len, n_heads, n_kv_heads, h0,        \
-                                                                               n_splits) :                             \
+                                                                               n_splits, mask_threshold) :             \
                  launch_decode_pass<D, GH, QO_F32, kDecSplit, kDecThreads>(stream, grid, workspace, q, k, v, mask,  \
-                                                                              kv_len, n_heads, n_kv_heads, h0, n_splits)
+                                                                              kv_len, n_heads, n_kv_heads, h0, n_splits, \
+                                                                              mask_threshold)
     if (gh > 4) {
       HTPOPS_DECODE(8);
     } else if (gh > 2) {
@@ -959,7 +971,8 @@ size_t flash_attn_workspace_bytes(int qo_len, int kv_len, int n_heads, int head_
 
 hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const void *k, const void *v,
                              const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
-                             bool qo_is_f32, bool causal, void *workspace, void *q8_out) {
+                             bool qo_is_f32, bool causal, void *workspace, void *q8_out, int forced_key_groups,
+                             bool mask_threshold) {
   if (head_dim != 64 && head_dim != 128) {
     if (head_dim <= 0 || head_dim % 2 != 0 || head_dim > kGenMaxD || qo_len > 0x7fffffff || n_heads > 65535) {
       return hipErrorNotSupported;
@@ -968,11 +981,11 @@ hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const v
     if (qo_is_f32) {
       hipLaunchKernelGGL(flash_attn_any_dim_kernel<true>, grid, dim3(kGenThreads), 0, stream, o, q,
                          (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, qo_len, kv_len, n_heads,
-                         n_kv_heads, head_dim, causal ? 1 : 0);
+                         n_kv_heads, head_dim, (causal ? 1 : 0) | (mask_threshold ? 2 : 0));
     } else {
       hipLaunchKernelGGL(flash_attn_any_dim_kernel<false>, grid, dim3(kGenThreads), 0, stream, o, q,
                          (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, qo_len, kv_len, n_heads,
-                         n_kv_heads, head_dim, causal ? 1 : 0);
+                         n_kv_heads, head_dim, (causal ? 1 : 0) | (mask_threshold ? 2 : 0));
     }
     return hipGetLastError();
   }
@@ -980,19 +993,23 @@ hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const v
   if (qo_len == 1) {
     float *ws = static_cast<float *>(workspace);
     if (head_dim == 128) {
-      return qo_is_f32 ? launch_decode<128, true>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws, q8_out) :
-                         launch_decode<128, false>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws, q8_out);
+      return qo_is_f32 ? launch_decode<128, true>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws, q8_out, mask_threshold) :
+                         launch_decode<128, false>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws, q8_out, mask_threshold);
     }
-    return qo_is_f32 ? launch_decode<64, true>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws, q8_out) :
-                       launch_decode<64, false>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws, q8_out);
+    return qo_is_f32 ? launch_decode<64, true>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws, q8_out, mask_threshold) :
+                       launch_decode<64, false>(stream, o, q, k, v, mask, kv_len, n_heads, n_kv_heads, ws, q8_out, mask_threshold);
   }
   if (head_dim == 128) {
     return qo_is_f32 ?
-             launch_prefill<128, true>(stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, causal) :
-             launch_prefill<128, false>(stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, causal);
+             launch_prefill<128, true>(stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, causal,
+                                        forced_key_groups, mask_threshold) :
+             launch_prefill<128, false>(stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, causal,
+                                        forced_key_groups, mask_threshold);
   }
-  return qo_is_f32 ? launch_prefill<64, true>(stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, causal) :
-                     launch_prefill<64, false>(stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, causal);
+  return qo_is_f32 ? launch_prefill<64, true>(stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, causal,
+                                        forced_key_groups, mask_threshold) :
+                     launch_prefill<64, false>(stream, o, q, k, v, mask, qo_len, kv_len, n_heads, n_kv_heads, causal,
+                                        forced_key_groups, mask_threshold);
 }
 
 }  // namespace htpops

@@ -693,10 +693,9 @@ struct TileConfig {
 // With 32 x 32 tiles the split follows K alone: a wave should have some 48 blocks or more to work through (its ring of
 // loads and its epilogue are paid once), so short K is not split at all and the four waves of a workgroup take four
 // neighbouring column tiles instead.
-TileConfig tile_config(int m, int n, int k) {
+TileConfig tile_config(int m, int n, int k, int forced_unit) {
   const int m_tiles = (m + 31) / 32, n_tiles = (n + 31) / 32, nblk = k / 32;
   const int wave_tiles  = ((m_tiles + 1) / 2) * ((n_tiles + 1) / 2);
-  const int forced_unit = env_int("HTPOPS_GEMM_TILE_UNITS", 0);  // read per call: tests run both tile sizes
   const int unit        = forced_unit == 1 || forced_unit == 2 ? forced_unit : (wave_tiles < 512 ? 1 : 2);
   if (unit == 1) {
     return { 1, nblk >= 192 ? 4 : nblk >= 96 ? 2 : 1 };
@@ -745,8 +744,8 @@ const uint32_t *scales_of(const void *fragments, size_t tiles, size_t nblk) {
 
 }  // namespace
 
-bool gemm_i8_fragments_groupable(int m, int n) {
-  return tile_config(m, n, 32).unit == 1;
+bool gemm_i8_fragments_groupable(int m, int n, int forced_unit) {
+  return tile_config(m, n, 32, forced_unit).unit == 1;
 }
 
 hipError_t launch_act_to_i8_fragments_group(hipStream_t stream, int count, void *const *act_fragments,
@@ -786,16 +785,16 @@ hipError_t launch_act_to_i8_fragments_group(hipStream_t stream, int count, void 
   return hipGetLastError();
 }
 
-size_t gemm_i8_fragments_exchange_bytes(int m, int n, int k) {
+size_t gemm_i8_fragments_exchange_bytes(int m, int n, int k, int forced_unit) {
   const int           m_tiles = (m + 31) / 32, n_tiles = (n + 31) / 32, nblk = k / 32;
-  const SmallTilePlan plan    = small_tile_plan(m_tiles, nblk, tile_config(m, n, k), true);
+  const SmallTilePlan plan    = small_tile_plan(m_tiles, nblk, tile_config(m, n, k, forced_unit), true);
   return plan.kparts > 1 ? (size_t) ((n_tiles + 7) / 8 * 8) * m_tiles * plan.kparts * 1024 * sizeof(float) : 0;
 }
 
 hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *const *outs,
                                           const void *const *act_fragments, const void *const *weight_fragments,
                                           const int *ns, const int *ks, int m, void *exchange, size_t exchange_bytes,
-                                          unsigned *tickets, int ticket_slots) {
+                                          unsigned *tickets, int ticket_slots, int forced_unit) {
   if (count < 1 || count > kGemmGroupMax || m <= 0) {
     return hipErrorInvalidValue;
   }
@@ -811,14 +810,14 @@ hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *
   for (int i = 0; i < count; ++i) {
     order[i] = i;
   }
-  auto walk = [&](int i) { return ks[i] <= 0 || ns[i] <= 0 ? 0 : ks[i] / 32 / tile_config(m, ns[i], ks[i]).ksplit; };
+  auto walk = [&](int i) { return ks[i] <= 0 || ns[i] <= 0 ? 0 : ks[i] / 32 / tile_config(m, ns[i], ks[i], forced_unit).ksplit; };
   std::stable_sort(order, order + count, [&](int a, int b) { return walk(a) > walk(b); });
   for (int slot = 0; slot < count; ++slot) {
     const int i = order[slot];
     if (ks[i] <= 0 || ks[i] % 32 != 0 || ns[i] <= 0) {
       return hipErrorInvalidValue;
     }
-    const TileConfig c = tile_config(m, ns[i], ks[i]);
+    const TileConfig c = tile_config(m, ns[i], ks[i], forced_unit);
     if (slot > 0 && (c.unit != cfg.unit || (c.unit != 1 && c.ksplit != cfg.ksplit))) {
       return hipErrorNotSupported;  // every member runs in the configuration it would get alone
     }
@@ -835,7 +834,7 @@ hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *
     grp.m[slot].ksplit   = c.ksplit;
     grp.m[slot].wg_begin = total;
     // K split over workgroups while the caller's scratch for partial tiles and its ticket counters last
-    const size_t  xbytes  = gemm_i8_fragments_exchange_bytes(m, ns[i], ks[i]);
+    const size_t  xbytes  = gemm_i8_fragments_exchange_bytes(m, ns[i], ks[i], forced_unit);
     const int     xslots  = (n_tiles + 7) / 8 * 8 * m_tiles;
     const bool    split_k = exchange && tickets && xbytes > 0 && exchange_used + xbytes <= exchange_bytes &&
                          tickets_used + xslots <= ticket_slots;
@@ -864,7 +863,7 @@ hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *
 
 hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_fragments,
                                     int m, int k, int n, void *act_fragments, bool act_fragments_ready, void *exchange,
-                                    size_t exchange_bytes, unsigned *tickets, int ticket_slots) {
+                                    size_t exchange_bytes, unsigned *tickets, int ticket_slots, int forced_unit) {
   if (k % 32 != 0 || m <= 0 || n <= 0) {
     return hipErrorInvalidValue;
   }
@@ -875,7 +874,7 @@ hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *
   }
   const void *af = act_fragments;
   return launch_gemm_i8_fragments_group(stream, 1, &out, &af, &weight_fragments, &n, &k, m, exchange, exchange_bytes, tickets,
-                                        ticket_slots);
+                                        ticket_slots, forced_unit);
 }
 
 }  // namespace htpops

@@ -977,8 +977,7 @@ bool gemv_rows_fits(int m, int k, WeightType wt) {
   // free up to eight
   (void) wt;
   const int nblk = k / kQK;
-  return m >= 2 && m <= 3 && k % (2 * kQK) == 0 && nblk / 2 <= kSharedActMaxPairs &&
-         env_int("HTPOPS_GEMV_ROWS_KERNEL", 1) != 0;
+  return m >= 2 && m <= 3 && k % (2 * kQK) == 0 && nblk / 2 <= kSharedActMaxPairs;
 }
 
 hipError_t launch_gemv_rows_group_q8_0_act(hipStream_t stream, int count, float *const *outs, const void *const *acts,

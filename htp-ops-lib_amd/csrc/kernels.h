@@ -70,7 +70,7 @@ hipError_t launch_weights_to_lane_order(hipStream_t stream, void *dst, const voi
 // (one launch for `count` matmuls of the same m, k and weight type; member i reads the activation rows acts[i])
 hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *const *outs, const void *const *acts,
                                           const void *const *lane_order_weights, const int *ns, int m, int k,
-                                          WeightType wt);
+                                          WeightType wt, int forced_tiles);  // forced_tiles 2 / 3: one / two tiles per workgroup
 // many-row path for Q4_0 weights, k % 64 == 0: FP6 scaled MFMA (exact: int8 = 16 hi + lo, all parts |t| <= 15) over operand
 // tiles staged in LDS by DMA. The weight tiles (gemm_fp6_lds_weight_tile_bytes, 1 byte per weight) are converted once
 // (launch_q4_0_to_fp6_tiles) and can be cached by the caller; the activation tiles (gemm_fp6_lds_act_tile_bytes) are
@@ -92,17 +92,18 @@ hipError_t launch_weights_to_i8_fragments(hipStream_t stream, void *dst, const v
                                           WeightType wt);
 // `exchange` (gemm_i8_fragments_exchange_bytes; may be 0) and `tickets` (zeroed counters, left zeroed): scratch for shapes
 // whose K is split over workgroups. Without them those shapes run unsplit: correct, slower, and rounded differently.
-size_t     gemm_i8_fragments_exchange_bytes(int m, int n, int k);
+// (`forced_unit` 1 / 2 forces the tile size that the shape would otherwise choose; 0: the kernel's own choice)
+size_t     gemm_i8_fragments_exchange_bytes(int m, int n, int k, int forced_unit);
 hipError_t launch_gemm_i8_fragments(hipStream_t stream, float *out, const void *act_q8_0, const void *weight_fragments,
                                     int m, int k, int n, void *act_fragments, bool act_fragments_ready, void *exchange,
-                                    size_t exchange_bytes, unsigned *tickets, int ticket_slots);
+                                    size_t exchange_bytes, unsigned *tickets, int ticket_slots, int forced_unit);
 // The same for up to kGemmGroupMax matmuls of one row count m in one launch each for the conversions and the products:
 // member i multiplies the converted activations act_fragments[i] (gemm_i8_act_fragment_bytes(m, ks[i]) each; members
 // that read the same rows may share one) by weight_fragments[i]. Every member must be `groupable` (the tile
 // configuration it gets depends on (m, n) alone, and a launch has one), else hipErrorNotSupported; a member's result
 // is bit for bit what its own launch gives, provided `exchange` holds the sum of the members' exchange bytes.
 constexpr int kGemmGroupMax = 8;
-bool       gemm_i8_fragments_groupable(int m, int n);
+bool       gemm_i8_fragments_groupable(int m, int n, int forced_unit);
 // launch_gemm_fp6_lds for up to kGemmGroupMax matmuls over the SAME activation rows (one conversion, act_tiles): the
 // members that take the same kernel share one launch, whose grid keeps the compute units fed to the end (measured at
 // 512 x 11008 x 4096: 65 us alone, 60 / 52 / 50 us per matmul with 2 / 4 / 8 in a launch). A member's result is bit
@@ -115,7 +116,7 @@ hipError_t launch_act_to_i8_fragments_group(hipStream_t stream, int count, void 
 hipError_t launch_gemm_i8_fragments_group(hipStream_t stream, int count, float *const *outs,
                                           const void *const *act_fragments, const void *const *weight_fragments,
                                           const int *ns, const int *ks, int m, void *exchange, size_t exchange_bytes,
-                                          unsigned *tickets, int ticket_slots);
+                                          unsigned *tickets, int ticket_slots, int forced_unit);
 // picks between the one-row and the small-batch kernel by m (any m; many rows are better served by the fragment path)
 size_t     mat_mul_workspace_bytes(int m, int k, int n);
 hipError_t launch_mat_mul_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,
@@ -134,11 +135,14 @@ hipError_t launch_mat_mul_fragments(hipStream_t stream, float *out, const float 
 // attention; see htpops_flash_attn_ptr. `workspace` holds split-KV partials (decode), size from
 // flash_attn_workspace_bytes. `q8_out` (or nullptr; used only where flash_attn_writes_q8_0 says so: decode with
 // head_dim 64 / 128 and fp32 output): the output row is also written there as Q8_0 blocks, bit for bit what
-// launch_quantize_q8_0 makes of it.
+// launch_quantize_q8_0 makes of it. `forced_key_groups` 1 / 2 forces how many key groups a prefill workgroup holds
+// (0: by grid size). `mask_threshold`: the mask selects keys (keep iff mask > -16, reference:
+// src/dsp/ops/flash_attn.c:448-460) instead of being added to the scores (:1505-1512).
 size_t     flash_attn_workspace_bytes(int qo_len, int kv_len, int n_heads, int head_dim);
 hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const void *k, const void *v,
                              const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
-                             bool qo_is_f32, bool causal, void *workspace, void *q8_out);
+                             bool qo_is_f32, bool causal, void *workspace, void *q8_out, int forced_key_groups,
+                             bool mask_threshold);
 bool       flash_attn_writes_q8_0(int qo_len, int head_dim, bool qo_is_f32);
 
 // measurement helpers
@@ -146,8 +150,5 @@ hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t by
 // one pass over `bytes` (16-byte multiples) that keeps nothing; `sink` is one device word the kernel never writes in practice
 hipError_t launch_read(hipStream_t stream, const void *src, size_t bytes, unsigned *sink);
 hipError_t launch_mfma_loop(hipStream_t stream, int kind, int iters, int *sink, int n_blocks);
-
-// Integer value of an environment switch (the few there are select a kernel for tests and A/B measurements).
-int env_int(const char *name, int fallback);
 
 }  // namespace htpops

@@ -340,7 +340,7 @@ hipError_t launch_weights_to_lane_order(hipStream_t stream, void *dst, const voi
 
 hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *const *outs, const void *const *acts,
                                           const void *const *lane_order_weights, const int *ns, int m, int k,
-                                          WeightType wt) {
+                                          WeightType wt, int forced_tiles) {
   if (count < 1 || count > kGemvGroupMax) {
     return hipErrorNotSupported;
   }
@@ -380,8 +380,7 @@ hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *
   for (int i = 0; i < count; ++i) {
     pairs += (ns[i] / kLoRows + 1) / 2;
   }
-  const int    forced = env_int("HTPOPS_LANE_ORDER", 1);  // 2 / 3: one / two tiles per workgroup (read per call: tests run both)
-  const int    tpw    = forced == 2 || forced == 3 ? forced - 1 : (pairs >= 512 ? 2 : 1);
+  const int    tpw    = forced_tiles == 2 || forced_tiles == 3 ? forced_tiles - 1 : (pairs >= 512 ? 2 : 1);
   const dim3   grid((unsigned) ((n_max / kLoRows + tpw - 1) / tpw), (unsigned) count);
   const int    rows = panel_rows(m);
   const size_t lds  = panel_bytes(k, rows);

@@ -116,9 +116,4 @@ hipError_t launch_mfma_loop(hipStream_t stream, int kind, int iters, int *sink, 
   return hipGetLastError();
 }
 
-int env_int(const char *name, int fallback) {
-  const char *v = getenv(name);
-  return (v && *v) ? atoi(v) : fallback;
-}
-
 }  // namespace htpops

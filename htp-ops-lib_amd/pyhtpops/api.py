@@ -47,7 +47,9 @@ GGML_TYPE_Q4_0 = 2
 GGML_TYPE_Q8_0 = 8
 
 EXPORTED_SYMBOLS = [
-    "htpops_init_backend", "htpops_close", "htpops_last_error", "htpops_synchronize", "htpops_get_stream",
+    "htpops_init_backend", "htpops_close", "htpops_last_error", "htpops_set_option", "htpops_get_option",
+    "htpops_synchronize", "htpops_get_stream", "htpops_buffer_prepare_weights", "htpops_converted_bytes",
+    "htpops_workspace_bytes",
     "htpops_buffer_alloc", "htpops_buffer_register", "htpops_buffer_release", "htpops_buffer_device_ptr",
     "htpops_buffer_size", "htpops_buffer_invalidate", "htpops_buffer_write", "htpops_buffer_read", "htpops_execute_op",
     "htpops_process_message", "htpops_enqueue_message", "htpops_finish_message", "htpops_last_message_submissions",
@@ -57,6 +59,11 @@ EXPORTED_SYMBOLS = [
     "htpops_flash_attn_ptr", "htpops_flash_attn_noalloc_ptr", "htpops_timer_start", "htpops_timer_stop", "htpops_timer_elapsed_ms",
     "htpops_measure_mfma_peak", "htpops_measure_copy_bandwidth", "htpops_measure_read_us",
 ]
+
+
+# the switches of a context (htpops_set_option) and the values they start from
+DEFAULT_OPTIONS = {"lane_order": 1, "gemm_fp6": -1, "gemv_rows_kernel": 1, "gemm_tile_units": 0, "attn_key_groups": 0,
+                   "attn_mask_threshold": 0, "converted_cap_mib": 0, "log": 0}
 
 
 def build_library():
@@ -76,6 +83,11 @@ def load_library(path=None):
         "htpops_init_backend": (ci, [ctypes.POINTER(vp), ci]),
         "htpops_close": (ci, [vp]),
         "htpops_last_error": (ctypes.c_char_p, [vp]),
+        "htpops_set_option": (ci, [vp, ctypes.c_char_p, ci]),
+        "htpops_get_option": (ci, [vp, ctypes.c_char_p, ctypes.POINTER(ci)]),
+        "htpops_buffer_prepare_weights": (ci, [vp, ci, sz, ci, ci, ci, ci, ctypes.POINTER(sz)]),
+        "htpops_converted_bytes": (sz, [vp]),
+        "htpops_workspace_bytes": (sz, [vp]),
         "htpops_synchronize": (ci, [vp]),
         "htpops_get_stream": (vp, [vp]),
         "htpops_buffer_alloc": (ci, [vp, sz]),
@@ -213,6 +225,30 @@ class Context:
     def synchronize(self):
         self._check(self.lib.htpops_synchronize(self._ctx))
 
+    # -- switches --
+    def set_option(self, name, value):
+        self._check(self.lib.htpops_set_option(self._ctx, name.encode(), int(value)))
+
+    def get_option(self, name):
+        v = ctypes.c_int()
+        self._check(self.lib.htpops_get_option(self._ctx, name.encode(), ctypes.byref(v)))
+        return int(v.value)
+
+    def option(self, name, value):
+        """Context manager: the switch `name` holds `value` inside the with block and its old value afterwards."""
+        ctx = self
+
+        class _Scoped:
+            def __enter__(self_inner):
+                self_inner.old = ctx.get_option(name)
+                ctx.set_option(name, value)
+                return ctx
+
+            def __exit__(self_inner, *exc):
+                ctx.set_option(name, self_inner.old)
+
+        return _Scoped()
+
     # -- buffers --
     def alloc(self, nbytes):
         return self._check(self.lib.htpops_buffer_alloc(self._ctx, int(nbytes)))
@@ -232,6 +268,19 @@ class Context:
 
     def invalidate(self, handle):
         return self.lib.htpops_buffer_invalidate(self._ctx, int(handle))
+
+    def prepare_weights(self, handle, weight_type, n, k, m_hint, offset=0):
+        """htpops_buffer_prepare_weights; returns the bytes of converted copies the call added."""
+        added = ctypes.c_size_t()
+        self._check(self.lib.htpops_buffer_prepare_weights(self._ctx, int(handle), int(offset), int(weight_type), int(n),
+                                                           int(k), int(m_hint), ctypes.byref(added)))
+        return int(added.value)
+
+    def converted_bytes(self):
+        return int(self.lib.htpops_converted_bytes(self._ctx))
+
+    def workspace_bytes(self):
+        return int(self.lib.htpops_workspace_bytes(self._ctx))
 
     def write(self, handle, array, offset=0):
         a = np.ascontiguousarray(array)

@@ -8,7 +8,8 @@
  * runs messages while the host thread allocates, writes and releases
  * buffers): they are serialised by a lock inside the context. Ordering of
  * the work itself is the caller's: ops run in the order they are enqueued.
- * Several contexts may coexist.
+ * Every entry point takes that lock, htpops_last_error included (it returns a copy that belongs to the calling
+ * thread and stays valid until that thread's next call of it). Several contexts may coexist.
  *
  * Return codes: 0 success, -1 rejected request (same meaning as the
  * reference's ops: bad sizes, null/unknown buffers, misalignment), other
@@ -49,6 +50,22 @@ int htpops_close(htpops_context *ctx);
 /* Text of the most recent failure on this context (never NULL). */
 const char *htpops_last_error(const htpops_context *ctx);
 
+/* Switches of a context (no counterpart in the reference): kernel choices that tests and A/B measurements override,
+ * and two behaviours a host may want. Each starts from the environment variable HTPOPS_<NAME> (upper case) read when
+ * the context is created; nothing on the op path reads the environment afterwards. Unknown names return -1.
+ *   "attn_mask_threshold"  0 (default): the attention mask is ADDED to the scaled scores, the convention of the
+ *                          reference's scalar routine (src/dsp/ops/flash_attn.c:1505-1512). 1: the mask SELECTS keys,
+ *                          keep iff mask > -16 (compared in fp16), every other key is dropped, the convention of the
+ *                          kernel the reference dispatches for op 5 (src/dsp/ops/flash_attn.c:448-460). The two agree
+ *                          for masks of 0 and -inf only.
+ *   "converted_cap_mib"    0 (default): no limit. > 0: converted weight copies beyond this many MiB are evicted, least
+ *                          recently used first (copies used by the message being walked stay).
+ *   "lane_order", "gemm_fp6", "gemv_rows_kernel", "gemm_tile_units", "attn_key_groups"   force or forbid a kernel
+ *                          family / tile shape (for tests; results stay within every op's tolerance).
+ *   "log"                  1: failures are also printed to stderr. */
+int htpops_set_option(htpops_context *ctx, const char *name, int value);
+int htpops_get_option(htpops_context *ctx, const char *name, int *value);
+
 /* Blocks until everything enqueued on the context's stream has finished. */
 int htpops_synchronize(htpops_context *ctx);
 
@@ -74,7 +91,8 @@ int htpops_buffer_release(htpops_context *ctx, int handle);
  * The context keeps converted copies of WEIGHTS that live in buffers it allocated (made on first use by a matmul,
  * dropped by htpops_buffer_write and by ops that write into the buffer): a caller that rewrites such a buffer through
  * this address must say so with htpops_buffer_invalidate before the next op reads it. Activations, KV rows and
- * outputs need nothing; caller-registered memory is never cached. */
+ * outputs need nothing. Weights in caller-registered memory get no converted copy (they are converted per call or
+ * take the kernels that read them as they are) until the caller asks for one with htpops_buffer_prepare_weights. */
 void  *htpops_buffer_device_ptr(htpops_context *ctx, int handle);
 size_t htpops_buffer_size(htpops_context *ctx, int handle);
 
@@ -82,6 +100,21 @@ size_t htpops_buffer_size(htpops_context *ctx, int handle);
  * are immutable once mapped, src/dsp/op_executor.cc:130): converted weight copies made from it are dropped and
  * recorded messages that use them refuse to launch. Unknown handles return -1. */
 int htpops_buffer_invalidate(htpops_context *ctx, int handle);
+
+/* Makes, now, the converted copy of the weight matrix [n][k/32] (weight_type GGML_TYPE_Q4_0 or GGML_TYPE_Q8_0) at
+ * `offset` of the buffer that matmuls over `m_hint` activation rows will use (none at m_hint = 1; operand-order nibbles
+ * for 2..16 rows; FP6 tiles or int8 fragments from 33 rows), so that the first matmul does not pay for the conversion
+ * and its hipMalloc. The reference maps weights once and treats them as immutable (src/dsp/op_executor.cc:124-130);
+ * this call states the same for the buffer: it is the opt-in that puts CALLER-REGISTERED memory under the contract of
+ * the context's own buffers -- converted copies of its weights are kept from now on (also those that later matmuls at
+ * other row counts make on first use), and the caller says htpops_buffer_invalidate after rewriting it.
+ * *converted_bytes (may be NULL) receives the bytes this call added. */
+int htpops_buffer_prepare_weights(htpops_context *ctx, int handle, size_t offset, int weight_type, int n, int k,
+                                  int m_hint, size_t *converted_bytes);
+
+/* Bytes of converted weight copies the context holds right now / size of its grown-on-demand workspace. */
+size_t htpops_converted_bytes(htpops_context *ctx);
+size_t htpops_workspace_bytes(htpops_context *ctx);
 
 /* Host <-> device copies ordered on the context's stream; both return after the copy is done. */
 int htpops_buffer_write(htpops_context *ctx, int handle, size_t offset, const void *src, size_t bytes);
@@ -178,7 +211,8 @@ int htpops_mat_mul_f32_act_ptr(htpops_context *ctx, float *dst, const float *act
 
 /* simple_flash_attn (src/dsp/ops/flash_attn.c:1368-1420). Q/O [qo_len][n_heads][head_dim] as fp32
  * (qo_is_f32 = 1, the reference op) or fp16; K/V fp16 [kv_len][n_kv_heads][head_dim]; mask fp16
- * [qo_len][align_up(kv_len, 64)] added to the scaled scores, or NULL; causal as in FlashAttnExParams.
+ * [qo_len][align_up(kv_len, 64)] added to the scaled scores (or selecting keys, option "attn_mask_threshold"), or
+ * NULL; causal as in FlashAttnExParams.
  * head_dim: any even value up to 256 (the reference sends head_dim % 64 != 0 to simple_flash_attn_sp_hdim,
  * src/dsp/ops/flash_attn_sp_hdim.c:782-832, and refuses odd values, :785). */
 int htpops_flash_attn_ptr(htpops_context *ctx, void *o, const void *q, const void *k, const void *v,
@@ -196,27 +230,6 @@ int htpops_flash_attn_ptr(htpops_context *ctx, void *o, const void *q, const voi
 int htpops_flash_attn_noalloc_ptr(htpops_context *ctx, void *o, const void *q, const void *k, const void *v,
                                   const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
                                   int qo_is_f32, int causal);
-
-/* ---- measurement helpers (bench harness; no counterpart in the reference) ---- */
-
-/* Records an event on the context's stream / returns elapsed milliseconds between the two most
- * recent start and stop marks after waiting for the stop mark. */
-int htpops_timer_start(htpops_context *ctx);
-int htpops_timer_stop(htpops_context *ctx);
-int htpops_timer_elapsed_ms(htpops_context *ctx, float *ms);
-
-/* Runs `iters` back-to-back v_mfma_i32_32x32x32_i8 (kind 0), v_mfma_i32_16x16x64_i8 (kind 1) or
- * v_mfma_f32_32x32x16_f16 (kind 2) loops on every CU and reports the achieved op rate in Tera-ops/s. */
-int htpops_measure_mfma_peak(htpops_context *ctx, int kind, int iters, double *tera_ops);
-
-/* Plain device-to-device copy kernel (16 B per lane, grid-stride) used to calibrate HBM counters and to
- * measure the attainable copy bandwidth; reports bytes read + written per second in GB/s. */
-int htpops_measure_copy_bandwidth(htpops_context *ctx, size_t bytes, int iters, double *gbps);
-
-/* Time of one launch that reads `bytes` once and keeps nothing (every wave 4 KiB, 16 bytes per lane and load), averaged
- * over `iters` rounds over `buffers` distinct buffers of that size read in turn (buffers x bytes beyond the 256 MB
- * memory-side cache = every launch reads HBM). The floor under any one-launch weight stream of that size. */
-int htpops_measure_read_us(htpops_context *ctx, size_t bytes, int buffers, int iters, double *us_per_launch);
 
 #ifdef __cplusplus
 }

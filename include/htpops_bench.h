@@ -1,0 +1,40 @@
+/*
+ * htpops_bench.h -- timers and calibration kernels of the bench harness.
+ *
+ * Exported by the same shared library as include/htpops.h but not part of the op backend's interface: nothing here
+ * replaces a reference interface, and no op depends on it. bench.py uses these to time the stream the ops are
+ * launched on and to measure the device's own ceilings beside them.
+ */
+#ifndef HTPOPS_BENCH_H
+#define HTPOPS_BENCH_H
+
+#include "htpops.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Records an event on the context's stream / returns elapsed milliseconds between the two most
+ * recent start and stop marks after waiting for the stop mark. */
+int htpops_timer_start(htpops_context *ctx);
+int htpops_timer_stop(htpops_context *ctx);
+int htpops_timer_elapsed_ms(htpops_context *ctx, float *ms);
+
+/* Runs `iters` back-to-back v_mfma_i32_32x32x32_i8 (kind 0), v_mfma_i32_16x16x64_i8 (kind 1) or
+ * v_mfma_f32_32x32x16_f16 (kind 2) loops on every CU and reports the achieved op rate in Tera-ops/s. */
+int htpops_measure_mfma_peak(htpops_context *ctx, int kind, int iters, double *tera_ops);
+
+/* Plain device-to-device copy kernel (16 B per lane, grid-stride) used to calibrate HBM counters and to
+ * measure the attainable copy bandwidth; reports bytes read + written per second in GB/s. */
+int htpops_measure_copy_bandwidth(htpops_context *ctx, size_t bytes, int iters, double *gbps);
+
+/* Time of one launch that reads `bytes` once and keeps nothing (every wave 4 KiB, 16 bytes per lane and load), averaged
+ * over `iters` rounds over `buffers` distinct buffers of that size read in turn (buffers x bytes beyond the 256 MB
+ * memory-side cache = every launch reads HBM). The floor under any one-launch weight stream of that size. */
+int htpops_measure_read_us(htpops_context *ctx, size_t bytes, int buffers, int iters, double *us_per_launch);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* HTPOPS_BENCH_H */

@@ -185,6 +185,18 @@ class Oracle:
             raise ValueError("oracle_flash_attn rejected its arguments")
         return out
 
+    @staticmethod
+    def threshold_mask(mask):
+        """The additive mask that selects the same keys as the kernel the reference dispatches for op 5: that kernel
+        keeps a key iff its fp16 mask value is > -16 and sets the score of every other key to -inf
+        (src/dsp/ops/flash_attn.c:448-460: Q6_Q_vcmp_gt_VhfVhf against 0xcc00, then a mux with -inf); a NaN compares
+        false and is dropped. flash_attn(..., threshold_mask(mask)) is therefore that kernel's rule on top of the
+        scalar routine's arithmetic."""
+        m = np.asarray(mask, dtype=np.float16)
+        with np.errstate(invalid="ignore"):
+            keep = m > np.float16(-16.0)
+        return np.where(keep, np.float16(0.0), np.float16(-np.inf)).astype(np.float16)
+
     # -- fp16 tiles --------------------------------------------------------
     def mat_mul_w16a32(self, act, w_tiles, m, k, n):
         act = np.ascontiguousarray(act, dtype=np.float32)

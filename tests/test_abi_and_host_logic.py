@@ -32,14 +32,14 @@ def ctx(lib):
 
 def test_abi_header_compiles_as_c_and_cxx_with_the_reference_sizes(tmp_path):
     src = tmp_path / "probe.c"
-    src.write_text('#include "htpops.h"\nint main(void){return 0;}\n')
+    src.write_text('#include "htpops.h"\n#include "htpops_bench.h"\nint main(void){return 0;}\n')
     inc = os.path.join(ROOT, "include")
     subprocess.run(["gcc", "-std=c11", "-Wall", "-Werror", "-I", inc, "-c", str(src), "-o", str(tmp_path / "c.o")], check=True)
     subprocess.run(["g++", "-std=c++17", "-Wall", "-I", inc, "-x", "c++", "-c", str(src), "-o", str(tmp_path / "cc.o")], check=True)
 
 
 def test_library_exports_every_symbol_the_header_declares(lib):
-    header = open(os.path.join(ROOT, "include", "htpops.h")).read()
+    header = "".join(open(os.path.join(ROOT, "include", h)).read() for h in ("htpops.h", "htpops_bench.h"))
     declared = sorted(set(re.findall(r"\b(htpops_[a-z0-9_]+)\s*\(", header)))
     assert declared == sorted(api.EXPORTED_SYMBOLS)
     for name in declared:

@@ -21,6 +21,15 @@ def ctx():
     c.close()
 
 
+@pytest.fixture(autouse=True)
+def default_switches(ctx):
+    """Tests that force a kernel or the mask convention do it through htpops_set_option; every test starts from the
+    defaults again."""
+    yield
+    for name, value in api.DEFAULT_OPTIONS.items():
+        ctx.set_option(name, value)
+
+
 CASES = [
     # qo, kv, heads, kv heads, D
     (1, 300, 8, 2, 128), (1, 4096, 32, 8, 128), (1, 70, 4, 4, 64), (1, 129, 16, 1, 128), (1, 1, 4, 2, 64),
@@ -63,10 +72,10 @@ def test_fp16_op_with_causal_flag(ctx, oracle, qo, kv, nh, nkv, d):
 @pytest.mark.parametrize("groups", ["1", "2"])
 @pytest.mark.parametrize("qo,kv,nh,nkv,d", [(40, 300, 4, 1, 128), (33, 517, 4, 4, 128), (64, 96, 2, 1, 64), (70, 200, 8, 2, 128),
                                             (128, 129, 8, 2, 128)])
-def test_prefill_with_one_and_two_key_groups(ctx, oracle, monkeypatch, groups, qo, kv, nh, nkv, d):
+def test_prefill_with_one_and_two_key_groups(ctx, oracle, groups, qo, kv, nh, nkv, d):
     # the prefill kernel runs its KV blocks in one or two key groups per workgroup depending on the grid; both must
     # meet the oracle on every shape (odd block counts leave the second group idle in the last iteration)
-    monkeypatch.setenv("HTPOPS_ATTN_KEY_GROUPS", groups)
+    ctx.set_option("attn_key_groups", int(groups))
     rng = wl.rng_for(63, qo * 1000 + kv + nh)
     q, k, v = wl.make_attention_inputs(rng, qo, kv, nh, nkv, d)
     for causal, mask in ((True, None), (False, wl.make_causal_mask(qo, kv)), (False, None)):

@@ -21,6 +21,14 @@ def ctx():
     c.close()
 
 
+@pytest.fixture(autouse=True)
+def default_switches(ctx):
+    """Tests that force a kernel do it through htpops_set_option; every test starts from the defaults again."""
+    yield
+    for name, value in api.DEFAULT_OPTIONS.items():
+        ctx.set_option(name, value)
+
+
 # ---------------------------------------------------------------------------------------- quantizer
 
 @pytest.mark.parametrize("m,k", [(1, 4096), (8, 4096), (1, 11008), (3, 32), (5, 96), (128, 1536), (512, 4096), (7, 8960)])
@@ -302,7 +310,7 @@ def test_small_batch_repeated_launches_are_bit_identical(ctx):
 @pytest.mark.parametrize("wt,m", [(wl.GGML_TYPE_Q4_0, 2), (wl.GGML_TYPE_Q4_0, 3), (wl.GGML_TYPE_Q8_0, 2), (wl.GGML_TYPE_Q8_0, 3)])
 @pytest.mark.parametrize("k,n", [(64, 1), (128, 33), (1024, 100), (4096, 4096), (4096 + 64, 70), (8192, 9), (11008, 272),
                                  (12288, 64), (2048 + 64, 1000)])
-def test_two_and_three_rows_on_the_decode_kernels_weight_stream(ctx, oracle, monkeypatch, wt, m, k, n):
+def test_two_and_three_rows_on_the_decode_kernels_weight_stream(ctx, oracle, wt, m, k, n):
     # 2 and 3 rows run the decode kernel's stream over the weights with the rows held in registers: one, two or three
     # waves per weight row (k <= 4096, <= 8192, <= 12288), rows past the last whole walk of a workgroup, one lane of a
     # chunk only (k = 4096 + 64). Against the oracle, against the kernels they replace (HTPOPS_GEMV_ROWS_KERNEL=0), bit for bit on a repeat, and
@@ -316,7 +324,7 @@ def test_two_and_three_rows_on_the_decode_kernels_weight_stream(ctx, oracle, mon
     for r in range(m):
         one = ctx.run_mat_mul(a[r:r + 1], w, 1, k, n, wt)[0]
         assert np.all(np.abs(one - got[r]) <= 1e-6 * mag[r]), "row %d differs from the one-row kernel" % r
-    monkeypatch.setenv("HTPOPS_GEMV_ROWS_KERNEL", "0")
+    ctx.set_option("gemv_rows_kernel", 0)
     other = ctx.run_mat_mul(a, w, m, k, n, wt)
     assert np.all(np.abs(other - got) <= 2 * MATMUL_RTOL * mag)
 
@@ -366,13 +374,13 @@ def test_gemm_mfma_integer_exact(ctx, wt):
 
 @pytest.mark.parametrize("wt", [wl.GGML_TYPE_Q4_0, wl.GGML_TYPE_Q8_0])
 @pytest.mark.parametrize("m,k,n", [(128, 1536, 256), (129, 320, 65), (100, 11008, 96), (33, 2048, 70), (256, 4096, 512)])
-def test_gemm_mfma_with_small_and_large_tiles(ctx, oracle, monkeypatch, wt, m, k, n):
+def test_gemm_mfma_with_small_and_large_tiles(ctx, oracle, wt, m, k, n):
     # launches with few output tiles run 32 x 32 tiles per workgroup, the others 64 x 64 (HTPOPS_GEMM_TILE_UNITS forces
     # one or the other): both must meet the oracle on the same inputs
-    monkeypatch.setenv("HTPOPS_GEMM_FP6", "0")
+    ctx.set_option("gemm_fp6", 0)
     got = {}
     for units in ("1", "2"):
-        monkeypatch.setenv("HTPOPS_GEMM_TILE_UNITS", units)
+        ctx.set_option("gemm_tile_units", int(units))
         got[units], _, _ = check_mat_mul(ctx, oracle, wl.rng_for(58, m * 131 + k + n + wt), m, k, n, wt)
     scale = np.abs(got["1"]).max()
     assert np.abs(got["1"] - got["2"]).max() <= 2e-5 * scale
@@ -433,7 +441,7 @@ def test_message_shares_one_activation_conversion_between_many_row_matmuls(ctx, 
 @pytest.mark.parametrize("m,k,n", [(2, 256, 16), (8, 256, 48), (3, 512, 4096), (8, 4096, 4096), (5, 11008, 272), (8, 2048 + 256, 1024),
                                    (7, 8960, 1536), (9, 256, 32), (16, 4096, 4096), (12, 2048 + 256, 1040), (13, 8192, 48),
                                    (16, 8960, 64), (11, 11008, 64)])
-def test_few_rows_over_repacked_weights(ctx, oracle, monkeypatch, wt, m, k, n):
+def test_few_rows_over_repacked_weights(ctx, oracle, wt, m, k, n):
     # 2..16 rows against Q4_0 or Q8_0 weights with n % 16 == 0, k % 256 == 0 run on a copy of the weights repacked into
     # matrix-core operand order (9..16 rows only while 16 activation rows fit the LDS panel: k = 8960 does not,
     # nor 11008; they take the K-sliced kernel). It must meet the oracle, agree with the kernels that read the weights as they are
@@ -446,11 +454,11 @@ def test_few_rows_over_repacked_weights(ctx, oracle, monkeypatch, wt, m, k, n):
     # one and two weight tiles per workgroup (the launcher picks by the number of tiles; HTPOPS_LANE_ORDER=2 / 3 force
     # one / two) sum the same blocks in different wave order
     for tiles in ("2", "3"):
-        monkeypatch.setenv("HTPOPS_LANE_ORDER", tiles)
+        ctx.set_option("lane_order", int(tiles))
         forced = ctx.run_mat_mul(a, w, m, k, n, wt)
         assert np.all(np.abs(forced - got) <= 2 * MATMUL_RTOL * mag)
         assert np.array_equal(forced, ctx.run_mat_mul(a, w, m, k, n, wt))
-    monkeypatch.setenv("HTPOPS_LANE_ORDER", "0")
+    ctx.set_option("lane_order", 0)
     plain = ctx.run_mat_mul(a, w, m, k, n, wt)
     assert np.all(np.abs(plain - got) <= 2 * MATMUL_RTOL * mag)
 
@@ -488,9 +496,9 @@ def test_few_rows_repacked_weights_extremes_and_cache(ctx, oracle):
 
 
 @pytest.fixture
-def fp6_kernel(monkeypatch):
+def fp6_kernel(ctx):
     """Forces the FP6 many-row kernel (by default it only takes shapes that fill the device with whole tiles)."""
-    monkeypatch.setenv("HTPOPS_GEMM_FP6", "1")
+    ctx.set_option("gemm_fp6", 1)
 
 
 # ragged rows / columns / odd K-block counts; one tile shared by many workgroups (k = 4128, 11008); several tiles per
@@ -798,7 +806,7 @@ def test_message_groups_many_row_matmuls_over_the_same_rows(ctx, oracle):
     # weights live in buffers of the context share the launch of the FP6-tile kernel (one grid keeps the compute units
     # fed to the end). Every request must equal its own launch bit for bit; one that reads other rows starts a new launch.
     wt, op = wl.GGML_TYPE_Q4_0, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0
-    fp6 = os.environ.get("HTPOPS_GEMM_FP6", "-1") != "0"   # (switched off, every request is a launch of the int8 kernel)
+    fp6 = ctx.get_option("gemm_fp6") != 0   # (switched off, every request is a launch of the int8 kernel)
     rng = wl.rng_for(81, 0)
     m, k = 512, 1024
     ns = [4096, 3072, 6144, 3072]

@@ -167,3 +167,28 @@ def test_w16_tile_layout_and_matmul(oracle):
     got = oracle.mat_mul_w16a32(act, tiles, m, k, n)
     want = act.astype(np.float64) @ w.astype(np.float64)
     assert np.abs(got - want).max() < 1e-4
+
+
+def test_threshold_mask_follows_the_dispatched_kernels_rule(oracle):
+    # src/dsp/ops/flash_attn.c:452-455: keep iff mask > -16.0 in fp16 (0xcc00); equality, anything below, and NaN
+    # (an ordered compare is false) are dropped; 0, positive biases, +inf and -15.99 (rounds to an fp16 above -16) stay
+    vals = np.array([0.0, -15.99, -16.0, -16.02, -1e4, -np.inf, 3.0, np.inf, np.nan, -0.0], np.float16)
+    got = oracle.threshold_mask(vals)
+    want = np.array([0, 0, -np.inf, -np.inf, -np.inf, -np.inf, 0, 0, -np.inf, 0], np.float16)
+    assert np.array_equal(got, want)
+    assert vals[1] > np.float16(-16) and vals[3] < np.float16(-16)
+    # on a 0 / -inf mask the two conventions are the same function (the survey's "identical for 0 / -inf")
+    rng = np.random.default_rng(5)
+    q = rng.standard_normal((3, 2, 64)).astype(np.float32)
+    k = rng.standard_normal((70, 1, 64)).astype(np.float16)
+    v = rng.standard_normal((70, 1, 64)).astype(np.float16)
+    mask = np.where(rng.random((3, 128)) < 0.3, -np.inf, 0.0).astype(np.float16)
+    mask[:, 0] = 0
+    a = oracle.flash_attn(q, k, v, mask, 2, 1, 64)
+    b = oracle.flash_attn(q, k, v, oracle.threshold_mask(mask), 2, 1, 64)
+    assert np.array_equal(a, b)
+    # with finite biases they differ: a bias of -3 lowers a key's weight when added and leaves it alone when it selects
+    biased = np.zeros((3, 128), np.float16)
+    biased[:, 5] = -3.0
+    assert np.abs(oracle.flash_attn(q, k, v, biased, 2, 1, 64) - oracle.flash_attn(q, k, v, oracle.threshold_mask(biased), 2, 1, 64)).max() > 1e-3
+    assert np.array_equal(oracle.flash_attn(q, k, v, oracle.threshold_mask(biased), 2, 1, 64), oracle.flash_attn(q, k, v, None, 2, 1, 64))
