@@ -17,6 +17,12 @@ namespace {
 // that hipGetSymbolAddress returned for the context's device (htpops_context::scratch_ptr), never the name.
 static __device__ __align__(256) unsigned char scratch[htpops::host::kNoAllocScratchBytes];
 
+// Which context's work may be using a device's copy of the array: all contexts on a GPU share it, and two streams
+// writing partials into it at once would race. A context claims the array with its first call of the entry point and
+// gives it back when it has waited for its stream (htpops_synchronize, htpops_finish_message, htpops_close).
+constexpr int kMaxDevices = 64;
+std::atomic<htpops_context *> scratch_owner[kMaxDevices];
+
 struct OptionName {
   const char *name;
   int htpops::host::Options::*field;
@@ -78,6 +84,21 @@ int need_device(htpops_context *ctx) {
     return fail(ctx, HTPOPS_ERR_NO_DEVICE, "context was created without a GPU; compute ops are unavailable");
   }
   return HTPOPS_OK;
+}
+
+bool claim_static_scratch(htpops_context *ctx) {
+  if (ctx->device < 0 || ctx->device >= kMaxDevices) {
+    return false;
+  }
+  htpops_context *expected = nullptr;
+  return scratch_owner[ctx->device].compare_exchange_strong(expected, ctx) || expected == ctx;
+}
+
+void release_static_scratch(htpops_context *ctx) {
+  if (ctx->device >= 0 && ctx->device < kMaxDevices) {
+    htpops_context *expected = ctx;
+    scratch_owner[ctx->device].compare_exchange_strong(expected, nullptr);
+  }
 }
 
 bool mul3(size_t a, size_t b, size_t c, size_t *out) {
@@ -155,6 +176,7 @@ extern "C" int htpops_close(htpops_context *ctx) {
   if (ctx->has_device) {
     (void) hipSetDevice(ctx->device);
     (void) hipStreamSynchronize(ctx->stream);
+    release_static_scratch(ctx);
   }
   for (htpops_recorded_message *rec : ctx->recordings) {  // recordings the caller did not release
     if (rec->exec) {
@@ -242,6 +264,7 @@ extern "C" int htpops_synchronize(htpops_context *ctx) {
     return HTPOPS_OK;
   }
   HTPOPS_HIP(ctx, hipStreamSynchronize(ctx->stream));
+  release_static_scratch(ctx);  // (nothing of this context is in flight: another context may take the static scratch)
   return HTPOPS_OK;
 }
 

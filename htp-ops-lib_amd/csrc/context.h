@@ -164,6 +164,10 @@ int hip_fail(htpops_context *ctx, hipError_t e, const char *what);
   } while (0)
 
 int need_device(htpops_context *ctx);
+// The static device array of the entry point that allocates nothing is shared by the contexts of a GPU: true when
+// `ctx` holds it (or has just taken it), false while another context that has not yet waited for its stream does.
+bool claim_static_scratch(htpops_context *ctx);
+void release_static_scratch(htpops_context *ctx);
 
 // ---- small helpers ----
 inline bool aligned(const void *p, size_t a) {

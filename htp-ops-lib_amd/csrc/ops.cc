@@ -390,6 +390,11 @@ int op_flash_attn(htpops_context *ctx, void *o, const void *q, const void *k, co
     if (ctx->act_fragments.src && ranges_overlap(o, o_bytes, ctx->act_fragments.src, ctx->act_fragments.src_bytes)) {
       ctx->act_fragments.src = nullptr;
     }
+    if (ws_bytes > 0 && !claim_static_scratch(ctx)) {
+      return fail(ctx, HTPOPS_ERR_BUSY,
+                  "flash_attn (no allocation): another context on this GPU is using the static scratch and has not "
+                  "synchronized since");
+    }
     ws = ctx->scratch_ptr;
   } else {
     if (int r = ensure_workspace(ctx, ws_bytes)) {

@@ -225,8 +225,10 @@ int htpops_flash_attn_ptr(htpops_context *ctx, void *o, const void *q, const voi
  * inside the library instead of the context's grown-on-demand workspace, and the call performs no hipMalloc / hipFree
  * of any kind. Limit: n_heads * ceil(kv_len / 64) * (head_dim + 2) * 4 bytes <= 8 MiB (e.g. 32 heads of 128 up to
  * kv_len 32256); larger requests, and outputs that overlap weights the context holds a converted copy of, return -1
- * with a message. All contexts on one GPU share the array, and it keeps the last call's contents: calls that overlap
- * in time on one GPU (two contexts, i.e. two streams) race; calls on one context are ordered by its stream. */
+ * with a message. All contexts on one GPU share the array, and it keeps the last call's contents: calls on one
+ * context are ordered by its stream; a context that calls this while ANOTHER context's calls may still be running
+ * (that context has not been through htpops_synchronize, htpops_finish_message or htpops_close since its last such
+ * call) gets HTPOPS_ERR_BUSY instead of a race. */
 int htpops_flash_attn_noalloc_ptr(htpops_context *ctx, void *o, const void *q, const void *k, const void *v,
                                   const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
                                   int qo_is_f32, int causal);

@@ -180,3 +180,34 @@ def test_rejections(ctx):
     p = api.flash_attn_params((q, 0), (q, 0), (k, 0), (k, 0), (-1, 0), 1, 4096, 8, 2, 128)
     assert ctx.execute(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16, p) == R     # K/V buffer too small
     ctx.release(q), ctx.release(k)
+
+
+@pytest.mark.parametrize("qo,kv,nh,nkv,d", [(1, 300, 8, 2, 128), (1, 4096, 32, 8, 128), (40, 300, 4, 1, 128), (5, 70, 4, 2, 64),
+                                            (3, 130, 2, 1, 80), (70, 200, 8, 2, 128)])
+def test_mask_selects_keys_when_the_threshold_option_is_set(ctx, oracle, qo, kv, nh, nkv, d):
+    # The kernel the reference dispatches for op 5 keeps a key iff mask > -16 (src/dsp/ops/flash_attn.c:448-460); its
+    # scalar routine adds the mask (:1505-1512). The default here is the additive convention; with the option
+    # "attn_mask_threshold" the same op selects keys. A mask with finite biases on both sides of -16, exact -16, -inf and
+    # NaN tells the two apart; each mode is checked against the oracle under its own convention.
+    rng = wl.rng_for(64, qo * 1000 + kv + nh)
+    q, k, v = wl.make_attention_inputs(rng, qo, kv, nh, nkv, d)
+    q = q.astype(np.float32)  # the reference op (id 5): fp32 Q / O
+    ld = (kv + 63) // 64 * 64
+    values = np.array([0.0, 0.0, 0.0, -3.0, -15.5, -16.0, -17.0, -40.0, -np.inf, 2.0], np.float16)
+    mask = values[rng.integers(0, len(values), size=(qo, ld))]
+    mask[:, 0] = 0
+    additive = ctx.run_flash_attn(q, k, v, mask, nh, nkv, d)
+    assert np.abs(additive - oracle.flash_attn(q, k, v, mask, nh, nkv, d)).max() <= ATOL
+    with_nan = mask.copy()
+    with_nan[:, 1] = np.nan  # dropped by the selecting convention (an ordered compare), poison for the additive one
+    ctx.set_option("attn_mask_threshold", 1)
+    selecting = ctx.run_flash_attn(q, k, v, with_nan, nh, nkv, d)
+    want = oracle.flash_attn(q, k, v, oracle.threshold_mask(with_nan), nh, nkv, d)
+    assert np.all(np.isfinite(selecting))
+    assert np.abs(selecting - want).max() <= ATOL
+    assert np.abs(selecting - additive).max() > 10 * ATOL  # (the two conventions really differ on this mask)
+    # 0 / -inf masks: the same answer either way
+    plain = np.where(mask > np.float16(-16), np.float16(0), np.float16(-np.inf)).astype(np.float16)
+    a = ctx.run_flash_attn(q, k, v, plain, nh, nkv, d)
+    ctx.set_option("attn_mask_threshold", 0)
+    assert np.array_equal(a, ctx.run_flash_attn(q, k, v, plain, nh, nkv, d))

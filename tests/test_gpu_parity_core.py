@@ -1124,3 +1124,105 @@ def test_a_failed_device_allocation_is_reported_and_the_context_stays_usable(ctx
         assert np.all(np.abs(got - want) <= MATMUL_RTOL * mag)
     finally:
         ctx.release(h)
+
+
+def test_registered_weights_take_the_fast_kernels_once_prepared(ctx, oracle):
+    # Weights in memory the context does not own (a framework's tensor, here a buffer of a second context registered by
+    # address) get no converted copy on their own: nothing tells the context when they change. htpops_buffer_prepare_weights
+    # is the opt-in (the reference maps weights once and treats them as immutable, src/dsp/op_executor.cc:124-130): it
+    # makes the copy now, and from then on the buffer is treated like one of the context's own, htpops_buffer_invalidate
+    # included. Same kernel = same bits as the owned-buffer run (the kernels that read the weights as they are sum in
+    # another order).
+    wt, op = wl.GGML_TYPE_Q4_0, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0
+    rng = wl.rng_for(95, 0)
+    k, n = 1024, 3072
+    w = wl.make_q4_0_weights(rng, n, k)
+    acts = {m: oracle.quantize_q8_0(wl.make_activations(rng, m, k)) for m in (8, 512)}
+    with api.Context(device=0) as owner:
+        theirs = owner.upload(w)
+        ours = ctx.upload(w)
+        alias = ctx.register(owner.device_ptr(theirs), w.nbytes)
+        h_act = {m: ctx.upload(a) for m, a in acts.items()}
+        h_out = {m: ctx.alloc(m * n * 4) for m in acts}
+
+        def run(hw, m):
+            msg = api.build_message([(api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(
+                op, api.mat_mul_params((h_out[m], 0), (h_act[m], 0), (hw, 0), m, k, n)))])
+            assert ctx.process_message(msg) == 0 and api.message_request_states(msg) == [0], ctx.last_error()
+            assert ctx.last_message_submissions() == 1
+            return ctx.read(h_out[m], np.float32, m * n).reshape(m, n)
+
+        def check(got, m, weights):
+            cols = np.unique(np.linspace(0, n - 1, 40).astype(int))
+            rows = np.arange(m) if m <= 8 else np.array([0, 1, 31, 32, 127, 128, 300, 511])
+            want, mag = oracle.mat_mul_q8_0_act_f64(acts[m][rows], weights[cols], len(rows), k, len(cols), wt)
+            assert np.all(np.abs(got[np.ix_(rows, cols)] - want) <= MATMUL_RTOL * mag)
+
+        try:
+            base = ctx.converted_bytes()
+            owned = {m: run(ours, m) for m in (8, 512)}   # repacked-weight kernel / FP6-tile kernel over cached copies
+            owned_bytes = ctx.converted_bytes() - base
+            assert owned_bytes >= 2 * w.nbytes             # operand-order nibbles (1 x) + FP6 tiles (1.78 x)
+            for m in (8, 512):
+                check(owned[m], m, w)
+            # before the opt-in: right answers, nothing kept
+            before = ctx.converted_bytes()
+            for m in (8, 512):
+                check(run(alias, m), m, w)
+            assert ctx.converted_bytes() == before
+            # the opt-in, one row count at a time
+            added8 = ctx.prepare_weights(alias, wt, n, k, 8)
+            assert added8 == w.nbytes and ctx.converted_bytes() == before + added8
+            assert ctx.prepare_weights(alias, wt, n, k, 8) == 0          # already there
+            assert np.array_equal(run(alias, 8), owned[8])
+            added512 = ctx.prepare_weights(alias, wt, n, k, 512)
+            assert added8 + added512 == owned_bytes
+            assert np.array_equal(run(alias, 512), owned[512])
+            assert ctx.converted_bytes() == before + owned_bytes          # the matmuls made nothing more
+            # the owner rewrites its memory and says so: the copies go, the next matmuls see the new weights and, the
+            # buffer staying under the contract, keep new copies
+            w2 = wl.make_q4_0_weights(rng, n, k)
+            owner.write(theirs, w2)
+            assert ctx.invalidate(alias) == 0
+            assert ctx.converted_bytes() == before
+            for m in (8, 512):
+                check(run(alias, m), m, w2)
+            assert ctx.converted_bytes() == before + owned_bytes
+            # bad arguments
+            assert ctx.lib.htpops_buffer_prepare_weights(ctx._ctx, alias, 0, wt, n, k + 32, 8, None) == api.HTPOPS_ERR_REJECTED
+            assert ctx.lib.htpops_buffer_prepare_weights(ctx._ctx, 12345, 0, wt, n, k, 8, None) == api.HTPOPS_ERR_REJECTED
+            assert ctx.lib.htpops_buffer_prepare_weights(ctx._ctx, alias, 0, 3, n, k, 8, None) == api.HTPOPS_ERR_REJECTED
+        finally:
+            for h in [alias, ours] + list(h_act.values()) + list(h_out.values()):
+                ctx.release(h)
+            owner.release(theirs)
+
+
+def test_converted_copies_stay_under_the_cap(ctx, oracle):
+    # With "converted_cap_mib" set, the least recently used converted copies are evicted when a new one would pass the
+    # cap; results do not change, and a copy that went is simply made again.
+    wt, op = wl.GGML_TYPE_Q4_0, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0
+    rng = wl.rng_for(96, 0)
+    m, k, n = 8, 2048, 4096                       # 4.5 MiB of weights each, the same again as a repacked copy
+    ws = [wl.make_q4_0_weights(rng, n, k) for _ in range(3)]
+    a = oracle.quantize_q8_0(wl.make_activations(rng, m, k))
+    hws, ha, ho = [ctx.upload(w) for w in ws], ctx.upload(a), ctx.alloc(m * n * 4)
+    try:
+        base = ctx.converted_bytes()
+        ctx.set_option("converted_cap_mib", (base >> 20) + 10)   # room for two copies, not three
+
+        def run(i):
+            assert ctx.execute(op, api.mat_mul_params((ho, 0), (ha, 0), (hws[i], 0), m, k, n)) == 0
+            ctx.synchronize()
+            return ctx.read(ho, np.float32, m * n).reshape(m, n)
+        first = [run(i) for i in range(3)]
+        assert ctx.converted_bytes() - base == 2 * ws[0].nbytes   # the copy of weights 0 went when weights 2 came
+        for i in (0, 1, 2, 0):
+            assert np.array_equal(run(i), first[i])
+            assert ctx.converted_bytes() - base <= 2 * ws[0].nbytes
+        cols = np.unique(np.linspace(0, n - 1, 32).astype(int))
+        want, mag = oracle.mat_mul_q8_0_act_f64(a, ws[2][cols], m, k, len(cols), wt)
+        assert np.all(np.abs(first[2][:, cols] - want) <= MATMUL_RTOL * mag)
+    finally:
+        for h in hws + [ha, ho]:
+            ctx.release(h)

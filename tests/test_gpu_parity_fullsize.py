@@ -120,3 +120,122 @@ def test_qwen2_q8_0_block_message_at_full_size(ctx, oracle, m):
             2: oracle.quantize_q8_0(wl.make_activations(rng, m, 1536)), 3: oracle.quantize_q8_0(wl.make_activations(rng, m, 8960))}
     act_rows = None if m <= 8 else np.array([0, 1, 31, 32, 63, 64, 100, 126, 127])
     run_layer_message(ctx, oracle, wl.QWEN2_1P5B_LAYER, weights, acts, m, Q8, act_rows, launches=1)
+
+
+ATTN_ATOL = 2e-3
+
+
+@pytest.mark.parametrize("qo,kv", [(2048, 2048), (1, 4096), (1, 16384)])
+def test_attention_at_full_size_against_the_oracle_on_sampled_rows(ctx, oracle, qo, kv):
+    # config 3 (32 query / 8 KV heads of 128, fp16, causal): the kernel the benchmark times, against the oracle's scalar
+    # attention for sampled query rows -- both ends, both sides of a 32-row tile edge, the middle, and the whole last
+    # tile -- every head. The oracle gets the sampled rows with their rows of the causal mask written out (0 on and
+    # below the diagonal, -inf above: the convention both reference variants agree on, flash_attn.c:452-455 / :1505-1512).
+    nh, nkv, hd = 32, 8, 128
+    rng = wl.rng_for(3, qo * 7 + kv)
+    q, k, v = wl.make_attention_inputs(rng, qo, kv, nh, nkv, hd)
+    print("full-size attention qo=%d kv=%d" % (qo, kv), flush=True)
+    got = ctx.run_flash_attn(q, k, v, None, nh, nkv, hd, causal=True)
+    rows = np.array(sorted({0, 31, 32, qo // 2 - 1, qo // 2} | set(range(max(0, qo - 32), qo)))) if qo > 1 else np.array([0])
+    rows = rows[rows >= 0]
+    ld = (kv + 63) // 64 * 64
+    mask = np.full((len(rows), ld), -np.inf, np.float16)
+    for i, r in enumerate(rows):
+        mask[i, :r + (kv - qo) + 1] = 0
+    want = oracle.flash_attn(np.ascontiguousarray(q[rows]), k, v, mask, nh, nkv, hd, False)
+    err = np.abs(got[rows].astype(np.float32) - want.astype(np.float32)).max()
+    assert err <= ATTN_ATOL, err
+    # the reference op (id 5: fp32 Q / O, the mask as a buffer) on the same rows gives the same values
+    got32 = ctx.run_flash_attn(np.ascontiguousarray(q[rows]).astype(np.float32), k, v, mask, nh, nkv, hd)
+    assert np.abs(got32 - want.astype(np.float32)).max() <= ATTN_ATOL
+
+
+def test_decoder_layer_for_one_token_as_one_message(ctx, oracle, llama_weights):
+    # The twelve requests of a Llama-7B-like layer for one token, as ONE message: RMSNorm+Q8_0 -> q, k, v -> attention
+    # over 4096 cached keys -> Q8_0 -> o -> RMSNorm+Q8_0 -> gate, up -> Q8_0 -> down. The walk fuses and groups them
+    # into 6 submissions; every buffer the message writes must hold, byte for byte, what the same requests give when
+    # each is sent as a message of its own (12 submissions: the reference's one-op-per-request order,
+    # src/dsp/commu.c:91-114), and every stage must meet the oracle applied to the stage's own input.
+    nh, nkv, hd, kv = 32, 8, 128, 4096
+    rng = wl.rng_for(6, 1)
+    shapes = {name: (n, k) for name, n, k in wl.LLAMA7B_LAYER}
+    _, kk, vv = wl.make_attention_inputs(rng, 1, kv, nh, nkv, hd)
+    x = wl.make_activations(rng, 1, 4096)
+    g = (1 + 0.1 * rng.standard_normal(4096)).astype(np.float32)
+    hidden = wl.make_activations(rng, 1, 11008)
+    h_w = {name: ctx.upload(llama_weights[shapes[name]]) for name in shapes}
+    hx, hg, hh, hk, hv = ctx.upload(x), ctx.upload(g), ctx.upload(hidden), ctx.upload(kk), ctx.upload(vv)
+    sizes = {"qa": 4096 // 32 * 34, "qo": 4096 // 32 * 34, "qb": 4096 // 32 * 34, "qd": 11008 // 32 * 34, "attn": 4096 * 4}
+    sizes.update({name: shapes[name][0] * 4 for name in shapes})
+
+    def build(bufs):
+        def op(code, payload):
+            return (api.REQUEST_TYPE_OP_COMPUTE, api.op_compute_request(code, payload))
+
+        def mm(name, act):
+            n, k = shapes[name]
+            return op(api.HTP_OPS_MAT_MUL_Q4_0_Q8_0, api.mat_mul_params((bufs[name], 0), (bufs[act], 0), (h_w[name], 0), 1, k, n))
+        return [
+            op(api.HTP_OPS_RMS_NORM_QUANTIZE_Q8_0, api.rms_norm_ex_params((bufs["qa"], 0), (hx, 0), (hg, 0), 4096, 1, 1e-6)),
+            mm("q", "qa"), mm("k", "qa"), mm("v", "qa"),
+            op(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16,
+               api.flash_attn_params((bufs["attn"], 0), (bufs["q"], 0), (hk, 0), (hv, 0), (-1, 0), 1, kv, nh, nkv, hd)),
+            op(api.HTP_OPS_QUANTIZE_Q8_0, api.rms_norm_params((bufs["qo"], 0), (bufs["attn"], 0), 4096, 1)),
+            mm("o", "qo"),
+            op(api.HTP_OPS_RMS_NORM_QUANTIZE_Q8_0, api.rms_norm_ex_params((bufs["qb"], 0), (bufs["o"], 0), (hg, 0), 4096, 1, 1e-6)),
+            mm("gate", "qb"), mm("up", "qb"),
+            op(api.HTP_OPS_QUANTIZE_Q8_0, api.rms_norm_params((bufs["qd"], 0), (hh, 0), 11008, 1)),
+            mm("down", "qd")]
+
+    sets = [{name: ctx.alloc(nbytes) for name, nbytes in sizes.items()} for _ in range(2)]
+    try:
+        for bufs in sets:
+            for name, nbytes in sizes.items():
+                ctx.write(bufs[name], np.full(nbytes, 0xA5, np.uint8))
+        print("decoder layer: twelve requests in one message", flush=True)
+        msg = api.build_message(build(sets[0]))
+        assert ctx.process_message(msg) == 0 and api.message_request_states(msg) == [0] * 12, ctx.last_error()
+        assert ctx.last_message_submissions() == 6
+        print("decoder layer: one message per request", flush=True)
+        for req in build(sets[1]):
+            one = api.build_message([req])
+            assert ctx.process_message(one) == 0 and api.message_request_states(one) == [0], ctx.last_error()
+        out = [{name: ctx.read(bufs[name], np.uint8, nbytes) for name, nbytes in sizes.items()} for bufs in sets]
+        for name in sizes:
+            assert np.array_equal(out[0][name], out[1][name]), "%s differs between the one message and the twelve" % name
+        o = out[0]
+        f32 = {name: o[name].view(np.float32) for name in list(shapes) + ["attn"]}
+
+        def check_matmul(name, act):
+            n, k = shapes[name]
+            want, mag = oracle.mat_mul_q8_0_act_f64(o[act].reshape(1, -1), llama_weights[(n, k)], 1, k, n, Q4)
+            assert np.all(np.abs(f32[name] - want[0]) <= MATMUL_RTOL * mag[0]), name
+
+        def check_norm_row(name, src_row):
+            # RMSNorm is held to 2e-3, so its Q8_0 row is: the oracle's quantizer applied to some row within 2e-3 of
+            # the oracle's normalized row -- every dequantized value within half a quantization step plus 2e-3 of it
+            normed = oracle.rms_norm(src_row.reshape(1, -1), g, 1e-6)[0]
+            blocks = o[name].reshape(-1, 34)
+            d = blocks[:, :2].copy().view(np.float16).astype(np.float32)
+            deq = (blocks[:, 2:].view(np.int8).astype(np.float32) * d).reshape(-1)
+            step = np.repeat(d[:, 0], 32)
+            assert np.all(np.abs(deq - normed) <= 0.5 * step * 1.002 + 2e-3), name
+
+        check_norm_row("qa", x[0])
+        for name in ("q", "k", "v"):
+            check_matmul(name, "qa")
+        want_attn = oracle.flash_attn(f32["q"].reshape(1, nh, hd), kk, vv, None, nh, nkv, hd)
+        assert np.abs(f32["attn"] - want_attn.reshape(-1)).max() <= ATTN_ATOL
+        assert np.array_equal(o["qo"], oracle.quantize_q8_0(f32["attn"].reshape(1, -1)).reshape(-1))
+        check_matmul("o", "qo")
+        check_norm_row("qb", f32["o"])
+        check_matmul("gate", "qb")
+        check_matmul("up", "qb")
+        assert np.array_equal(o["qd"], oracle.quantize_q8_0(hidden).reshape(-1))
+        check_matmul("down", "qd")
+    finally:
+        for bufs in sets:
+            for h in bufs.values():
+                ctx.release(h)
+        for h in list(h_w.values()) + [hx, hg, hh, hk, hv]:
+            ctx.release(h)
