@@ -54,14 +54,22 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def measured_traffic(launch):
+def measured_traffic(launch, timed_launch, timed_submissions):
     """HBM-side bytes per launch of the named launch, from hardware counters collected in separate profiler passes
     over this script (FETCH_SIZE and WRITE_SIZE, each scaled by the same counter's reading for the plain copy
-    kernel of known size); the figures live beside the package because counters cannot be read from inside a run."""
+    kernel of known size); the figures live beside the package because counters cannot be read from inside a run.
+    Each figure is kept with the kernel instance and grid it was profiled on and the number of launches its message
+    became: when the launch timed in this run is another one (the kernel or its launch geometry changed since the
+    profile), the figure does not describe it and None is returned."""
     path = os.path.join(ROOT, "htp-ops-lib_amd", "pyhtpops", "measured_traffic.json")
     try:
         with open(path) as f:
-            return json.load(f)["launches"][launch]["traffic_bytes"]
+            entry = json.load(f)["launches"][launch]
+        if entry.get("launch") != timed_launch or entry.get("submissions") != timed_submissions:
+            log("measured_traffic: profiled on %r (%r launches), timed %r (%r): traffic left out" % (
+                entry.get("launch"), entry.get("submissions"), timed_launch, timed_submissions))
+            return None
+        return entry["traffic_bytes"]
     except (OSError, KeyError, ValueError):
         return None
 
@@ -208,13 +216,19 @@ def main():
         return ev_ms / steps
 
     ms_step, wall_step = time_layers(1, args.steps, args.warmup)
+    step_launch = ctx.last_gemv_launch()   # kernel instance and grid of the launch just timed
     value = layer_bytes[1] / (ms_step * 1e-3) / 1e9
     log("layer m=1: %.2f us/step (events) %.2f us/step (wall)  %.0f GB/s (%.1f%% of 8 TB/s)" % (
         ms_step * 1e3, wall_step * 1e3, value, value / 80))
     if args.only_step:
         ctx.close()
-        print(json.dumps({"metric": "layer step only", "value": round(value, 1), "unit": "GB/s", "ms_per_step": round(ms_step, 6)}))
+        print(json.dumps({"metric": "layer step only", "value": round(value, 1), "unit": "GB/s", "ms_per_step": round(ms_step, 6),
+                          "launch": step_launch, "submissions": subs1}))
         return
+    # host side of a step: the message walk (validation, handle lookups, batching, one hipLaunchKernel) timed on the
+    # host clock while the stream has a backlog
+    host_walk_us = ctx.measure_host_walk_us(layer_message(0, 1), 2000)
+    log("host walk of the layer message: %.2f us per message (GPU time per message %.2f us)" % (host_walk_us, ms_step * 1e3))
     block_us = [time_layers(1, 40, LAYERS)[0] * 1e3 for _ in range(20)]
     step_stats = percentiles(block_us)
     log("layer m=1 over 20 blocks of 40 steps: median %.2f us  p10 %.2f  p90 %.2f" % (
@@ -288,6 +302,9 @@ def main():
     prefill = []
     rng2 = wl.rng_for(2, 0)
     prefill_inputs = {}
+    # weights that this context does not own: buffers of a second context on the same GPU
+    other = api.Context(device=0)
+    other_ctx_weights = {(n, k): (other, other.upload(uniq[(n, k)])) for (n, k) in ((11008, 4096), (4096, 11008))}
     for (n, k) in ((11008, 4096), (4096, 11008)):
         m = 512
         x = wl.make_activations(rng2, m, k)
@@ -306,6 +323,19 @@ def main():
         hw = layers[0][4] if (n, k) == (11008, 4096) else layers[0][6]
         us = time_single(n, k, m, Q4, [hw] * 8, ha, ho, 10, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)  # 8 launches per message share the re-tiled activations
         us_alone = time_single(n, k, m, Q4, [hw], ha, ho, 20, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)  # re-tiling + one launch
+        # the same weights as caller-owned memory (registered by address, as a framework hands over its tensors):
+        # prepared once (htpops_buffer_prepare_weights), then the same kernel over the kept copy
+        h_reg = ctx.register(other.device_ptr(other_ctx_weights[(n, k)][1]), uniq[(n, k)].nbytes)
+        ctx.synchronize()
+        t_prep = time.perf_counter()
+        prep_bytes = ctx.prepare_weights(h_reg, Q4, n, k, m)
+        ctx.synchronize()
+        prep_us = (time.perf_counter() - t_prep) * 1e6
+        us_registered = time_single(n, k, m, Q4, [h_reg] * 8, ha, ho, 10, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)
+        got_reg = ctx.read(ho, np.float32, m * n)
+        us = time_single(n, k, m, Q4, [hw] * 8, ha, ho, 10, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0)
+        assert np.array_equal(got_reg, ctx.read(ho, np.float32, m * n)), "registered weights give other bits than owned ones"
+        ctx.release(h_reg)
         # independent matmuls over the same rows (q/k/v, gate/up of a prefill chunk: distinct weights, distinct outputs)
         # share a launch: three and eight per message
         idx = 4 if (n, k) == (11008, 4096) else 6
@@ -343,6 +373,12 @@ def main():
                         "us_per_matmul_8_in_one_message": round(grouped[8], 2),
                         "tera_ops_8_in_one_message": round(2.0 * m * n * k / grouped[8] / 1e6, 1),
                         "us_with_activation_retiling": round(us_alone, 2),
+                        "us_registered_weights": round(us_registered, 2),
+                        "prepare_registered_weights_us": round(prep_us, 1), "prepared_copy_bytes": prep_bytes,
+                        # per 32 x 32 x 32 block the format needs, besides the block-sum instruction, one scale-product
+                        # matrix instruction and 16 fp32 multiply-adds that no matrix instruction can do: measured with
+                        # every operand in registers, that arithmetic alone runs at 1.68 Pop/s (27.5 us for this shape)
+                        "tera_ops_arithmetic_only_ceiling": 1680.0,
                         "activation_retiling_us": round(max(0.0, us_alone - us) * 8 / 7, 2),
                         "first_use_us_incl_weight_conversion": round(first_us, 1),
                         "converted_weight_copy_bytes": n * k,
@@ -350,6 +386,7 @@ def main():
         log("prefill GEMM m=512 n=%d k=%d: %.1f us  %.1f Tops (%.1f%% of 5 Pop/s); 3 / 8 independent ones in a message: %.1f / %.1f us each; alone with re-tiling %.1f us; first use %.0f us" % (
             n, k, us, tops, tops / 50, grouped[3], grouped[8], us_alone, first_us))
         ctx.release(ha), ctx.release(ho)
+    other.close()
 
     # ------------------------------------------------------------------ decode chain (config 0)
     # RMSNorm -> Q8_0 -> GEMV (4096 x 4096, Q4_0) for one token as one message: the norm + quantize request and the
@@ -699,11 +736,22 @@ def main():
         "config": {"workload": "configs[1]: Llama-7B decode layer, 7 Q4_0xQ8_0 GEMVs at m=1 submitted as one message "
                                "(one launch), %d layers of distinct weights rotated (cold HBM reads)" % LAYERS,
                    "algorithmic_bytes_per_step": layer_bytes[1], "pct_of_hbm_peak": round(value / HBM_PEAK_GBPS * 100, 2),
-                   "wall_ms_per_step": round(wall_step, 6), "launches_per_step": subs1},
+                   "wall_ms_per_step": round(wall_step, 6), "launches_per_step": subs1,
+                   "host_walk_us_per_message": round(host_walk_us, 3),
+                   # what the step is NOT: a decoder layer with its data dependencies. Its seven matmuls are four
+                   # dependent launches (q+k+v, o, gate+up, down), and with norms, attention and quantizations the layer
+                   # for one token is `decoder_layer_one_token`; both are reported here so that the headline fraction
+                   # is read as the one-launch weight stream it is
+                   "dependent_launches_us": {r["launch"]: r["us_per_launch"] for r in launches},
+                   "dependent_launches_frac_of_hbm_peak": round(
+                       layer_bytes[1] / sum(r["us_per_launch"] for r in launches) / 1e3 / HBM_PEAK_GBPS, 4),
+                   "decoder_layer_one_token_us": round(layer6_us, 2),
+                   "decoder_layer_one_token_frac_of_hbm_peak": round(layer6_bytes / layer6_us / 1e3 / HBM_PEAK_GBPS, 4)},
         "roofline": {"bound": "hbm", "achieved": round(value, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(value / HBM_PEAK_GBPS, 4), "traffic": measured_traffic("layer"),
+                     "frac": round(value / HBM_PEAK_GBPS, 4), "traffic": measured_traffic("layer", step_launch, subs1),
                      "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE over this script, profiled offline",
                      "kernel": "gemv_members_kernel<Q4_0>: the seven GEMVs of the layer message in one launch (m=1)",
+                     "launch": step_launch,
                      "bytes_per_launch": layer_bytes[1], "us_per_launch": round(ms_step * 1e3, 3)},
         "step_us": step_stats,
         "launches": launches,

@@ -3,6 +3,9 @@
 #include "context.h"
 #include "htpops_bench.h"
 
+#include <chrono>
+#include <cstdio>
+
 using namespace htpops;
 using namespace htpops::host;
 
@@ -145,4 +148,38 @@ extern "C" int htpops_measure_copy_bandwidth(htpops_context *ctx, size_t bytes, 
   }
   *gbps = 2.0 * (double) (bytes / 16 * 16) * iters / ((double) ms * 1e-3) / 1e9;
   return HTPOPS_OK;
+}
+
+extern "C" int htpops_last_gemv_launch(htpops_context *ctx, char *text, size_t cap) {
+  if (!ctx || !text || cap == 0) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  const LaunchRecord &r = last_gemv_launch();
+  snprintf(text, cap, "%s<%d,%d,%d> grid=%u block=%u lds=%u", r.kernel, r.t0, r.t1, r.t2, r.grid, r.block, r.lds);
+  return HTPOPS_OK;
+}
+
+extern "C" int htpops_measure_host_walk_us(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes, int iters,
+                                           double *us_per_message) {
+  if (!ctx || !msg || !us_per_message || iters <= 0) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  // keep the stream busy first: with a backlog in the queue, an enqueue returns as soon as the host side of it is done
+  for (int i = 0; i < 64; ++i) {
+    if (int r = htpops_enqueue_message(ctx, msg, msg_bytes)) {
+      return r;
+    }
+  }
+  const auto t0 = std::chrono::steady_clock::now();
+  for (int i = 0; i < iters; ++i) {
+    if (int r = htpops_enqueue_message(ctx, msg, msg_bytes)) {
+      return r;
+    }
+  }
+  const auto t1 = std::chrono::steady_clock::now();
+  *us_per_message = std::chrono::duration<double, std::micro>(t1 - t0).count() / iters;
+  return htpops_synchronize(ctx);
 }

@@ -696,6 +696,8 @@ hipError_t launch_gemv_members(hipStream_t stream, GemvMembers &grp, const GemvN
   }
 #define HTPOPS_GEMV_LAUNCH(LONG, T) \
   hipLaunchKernelGGL((gemv_members_kernel<WT, LONG, T>), grid, dim3(T), lds, stream, b[1], b[2], b[3], b[4], b[5], b[6], b[7], grp)
+  last_gemv_launch() = { norm ? "gemv_members_norm_kernel" : "gemv_members_kernel", WT, norm ? 0 : (int) any_long,
+                         threads, (unsigned) blocks, (unsigned) threads, (unsigned) lds };
   if (norm) {
     hipLaunchKernelGGL((gemv_members_norm_kernel<WT, false, 512>), grid, dim3(512), lds, stream, b[1], b[2], b[3], b[4],
                        b[5], b[6], b[7], grp, *norm);
@@ -895,6 +897,11 @@ hipError_t launch_gemv_row(hipStream_t stream, float *out, const uint32_t *act, 
 }
 
 }  // namespace
+
+LaunchRecord &last_gemv_launch() {
+  static thread_local LaunchRecord rec;
+  return rec;
+}
 
 // m rows of activations, one pass over the weights per activation row. The caller routes larger m to the MFMA path.
 hipError_t launch_gemv_q8_0_act(hipStream_t stream, float *out, const void *act, const void *weight, int m, int k,

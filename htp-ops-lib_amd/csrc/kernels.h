@@ -145,6 +145,16 @@ hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const v
                              bool mask_threshold);
 bool       flash_attn_writes_q8_0(int qo_len, int head_dim, bool qo_is_f32);
 
+// What the calling thread's most recent launch of the one-row matmul kernel was: kernel instance and geometry. The bench
+// harness compares it with the launch its hardware-counter figures were taken from.
+struct LaunchRecord {
+  const char *kernel = "";  // kernel family
+  int         t0 = 0, t1 = 0, t2 = 0;  // template arguments of the instance
+  unsigned    grid = 0, block = 0;
+  unsigned    lds = 0;
+};
+LaunchRecord &last_gemv_launch();
+
 // measurement helpers
 hipError_t launch_copy(hipStream_t stream, void *dst, const void *src, size_t bytes);
 // one pass over `bytes` (16-byte multiples) that keeps nothing; `sink` is one device word the kernel never writes in practice

@@ -435,6 +435,7 @@ __global__ __launch_bounds__(kSlThreads) void matmul_skinny_slice_kernel(SkinnyG
     if (lds_ticket != (unsigned) (nslices - 1)) {
       return;
     }
+    __atomic_signal_fence(__ATOMIC_SEQ_CST);  // (compile time: the loads below stay behind the ticket; the barrier above orders them in hardware)
     const float *all = partials + (size_t) gtile * nslices * (MR * 64);
 #pragma unroll
     for (int e = 0; e < EPT; ++e) {

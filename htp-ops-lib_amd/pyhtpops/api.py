@@ -57,7 +57,8 @@ EXPORTED_SYMBOLS = [
     "htpops_mat_mul_permuted_w16a32", "htpops_rms_norm_f32_ex_ptr", "htpops_quantize_q8_0_ptr",
     "htpops_rms_norm_quantize_q8_0_ptr", "htpops_mat_mul_q8_0_act_ptr", "htpops_mat_mul_f32_act_ptr",
     "htpops_flash_attn_ptr", "htpops_flash_attn_noalloc_ptr", "htpops_timer_start", "htpops_timer_stop", "htpops_timer_elapsed_ms",
-    "htpops_measure_mfma_peak", "htpops_measure_copy_bandwidth", "htpops_measure_read_us",
+    "htpops_measure_mfma_peak", "htpops_measure_copy_bandwidth", "htpops_measure_read_us", "htpops_last_gemv_launch",
+    "htpops_measure_host_walk_us",
 ]
 
 
@@ -123,6 +124,8 @@ def load_library(path=None):
         "htpops_measure_mfma_peak": (ci, [vp, ci, ci, ctypes.POINTER(ctypes.c_double)]),
         "htpops_measure_copy_bandwidth": (ci, [vp, sz, ci, ctypes.POINTER(ctypes.c_double)]),
         "htpops_measure_read_us": (ci, [vp, sz, ci, ci, ctypes.POINTER(ctypes.c_double)]),
+        "htpops_last_gemv_launch": (ci, [vp, ctypes.c_char_p, sz]),
+        "htpops_measure_host_walk_us": (ci, [vp, vp, sz, ci, ctypes.POINTER(ctypes.c_double)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -364,6 +367,19 @@ class Context:
         v = ctypes.c_double()
         self._check(self.lib.htpops_measure_read_us(self._ctx, int(nbytes), buffers, iters, ctypes.byref(v)))
         return v.value
+
+    def last_gemv_launch(self):
+        buf = ctypes.create_string_buffer(256)
+        self._check(self.lib.htpops_last_gemv_launch(self._ctx, buf, len(buf)))
+        return buf.value.decode()
+
+    def measure_host_walk_us(self, msg, iters=2000):
+        """Host microseconds per htpops_enqueue_message of `msg` with the stream kept busy (no kernel time)."""
+        buf = (ctypes.c_char * len(msg)).from_buffer(msg)
+        v = ctypes.c_double()
+        self._check(self.lib.htpops_measure_host_walk_us(self._ctx, ctypes.cast(buf, ctypes.c_void_p), len(msg), iters,
+                                                         ctypes.byref(v)))
+        return float(v.value)
 
     def measure_copy_bandwidth(self, nbytes, iters=20):
         v = ctypes.c_double()

@@ -33,6 +33,17 @@ int htpops_measure_copy_bandwidth(htpops_context *ctx, size_t bytes, int iters, 
  * memory-side cache = every launch reads HBM). The floor under any one-launch weight stream of that size. */
 int htpops_measure_read_us(htpops_context *ctx, size_t bytes, int buffers, int iters, double *us_per_launch);
 
+/* Kernel instance and launch geometry of the calling thread's most recent launch of the one-row matmul kernel, as text
+ * ("gemv_members_kernel<2,1,512> grid=2400 block=512 lds=..."): the harness checks that the launch it times is the
+ * launch its hardware-counter figures were profiled on. */
+int htpops_last_gemv_launch(htpops_context *ctx, char *text, size_t cap);
+
+/* Host time of walking a message: `iters` calls of htpops_enqueue_message timed on the host clock while the stream has
+ * a backlog (so that no call waits for the GPU); includes the HIP launch calls, nothing of the kernels' run time.
+ * Waits for the stream before returning. */
+int htpops_measure_host_walk_us(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes, int iters,
+                                double *us_per_message);
+
 #ifdef __cplusplus
 }
 #endif
