@@ -52,7 +52,7 @@ constexpr size_t kNoAllocScratchBytes = (size_t) 8 << 20;
 // when the context is created (HTPOPS_<NAME> in upper case), changed afterwards only through htpops_set_option; no
 // entry point on the op path reads the environment.
 struct Options {
-  int lane_order          = 1;   // 0: never the repacked-weight kernel; 2 / 3: force one / two tiles per workgroup
+  int lane_order          = 1;   // 0: never the repacked-weight kernels; 2 / 3: the one-block kernel with one / two tiles per workgroup
   int gemm_fp6            = -1;  // 0: never the FP6-tile kernel; 1: also on shapes that do not fill the device
   int gemv_rows_kernel    = 1;   // 0: two and three rows take the repacked-weight / K-sliced kernels
   int gemm_tile_units     = 0;   // 1 / 2: force the tile size of the int8 fragment kernel
@@ -219,6 +219,7 @@ constexpr int kManyRowsMinM    = 33;  // rows from which a matmul takes the matr
 
 constexpr int kFragKindRowLayout = 100;  // + ggml type: int8 fragments (kinds 1..4 are the tile-permuted formats of ops 1-4)
 constexpr int kFragKindLaneOrder = 300;  // + ggml type: weights in matrix-core operand order (2..16 activation rows)
+constexpr int kFragKindBlockPairs = 350; // + ggml type: the same for the two-blocks-per-instruction kernel (2..8 rows)
 constexpr int kFragKindFp6Tiles  = 400;  // + ggml type: FP6 operand tiles of the many-row Q4_0 matmul (LDS kernel)
 
 // Which kernel family a quantized matmul takes and how much of the context's workspace it needs.
@@ -242,10 +243,12 @@ MatMulPlan plan_mat_mul(htpops_context *ctx, const void *weight, bool act_aligne
 // The converted copy a plan wants, from the cache or made now and cached (plan.cacheable); *out stays nullptr for a
 // plan whose weights may not be cached (the caller converts into its workspace).
 int plan_weight_copy(htpops_context *ctx, MatMulPlan &plan, const void *weight, int k, int n, int wt, const void **out);
-// The repacked copy of `weight` for the few-row kernel: from the cache, or made now and cached. *out stays nullptr when
-// this matmul does not take that kernel.
+// The repacked copy of `weight` for the few-row kernels: from the cache, or made now and cached. *out stays nullptr
+// when this matmul takes neither of them. *block_pairs: which of the two operand orders the copy is in (the kernel
+// with two blocks per matrix instruction for up to 8 rows of Q4_0, the one-block kernel otherwise); the choice depends
+// on (m, k, weight type) and the context's switches only, so the members of a grouped launch agree on it.
 int lane_order_weights(htpops_context *ctx, const void *weight, const void *act, int m, int k, int n, int wt,
-                       const void **out);
+                       const void **out, bool *block_pairs);
 
 int op_rms_norm(htpops_context *ctx, float *dst, const float *src, const float *weight, float eps, int ne0, int ne1);
 int op_quantize(htpops_context *ctx, void *dst, const float *src, int k, int m);

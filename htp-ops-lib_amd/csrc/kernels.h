@@ -71,6 +71,14 @@ hipError_t launch_weights_to_lane_order(hipStream_t stream, void *dst, const voi
 hipError_t launch_matmul_lane_order_group(hipStream_t stream, int count, float *const *outs, const void *const *acts,
                                           const void *const *lane_order_weights, const int *ns, int m, int k,
                                           WeightType wt, int forced_tiles);  // forced_tiles 2 / 3: one / two tiles per workgroup
+// 2 <= m <= 8 rows against Q4_0 weights repacked once into another operand order (launch_weights_to_block_pairs, the
+// same size again): two blocks per matrix instruction, the second one in the result rows that 8 activation rows leave
+// unused. A workgroup keeps its member's activation rows in LDS and streams tiles of 16 weight rows over the whole of
+// K; members may differ in k. Conditions: k % 256 == 0, n % 16 == 0, `act` and the repacked weights 16-byte aligned.
+bool       matmul_block_pairs_fits(int n, int m, int k, WeightType wt);
+hipError_t launch_weights_to_block_pairs(hipStream_t stream, void *dst, const void *weight, int k, int n);
+hipError_t launch_matmul_block_pairs_group(hipStream_t stream, int count, float *const *outs, const void *const *acts,
+                                           const void *const *pair_order_weights, const int *ns, int m, const int *ks);
 // many-row path for Q4_0 weights, k % 64 == 0: FP6 scaled MFMA (exact: int8 = 16 hi + lo, all parts |t| <= 15) over operand
 // tiles staged in LDS by DMA. The weight tiles (gemm_fp6_lds_weight_tile_bytes, 1 byte per weight) are converted once
 // (launch_q4_0_to_fp6_tiles) and can be cached by the caller; the activation tiles (gemm_fp6_lds_act_tile_bytes) are

@@ -65,6 +65,7 @@ struct GemvBatch {
   } norm;
   bool fused = false;  // the members read norm.dst and run in the launch that makes it
   bool fp6   = false;  // many-row members of the FP6-tile kernel (all over the same activation rows and k)
+  bool pairs_fit = false;  // every member fits the two-blocks-per-instruction kernel (such members may differ in k)
 };
 
 // The many-row members of a batch: converted weights from the cache (made now where missing), the distinct activation
@@ -212,34 +213,41 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
       e = launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k, (WeightType) b.wt);
     } else {
       // 2..16 rows. Two or three rows are one launch of the weight stream that keeps them in registers, each member
-      // with its own rows and row length. Otherwise (same k) members whose weights have (or get) a repacked copy go
-      // to the kernel that streams it, again each with its own activation rows; the rest go to the K-sliced kernel,
-      // one launch per set of rows (it stages one). Which kernel a matrix gets depends on that matrix alone.
+      // with its own rows and row length. Otherwise members whose weights have (or get) a repacked copy go to the
+      // kernel that streams it, again each with its own activation rows (and, for the two-blocks-per-instruction
+      // kernel, its own k; the batch holds members of different k only where every one of them fits that kernel); the
+      // rest go to the K-sliced kernel, one launch per set of rows (it stages one). Which kernel a matrix gets depends
+      // on that matrix alone.
       if (ctx->opt.gemv_rows_kernel != 0 && gemv_rows_fits(b.m, k0, (WeightType) b.wt)) {
         e = launch_gemv_rows_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.m, b.k,
                                                     (WeightType) b.wt);
       } else {
         float      *out_a[kGemvGroupMax];
         const void *w_a[kGemvGroupMax], *act_a[kGemvGroupMax];
-        int         n_a[kGemvGroupMax], count_a = 0;
+        int         n_a[kGemvGroupMax], k_a[kGemvGroupMax], count_a = 0;
         bool        sliced[kGemvGroupMax] = {};
+        bool        pairs = false;  // which repacked-weight kernel (the same for every member: it depends on m, k, type)
         for (int i = 0; i < b.count; ++i) {
           const void *lw = nullptr;
-          if (int r = lane_order_weights(ctx, b.w[i], b.act[i], b.m, k0, b.n[i], b.wt, &lw)) {
+          bool        member_pairs = false;
+          if (int r = lane_order_weights(ctx, b.w[i], b.act[i], b.m, b.k[i], b.n[i], b.wt, &lw, &member_pairs)) {
             b.hdr[i]->state = r;
           } else if (lw) {
-            out_a[count_a] = b.out[i], w_a[count_a] = lw, act_a[count_a] = b.act[i], n_a[count_a++] = b.n[i];
+            pairs          = member_pairs;
+            out_a[count_a] = b.out[i], w_a[count_a] = lw, act_a[count_a] = b.act[i], k_a[count_a] = b.k[i];
+            n_a[count_a++] = b.n[i];
           } else if (b.m <= kSkinnyGroupMaxM) {
             sliced[i] = true;
           } else {
             // more rows than the K-sliced group launch takes: on its own
-            b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act[i], b.w[i], b.m, k0, b.n[i], b.wt);
+            b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act[i], b.w[i], b.m, b.k[i], b.n[i], b.wt);
           }
         }
         e = hipSuccess;
         if (count_a > 0) {
-          e = launch_matmul_lane_order_group(ctx->stream, count_a, out_a, act_a, w_a, n_a, b.m, k0, (WeightType) b.wt,
-                                             ctx->opt.lane_order);
+          e = pairs ? launch_matmul_block_pairs_group(ctx->stream, count_a, out_a, act_a, w_a, n_a, b.m, k_a) :
+                      launch_matmul_lane_order_group(ctx->stream, count_a, out_a, act_a, w_a, n_a, b.m, k0,
+                                                     (WeightType) b.wt, ctx->opt.lane_order);
         }
         for (int first = 0; first < b.count && e == hipSuccess && ret == HTPOPS_OK; ++first) {
           if (!sliced[first]) {
@@ -249,16 +257,16 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
           const void *w_b[kGemvGroupMax];
           int         n_b[kGemvGroupMax], count_b = 0;
           for (int i = first; i < b.count; ++i) {  // everybody left that reads the rows of `first`
-            if (sliced[i] && b.act[i] == b.act[first]) {
+            if (sliced[i] && b.act[i] == b.act[first] && b.k[i] == b.k[first]) {
               out_b[count_b] = b.out[i], w_b[count_b] = b.w[i], n_b[count_b++] = b.n[i];
               sliced[i] = false;
             }
           }
-          const size_t ws = matmul_skinny_group_workspace_bytes(count_b, n_b, b.m, k0);
+          const size_t ws = matmul_skinny_group_workspace_bytes(count_b, n_b, b.m, b.k[first]);
           if (int r = ensure_workspace(ctx, ws)) {
             ret = r;
           } else {
-            e = launch_matmul_skinny_group(ctx->stream, count_b, out_b, b.act[first], w_b, n_b, b.m, k0,
+            e = launch_matmul_skinny_group(ctx->stream, count_b, out_b, b.act[first], w_b, n_b, b.m, b.k[first],
                                                    (WeightType) b.wt, ctx->workspace, ctx->tickets, kTicketSlots);
           }
         }
@@ -363,7 +371,8 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
               b.fp6 == fp6 && (!fp6 || (b.act[0] == act && b.k[0] == p->k)) &&
               (p->m == 1 || many_rows || b.k[0] == p->k ||
                (ctx->opt.gemv_rows_kernel != 0 && gemv_rows_fits(p->m, p->k, (WeightType) wt) &&
-                gemv_rows_fits(b.m, b.k[0], (WeightType) wt)));
+                gemv_rows_fits(b.m, b.k[0], (WeightType) wt)) ||
+               (ctx->opt.lane_order == 1 && b.pairs_fit && matmul_block_pairs_fits(p->n, p->m, p->k, (WeightType) wt)));
   for (int i = 0; join && i < b.count; ++i) {
     const size_t wi = weight_bytes((size_t) b.n[i], (size_t) b.k[i], b.wt), oi = (size_t) b.m * b.n[i] * 4;
     const size_t ai = q8_0_bytes((size_t) b.m, (size_t) b.k[i]);
@@ -377,8 +386,9 @@ bool try_batch(htpops_context *ctx, const struct OpComputeRequest *req, struct R
     if (b.count > 0) {
       flush_batch(ctx, b);
     }
-    b.wt = wt, b.m = p->m, b.fp6 = fp6;
+    b.wt = wt, b.m = p->m, b.fp6 = fp6, b.pairs_fit = true;
   }
+  b.pairs_fit = b.pairs_fit && matmul_block_pairs_fits(p->n, p->m, p->k, (WeightType) wt);
   b.hdr[b.count] = hdr, b.out[b.count] = out, b.w[b.count] = w, b.act[b.count] = act, b.n[b.count] = p->n, b.k[b.count] = p->k;
   ++b.count;
   hdr->state = HTPOPS_OK;

@@ -98,12 +98,14 @@ int check_mat_mul(htpops_context *ctx, const void *dst, const void *act, const v
 // kernels that read the weights as they are. A failed allocation or conversion launch is an error, not a reason to
 // switch kernels.)
 int lane_order_weights(htpops_context *ctx, const void *weight, const void *act, int m, int k, int n, int wt,
-                       const void **out) {
-  *out = nullptr;
-  if (ctx->opt.lane_order == 0 || !aligned(act, 16) || !matmul_lane_order_fits(n, m, k, (WeightType) wt)) {
+                       const void **out, bool *block_pairs) {
+  *out         = nullptr;
+  *block_pairs = ctx->opt.lane_order == 1 && matmul_block_pairs_fits(n, m, k, (WeightType) wt);
+  if (ctx->opt.lane_order == 0 || !aligned(act, 16) ||
+      !(*block_pairs || matmul_lane_order_fits(n, m, k, (WeightType) wt))) {
     return HTPOPS_OK;
   }
-  const int kind = kFragKindLaneOrder + wt;
+  const int kind = (*block_pairs ? kFragKindBlockPairs : kFragKindLaneOrder) + wt;
   if ((*out = find_copy(ctx, weight, kind, k, n)) != nullptr) {
     return HTPOPS_OK;
   }
@@ -115,7 +117,8 @@ int lane_order_weights(htpops_context *ctx, const void *weight, const void *act,
   if (int r = new_copy(ctx, weight, w_bytes, kind, k, n, matmul_lane_order_weight_bytes(k, n, (WeightType) wt), &fresh)) {
     return r;
   }
-  const hipError_t e = launch_weights_to_lane_order(ctx->stream, fresh, weight, k, n, (WeightType) wt);
+  const hipError_t e = *block_pairs ? launch_weights_to_block_pairs(ctx->stream, fresh, weight, k, n) :
+                                      launch_weights_to_lane_order(ctx->stream, fresh, weight, k, n, (WeightType) wt);
   if (e != hipSuccess) {
     forget_copy(ctx, fresh);
     return hip_fail(ctx, e, "weight repack launch");
@@ -198,13 +201,15 @@ int run_few_rows(htpops_context *ctx, float *dst, const void *act, const void *w
     }
     (void) hipGetLastError();
   }
-  const void *lw = nullptr;
-  if (int r = lane_order_weights(ctx, weight, act, m, k, n, wt, &lw)) {
+  const void *lw    = nullptr;
+  bool        pairs = false;
+  if (int r = lane_order_weights(ctx, weight, act, m, k, n, wt, &lw, &pairs)) {
     return r;
   }
   if (lw) {
-    const hipError_t e = launch_matmul_lane_order_group(ctx->stream, 1, &dst, &act, &lw, &n, m, k, (WeightType) wt,
-                                                        ctx->opt.lane_order);
+    const hipError_t e = pairs ? launch_matmul_block_pairs_group(ctx->stream, 1, &dst, &act, &lw, &n, m, &k) :
+                                 launch_matmul_lane_order_group(ctx->stream, 1, &dst, &act, &lw, &n, m, k, (WeightType) wt,
+                                                                ctx->opt.lane_order);
     if (e == hipSuccess) {
       return HTPOPS_OK;
     }

@@ -346,8 +346,9 @@ extern "C" int htpops_buffer_prepare_weights(htpops_context *ctx, int handle, si
     }
   } else if (m_hint >= 2 && !(ctx->opt.gemv_rows_kernel != 0 && gemv_rows_fits(m_hint, k, (WeightType) weight_type))) {
     // (the two- and three-row kernel reads the weights as they are: nothing to make for it)
-    const void *copy = nullptr;
-    if (int r = lane_order_weights(ctx, w, nullptr, m_hint, k, n, weight_type, &copy)) {
+    const void *copy  = nullptr;
+    bool        pairs = false;
+    if (int r = lane_order_weights(ctx, w, nullptr, m_hint, k, n, weight_type, &copy, &pairs)) {
       return r;
     }
   }

@@ -801,6 +801,41 @@ def test_message_groups_independent_few_row_matmuls(ctx, oracle, wt, m):
             ctx.release(h)
 
 
+@pytest.mark.parametrize("m", [2, 5, 8])
+def test_message_groups_few_row_q4_0_matmuls_of_different_k(ctx, oracle, m):
+    # 2..8 rows against Q4_0 weights with n % 16 == 0, k % 256 == 0 take the two-blocks-per-instruction kernel, whose
+    # members bring their own k: matmuls over rows of different length share a launch (the longest rows size its LDS;
+    # k = 11008 leaves one workgroup per compute unit, which also changes how far ahead the weights are requested). A
+    # member of the first one's k that does not fit that kernel (n = 40) still joins the batch, and runs on the kernel
+    # that reads the weights as they are. Every request must equal its own launch bit for bit and meet the oracle.
+    ctx.set_option("gemv_rows_kernel", 0)  # (two and three rows would otherwise stay on the decode kernel's stream)
+    rng = wl.rng_for(77, m)
+    wt, op = wl.GGML_TYPE_Q4_0, api.HTP_OPS_MAT_MUL_Q4_0_Q8_0
+    ks = [512, 2048, 11008, 256, 2048, 512]
+    ns = [64, 48, 32, 16, 1008, 40]
+    ws = [wl.make_weights(rng, n, k, wt) for n, k in zip(ns, ks)]
+    acts = [oracle.quantize_q8_0(wl.make_activations(rng, m, k)) for k in ks]
+    has = [ctx.upload(a) for a in acts]
+    hws = [ctx.upload(w) for w in ws]
+    hos = [ctx.alloc(m * n * 4) for n in ns]
+    try:
+        msg = api.build_message([_mm(op, ho, ha, hw, m, k, n) for ho, ha, hw, n, k in zip(hos, has, hws, ns, ks)])
+        for _ in range(2):
+            for ho, n in zip(hos, ns):
+                ctx.write(ho, np.full(m * n, np.nan, np.float32))
+            assert ctx.process_message(msg) == 0
+            assert api.message_request_states(msg) == [0] * len(ns), ctx.last_error()
+            assert ctx.last_message_submissions() == 1
+            for ho, a, w, n, k in zip(hos, acts, ws, ns, ks):
+                got = ctx.read(ho, np.float32, m * n).reshape(m, n)
+                assert np.array_equal(got, ctx.run_mat_mul(a, w, m, k, n, wt)), "a request differs from its own launch"
+                want, mag = oracle.mat_mul_q8_0_act_f64(a, w, m, k, n, wt)
+                assert np.all(np.abs(got - want) <= MATMUL_RTOL * mag)
+    finally:
+        for h in has + hws + hos:
+            ctx.release(h)
+
+
 def test_message_groups_many_row_matmuls_over_the_same_rows(ctx, oracle):
     # Independent many-row Q4_0 matmuls over the SAME activation rows (q/k/v or gate/up of a prefill chunk) whose
     # weights live in buffers of the context share the launch of the FP6-tile kernel (one grid keeps the compute units
