@@ -548,6 +548,12 @@ def main():
         attention.append({"qo_len": qo, "kv_len": kv, "us": round(us, 2), "kv_GBps": round(kv_bytes / us / 1e3, 1),
                           "frac_of_hbm_peak": round(kv_bytes / us / 1e3 / HBM_PEAK_GBPS, 4),
                           "tera_flops_causal": round(flops / us / 1e6, 2), "max_abs_err_vs_f64": worst})
+        if qo == 1:
+            # the two launches of a one-token call by themselves (each `iters` times in a row between two events)
+            split_us, merge_us = ctx.measure_decode_attention_parts(ho, hq, hks, hvs, kv, nh, nkv, hd, False, 200)
+            attention[-1].update({"split_kv_launch_us": round(split_us, 2), "merge_launch_us": round(merge_us, 2),
+                                  "split_kv_launch_GBps": round(kv_bytes / split_us / 1e3, 1)})
+            log("  split-KV launch %.2f us (%.0f GB/s), merge launch %.2f us" % (split_us, kv_bytes / split_us / 1e3, merge_us))
         log("attention qo=%d kv=%d: %.2f us  KV %.0f GB/s  %.1f TFLOP/s  (max |err| %.1e)" % (
             qo, kv, us, kv_bytes / us / 1e3, flops / us / 1e6, worst))
         for h in [hq, ho] + hks + hvs:

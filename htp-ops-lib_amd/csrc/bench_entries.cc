@@ -183,3 +183,40 @@ extern "C" int htpops_measure_host_walk_us(htpops_context *ctx, struct MessageHe
   *us_per_message = std::chrono::duration<double, std::micro>(t1 - t0).count() / iters;
   return htpops_synchronize(ctx);
 }
+
+extern "C" int htpops_measure_decode_attention_parts(htpops_context *ctx, void *o, const void *q, const void *const *ks,
+                                                     const void *const *vs, int sets, int kv_len, int n_heads,
+                                                     int n_kv_heads, int head_dim, int qo_is_f32, int iters,
+                                                     double *split_us, double *merge_us) {
+  if (!ctx || !o || !q || !ks || !vs || sets <= 0 || iters <= 0 || !split_us || !merge_us || n_kv_heads <= 0 ||
+      n_heads % n_kv_heads != 0 || kv_len <= 0) {
+    return HTPOPS_ERR_REJECTED;
+  }
+  if (int r = need_device(ctx)) {
+    return r;
+  }
+  Lock lock(ctx->mu);
+  if (int r = ensure_workspace(ctx, flash_attn_workspace_bytes(1, kv_len, n_heads, head_dim))) {
+    return r;
+  }
+  double *out[2] = { split_us, merge_us };
+  for (int part = 1; part <= 2; ++part) {
+    for (int i = -8; i < iters; ++i) {  // (eight launches to warm up; the K/V sets take turns so that reads come from HBM)
+      if (i == 0) {
+        HTPOPS_HIP(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+      }
+      const int        s = ((i % sets) + sets) % sets;
+      const hipError_t e = launch_flash_attn_decode_part(ctx->stream, part, o, q, ks[s], vs[s], kv_len, n_heads, n_kv_heads,
+                                                         head_dim, qo_is_f32 != 0, ctx->workspace);
+      if (e != hipSuccess) {
+        return hip_fail(ctx, e, "decode attention part");
+      }
+    }
+    HTPOPS_HIP(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
+    HTPOPS_HIP(ctx, hipEventSynchronize(ctx->ev_stop));
+    float ms = 0.0f;
+    HTPOPS_HIP(ctx, hipEventElapsedTime(&ms, ctx->ev_start, ctx->ev_stop));
+    *out[part - 1] = (double) ms * 1e3 / iters;
+  }
+  return HTPOPS_OK;
+}

@@ -22,6 +22,8 @@
 #include "device_utils.h"
 #include "kernels.h"
 
+#include <algorithm>
+
 namespace htpops {
 
 namespace {
@@ -459,15 +461,23 @@ __device__ __forceinline__ float key_group_sum(float v) {
 }
 
 // partial record per (head, split): m, l, then D floats of un-normalised O.
-// A workgroup of THREADS threads owns SPLIT consecutive keys of one KV head. LPK = D / 8 lanes share a key (16 bytes of
-// K and of V each); every K and V load of the wave is issued before the first use and the scores of all GH heads are
-// formed against the same registers. The workgroup agrees on one maximum per head (lane exchange inside the wave, LDS
-// between the waves) BEFORE the exponentials, so the per-slot sums and O columns only have to be added up.
-// Measured on MI355X (32 query / 8 KV heads of 128, kv_len 4096, cold K/V): a call is 11.3-11.5 us of which about 9 us
-// are the two dependent launches themselves (the same call reading an eighth of the keys: 9.0 us; without the score
-// and P V arithmetic: 10.7 us); 512 threads per workgroup change nothing. Merging inside this launch -- records
-// written through, a ticket per KV head, the last workgroup merges -- is slower (18-19 us, 47 us at kv_len 16384):
-// the 32 to 128 ticket updates of one counter from all over the chip are served one after the other.
+// A workgroup of THREADS threads owns SPLIT consecutive keys of one KV head; each wave owns SPLIT / WAVES of them and
+// works without the others until the end. Every K and V load of the wave is issued before the first use.
+//  * scores: S = K Q^T on the matrix cores (v_mfma_f32_16x16x32_f16: 16 keys x up to 16 heads of the GQA group, the
+//    head dimension as k), K in the A operand as it lies in memory (a lane loads 16 bytes of a key row per k step), the
+//    queries of the group, scaled and rounded to fp16 like the prefill kernel's, in the B operand. A lane then holds the
+//    scores of 4 keys for one head per tile.
+//  * softmax against the wave's own maximum; the probabilities go through LDS (fp16, pairs of keys in a dword) to
+//  * O += P V on the vector ALU with v_dot2_f32_f16 (two keys per instruction, exact products, fp32 sums): LPK = D / 8
+//    lanes share a key, each with 16 bytes of its V row, all heads of the group against the same V registers.
+// The waves' (max, sum, O) are put together through LDS with the factor exp2(m_wave - m_all) per wave and head.
+// Measured on MI355X (32 query / 8 KV heads of 128, cold K/V) against the earlier all-vector-ALU version of this kernel
+// (8 multiply-adds, 4 lane exchanges and an exponential per key, head and lane: about 1000 vector instructions per
+// wave, which at kv_len 16384 kept the vector ALUs busy for longer than the K/V stream takes): see the table in the
+// launcher. Merging inside this launch -- records written through, a ticket per KV head, the last workgroup merges
+// -- was slower (18-19 us, 47 us at kv_len 16384).
+// (A variant in which a workgroup walks several chunks of SPLIT keys, the next chunk's K and V on their way while one is
+// worked on, about one workgroup per compute unit, was slower at kv_len 16384: 17.0 against 15.1 us.)
 template <int D, int GH, bool QO_F32, int SPLIT, int THREADS>
 __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__restrict__ part,
                                                                     const void *__restrict__ q_ptr,
@@ -476,200 +486,237 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
                                                                     const _Float16 *__restrict__ mask, int kv_len,
                                                                     int n_heads, int n_kv_heads, int head0_in_group,
                                                                     int n_splits, int mask_threshold) {
-  constexpr int LPK    = D / 8;        // lanes per key (8 halfs = 16 bytes each)
+  constexpr int LPK    = D / 8;        // lanes per key in the P V part (8 halfs = 16 bytes of the V row each)
   constexpr int KPW    = kWave / LPK;  // keys per wave per pass
   constexpr int WAVES  = THREADS / kWave;
   constexpr int SLOTS  = WAVES * KPW;  // independent partial streams in the workgroup
   constexpr int PASSES = SPLIT / SLOTS;
-  static_assert(SPLIT % SLOTS == 0 && PASSES >= 1, "whole passes");
-  extern __shared__ float dec_lds[];  // red_o[SLOTS][GH][D], red_l[SLOTS][GH], red_m[WAVES][GH]
-  float *red_o = dec_lds, *red_l = dec_lds + SLOTS * GH * D, *red_m = red_l + SLOTS * GH;
+  constexpr int TILE_PASSES = 16 / KPW;            // passes that make a 16-key score tile
+  constexpr int TILES       = PASSES / TILE_PASSES;  // score tiles of a wave
+  constexpr int KSTEPS      = D / 32;              // k steps of a score tile
+  static_assert(SPLIT % SLOTS == 0 && PASSES >= 2 && PASSES % 2 == 0 && PASSES % TILE_PASSES == 0, "whole tiles, pairs of passes");
+  static_assert(GH <= 16, "the heads of a pass are the columns of one score tile");
+  typedef float v4f __attribute__((ext_vector_type(4)));
+  // red_o[SLOTS][GH][D], red_l[WAVES][GH], red_m[WAVES][GH], then per wave the probabilities [PASSES / 2][KPW][GH] dwords
+  extern __shared__ float dec_lds[];
+  float    *red_o = dec_lds, *red_l = dec_lds + SLOTS * GH * D, *red_m = red_l + WAVES * GH;
+  uint32_t *p_sh  = reinterpret_cast<uint32_t *>(red_m + WAVES * GH);
 
   const int group = n_heads / n_kv_heads;
   const int h_kv  = blockIdx.y;
   const int split = blockIdx.x;
   const int lane  = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int sub   = lane % LPK;  // which 8 dims
-  const int kslot = lane / LPK;  // which key of the pass
+  const int sub   = lane % LPK;  // P V part: which 8 dims
+  const int kslot = lane / LPK;  // P V part: which key of the pass
   const int slot  = wave * KPW + kslot;
+  const int col   = lane & 15;   // score part: which head of the pass
+  const int kg    = lane >> 4;   // score part: which 8 of a k step's 32 dims; rows 4 kg .. 4 kg + 3 of the result
   const float scale = (1.0f / sqrtf((float) D)) * kLog2e;
   const size_t kv_stride = (size_t) n_kv_heads * D;
 
   const int k_begin = split * SPLIT;
   const int k_end   = min(kv_len, k_begin + SPLIT);
+  // key of (pass, key slot of this wave); keys from k_end on are read as key k_end - 1 and score -inf
+  auto key_of = [&](int pass, int ks) { return k_begin + pass * SLOTS + wave * KPW + ks; };
 
-  // q for the GH heads, this lane's 8 dims, requested FIRST, then all K, then all V: loads return in order, so the
-  // scores of a pass need only that pass's K to have arrived, and the exponentials only the scores. fp32 queries are
-  // pre-scaled and multiplied in fp32; fp16 queries stay fp16 pairs for v_dot2_f32_f16 (exact products, fp32 sums) and
-  // the scale is applied to the finished score.
-  typedef _Float16 v2h __attribute__((ext_vector_type(2)));
-  float q[GH][8];
-  v2h   q2[GH][4];
+  // the queries first (loads return in order): head `col` of the pass, dims 32 s + 8 kg .. + 7; fp32 queries are scaled
+  // before they are rounded, and what the rounding leaves over goes into a second operand (a second matrix
+  // instruction per k step: the scores are those of the fp32 queries to about 2^-22); fp16 queries stay as they are
+  // and the scale is applied to the score
+  v8h qf[KSTEPS], qf_lo[KSTEPS];
+  {
+    const bool   q_on = col < GH && head0_in_group + col < group;
+    const size_t base = (size_t) (h_kv * group + min(head0_in_group + col, group - 1)) * D + 8 * kg;
 #pragma unroll
-  for (int g = 0; g < GH; ++g) {
-    const int    hg   = min(head0_in_group + g, group - 1);
-    const size_t base = (size_t) (h_kv * group + hg) * D + sub * 8;
-    if (QO_F32) {
-      const float4 *qp = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(q_ptr) + base);
-      const float4  q0 = qp[0], q1 = qp[1];
-      q[g][0] = q0.x * scale, q[g][1] = q0.y * scale, q[g][2] = q0.z * scale, q[g][3] = q0.w * scale;
-      q[g][4] = q1.x * scale, q[g][5] = q1.y * scale, q[g][6] = q1.z * scale, q[g][7] = q1.w * scale;
-    } else {
-      const v8h qv = *reinterpret_cast<const v8h *>(reinterpret_cast<const _Float16 *>(q_ptr) + base);
+    for (int s = 0; s < KSTEPS; ++s) {
+      if (QO_F32) {
+        const float4 *qp = reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(q_ptr) + base + 32 * s);
+        const float4  q0 = qp[0], q1 = qp[1];
+        const float   on   = q_on ? scale : 0.0f;
+        const float   x[8] = { q0.x * on, q0.y * on, q0.z * on, q0.w * on, q1.x * on, q1.y * on, q1.z * on, q1.w * on };
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        q2[g][e] = (v2h){ qv[2 * e], qv[2 * e + 1] };
+        for (int e = 0; e < 8; ++e) {
+          qf[s][e]    = (_Float16) x[e];
+          qf_lo[s][e] = (_Float16) (x[e] - (float) qf[s][e]);
+        }
+      } else {
+        const v8h qv = *reinterpret_cast<const v8h *>(reinterpret_cast<const _Float16 *>(q_ptr) + base + 32 * s);
+        qf[s]        = q_on ? qv : (v8h){ 0, 0, 0, 0, 0, 0, 0, 0 };
+        qf_lo[s]     = (v8h){ 0, 0, 0, 0, 0, 0, 0, 0 };  // (not used)
       }
     }
   }
-
-  // all K and V of this lane, requested up front (keys of a pass are consecutive across slots)
-  v8h kreg[PASSES], vreg[PASSES];
+  // all K (score layout: row `col` of tile t is key slot col % KPW of pass t TILE_PASSES + col / KPW) and all V (P V
+  // layout) of this lane, requested up front
+  v8h kf[TILES][KSTEPS], vreg[PASSES];
 #pragma unroll
-  for (int p = 0; p < PASSES; ++p) {
-    const int    key = min(k_begin + p * SLOTS + slot, k_end - 1);
-    const size_t off = (size_t) key * kv_stride + (size_t) h_kv * D + sub * 8;
-    kreg[p]          = *reinterpret_cast<const v8h *>(k_ptr + off);
+  for (int t = 0; t < TILES; ++t) {
+    const int    key = min(key_of(t * TILE_PASSES + col / KPW, col % KPW), k_end - 1);
+    const size_t off = (size_t) key * kv_stride + (size_t) h_kv * D + 8 * kg;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      kf[t][s] = *reinterpret_cast<const v8h *>(k_ptr + off + 32 * s);
+    }
   }
 #pragma unroll
   for (int p = 0; p < PASSES; ++p) {
-    const int    key = min(k_begin + p * SLOTS + slot, k_end - 1);
+    const int    key = min(key_of(p, kslot), k_end - 1);
     const size_t off = (size_t) key * kv_stride + (size_t) h_kv * D + sub * 8;
     vreg[p]          = *reinterpret_cast<const v8h *>(v_ptr + off);
   }
 
-  float sc[PASSES][GH];
-  float m_loc[GH];
+  // scores of this lane: head `col`, rows 4 kg + i of every tile
+  float sc[TILES][4];
+  float m_run = -INFINITY;
 #pragma unroll
-  for (int g = 0; g < GH; ++g) {
-    m_loc[g] = -INFINITY;
-  }
+  for (int t = 0; t < TILES; ++t) {
+    v4f acc = { 0.0f, 0.0f, 0.0f, 0.0f };
 #pragma unroll
-  for (int p = 0; p < PASSES; ++p) {
-    const int  key  = k_begin + p * SLOTS + slot;
-    const bool live = key < k_end;
-    const float mk  = (mask && live) ? mask_term(mask[key], mask_threshold != 0) : 0.0f;  // row 0 of the mask (qo_len == 1)
-#pragma unroll
-    for (int g = 0; g < GH; ++g) {
-      float s = 0.0f;
+    for (int s = 0; s < KSTEPS; ++s) {
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[t][s], qf[s], acc, 0, 0, 0);
       if (QO_F32) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          s += q[g][e] * (float) kreg[p][e];
-        }
-        s = key_group_sum<LPK>(s) + mk;
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          s = __builtin_amdgcn_fdot2(q2[g][e], (v2h){ kreg[p][2 * e], kreg[p][2 * e + 1] }, s, false);
-        }
-        s = key_group_sum<LPK>(s) * scale + mk;
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[t][s], qf_lo[s], acc, 0, 0, 0);
       }
-      s        = live ? s : -INFINITY;
-      sc[p][g] = s;
-      m_loc[g] = fmaxf(m_loc[g], s);
     }
-  }
-  // one maximum per head for the whole workgroup: over the wave's key slots, then over the waves
 #pragma unroll
-  for (int g = 0; g < GH; ++g) {
-    // (the LPK lanes of a key hold the same score: DPP row operations over the key slots, the result in lane 63)
-    float v = m_loc[g];
-#define HTPOPS_DPP_MAX(ctrl, rows) \
-  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), ctrl, rows, 0xf, false)))
-    if (LPK == 8) {
-      HTPOPS_DPP_MAX(0x140, 0xf);  // row_mirror: the two keys of a 16-lane row
-    }
-    HTPOPS_DPP_MAX(0x142, 0xa);  // row_bcast15 into rows 1 and 3
-    HTPOPS_DPP_MAX(0x143, 0xc);  // row_bcast31 into rows 2 and 3
-#undef HTPOPS_DPP_MAX
-    m_loc[g] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
-    if (lane == 0) {
-      red_m[wave * GH + g] = m_loc[g];
+    for (int i = 0; i < 4; ++i) {
+      const int  row  = 4 * kg + i;
+      const int  key  = key_of(t * TILE_PASSES + row / KPW, row % KPW);
+      const bool live = key < k_end;
+      const float mk  = (mask && live) ? mask_term(mask[key], mask_threshold != 0) : 0.0f;  // row 0 of the mask (qo_len == 1)
+      const float v   = (QO_F32 ? acc[i] : acc[i] * scale) + mk;
+      sc[t][i]        = live ? v : -INFINITY;
+      m_run           = fmaxf(m_run, sc[t][i]);
     }
   }
-  __syncthreads();
+  // the wave's maximum of head `col`: over the four row groups
+  m_run = fmaxf(m_run, __shfl_xor(m_run, 16, kWave));
+  m_run = fmaxf(m_run, __shfl_xor(m_run, 32, kWave));
+  const float m_safe = (m_run == -INFINITY) ? 0.0f : m_run;
+  float       l_run  = 0.0f;  // (the sum of head `col`, still spread over the four row groups)
+  uint32_t   *p_wave = p_sh + wave * (PASSES / 2) * KPW * GH;
+#pragma unroll
+  for (int t = 0; t < TILES; ++t) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float pr = fast_exp2(sc[t][i] - m_safe);
+      l_run += pr;
+      const int row = 4 * kg + i, pass = t * TILE_PASSES + row / KPW, ks = row % KPW;
+      if (col < GH) {
+        reinterpret_cast<_Float16 *>(p_wave + ((pass >> 1) * KPW + ks) * GH + col)[pass & 1] = (_Float16) pr;
+      }
+    }
+  }
+  // (LDS serves a wave's accesses in order: the reads below see the wave's own writes above; no other wave touches
+  // this part of LDS)
+  __builtin_amdgcn_wave_barrier();
+
+  // O += P V for the key slot and the 8 dims of this lane, all heads, two passes (keys) per instruction
   float o[GH][8];
 #pragma unroll
   for (int g = 0; g < GH; ++g) {
-    float m_all = red_m[g];
-#pragma unroll
-    for (int w = 1; w < WAVES; ++w) {
-      m_all = fmaxf(m_all, red_m[w * GH + g]);
-    }
-    m_loc[g]           = m_all;
-    const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
-    float       l_loc  = 0.0f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       o[g][e] = 0.0f;
     }
+  }
 #pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const float pr = fast_exp2(sc[p][g] - m_safe);
-      l_loc += pr;
+  for (int pp = 0; pp < PASSES / 2; ++pp) {
+    uint32_t pk[GH];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        o[g][e] += pr * (float) vreg[p][e];
+    for (int g = 0; g < GH; ++g) {
+      pk[g] = p_wave[(pp * KPW + kslot) * GH + g];
+    }
+    const uint4 va = __builtin_bit_cast(uint4, vreg[2 * pp]), vb = __builtin_bit_cast(uint4, vreg[2 * pp + 1]);
+    const uint32_t a4[4] = { va.x, va.y, va.z, va.w }, b4[4] = { vb.x, vb.y, vb.z, vb.w };
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      // (dim 2 e of both keys, dim 2 e + 1 of both keys)
+      const v2h lo = __builtin_bit_cast(v2h, __builtin_amdgcn_perm(b4[e], a4[e], 0x05040100u));
+      const v2h hi = __builtin_bit_cast(v2h, __builtin_amdgcn_perm(b4[e], a4[e], 0x07060302u));
+#pragma unroll
+      for (int g = 0; g < GH; ++g) {
+        const v2h p2  = __builtin_bit_cast(v2h, pk[g]);
+        o[g][2 * e]     = __builtin_amdgcn_fdot2(p2, lo, o[g][2 * e], false);
+        o[g][2 * e + 1] = __builtin_amdgcn_fdot2(p2, hi, o[g][2 * e + 1], false);
       }
     }
+  }
+  float l_w = l_run + __shfl_xor(l_run, 16, kWave);
+  l_w += __shfl_xor(l_w, 32, kWave);
+  if (kg == 0 && col < GH) {
+    red_m[wave * GH + col] = m_run;
+    red_l[wave * GH + col] = l_w;
+  }
+#pragma unroll
+  for (int g = 0; g < GH; ++g) {
     float4 *dst = reinterpret_cast<float4 *>(red_o + ((size_t) slot * GH + g) * D + sub * 8);
     dst[0]      = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
     dst[1]      = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
-    if (sub == 0) {
-      red_l[slot * GH + g] = l_loc;
-    }
   }
   __syncthreads();
-  // add the slots up: two neighbouring columns per thread
+  // add the slots up, each wave's with its factor: two neighbouring columns per thread
   for (int i = threadIdx.x * 2; i < GH * D; i += THREADS * 2) {
     const int g = i / D, d = i % D;
     if (head0_in_group + g >= group) {
       continue;
     }
-    float v0 = 0.0f, v1 = 0.0f;
+    float m_all = red_m[g];
 #pragma unroll
-    for (int w = 0; w < SLOTS; ++w) {
-      const float2 x = *reinterpret_cast<const float2 *>(red_o + ((size_t) w * GH + g) * D + d);
-      v0 += x.x, v1 += x.y;
+    for (int w = 1; w < WAVES; ++w) {
+      m_all = fmaxf(m_all, red_m[w * GH + g]);
+    }
+    const float m_ref = (m_all == -INFINITY) ? 0.0f : m_all;
+    float       v0 = 0.0f, v1 = 0.0f, l = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const float f = fast_exp2(red_m[w * GH + g] - m_ref);
+      l += red_l[w * GH + g] * f;
+      float x0 = 0.0f, x1 = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < KPW; ++ks) {
+        const float2 x = *reinterpret_cast<const float2 *>(red_o + ((size_t) (w * KPW + ks) * GH + g) * D + d);
+        x0 += x.x, x1 += x.y;
+      }
+      v0 += x0 * f, v1 += x1 * f;
     }
     const int head = h_kv * group + head0_in_group + g;
     float    *rec  = part + ((size_t) head * n_splits + split) * (D + 2);
     *reinterpret_cast<float2 *>(rec + 2 + d) = make_float2(v0, v1);
-  }
-  // (maximum, sum) of head g by wave g % WAVES: a slot's sum per lane, added up across the wave
-  static_assert(SLOTS <= kWave, "a lane per slot");
-#pragma unroll
-  for (int g = 0; g < GH; ++g) {
-    if (g % WAVES == wave && head0_in_group + g < group) {
-      const float l = wave_sum(lane < SLOTS ? red_l[lane * GH + g] : 0.0f);
-      if (lane == 0) {
-        float *rec = part + ((size_t) (h_kv * group + head0_in_group + g) * n_splits + split) * (D + 2);
-        *reinterpret_cast<float2 *>(rec) = make_float2(m_loc[g], l);
-      }
+    if (d == 0) {
+      *reinterpret_cast<float2 *>(rec) = make_float2(m_all, l);
     }
   }
 }
 
-// One workgroup per head, one thread per output column. Splits are taken 64 at a time with every load of a chunk -- the
-// (max, sum) pair of split `lane` and this thread's column of all 64 records -- requested before the first use, so a
-// chunk costs one trip to memory (kv_len up to 8192 at 128 keys per split: the whole merge is one trip). Each
-// wave works the rescale factors out for itself (lane s holds that of split s, read back with v_readlane), so there
-// is neither LDS nor a barrier; chunks are folded into a running (max, sum, column) like KV blocks are.
-constexpr int kMergeChunk = 64;
+// One workgroup per head: MG groups of D threads, one thread per output column in each; group j merges the j-th part
+// of the splits, then the groups' (max, sum, column) are put together through LDS (MG = 1: nothing to put together;
+// measured at 32 heads of 128: 32 splits 3.2 us with one group, 4.2 with four; 128 splits 5.7 and 4.0). A group takes its splits
+// 64 at a time with every load of a chunk -- the (max, sum) pair of split `lane` and this thread's column of all 64
+// records -- requested before the first use, so a chunk costs one trip to memory (kv_len up to 32768 at 128 keys per
+// split: the whole merge is one trip). Each wave works the rescale factors out for itself (lane s holds that of split
+// s, read back with v_readlane); chunks are folded into a running (max, sum, column) like KV blocks are.
+constexpr int kMergeChunk  = 64;
+constexpr int kMergeGroups = 4;  // for more than kMergeChunk splits
 
-
-template <int D, bool QO_F32>
-__global__ __launch_bounds__(D) void flash_attn_decode_merge_kernel(void *__restrict__ o_ptr,
-                                                                    const float *__restrict__ part, int n_splits,
-                                                                    uint8_t *__restrict__ q8_out) {
+template <int D, bool QO_F32, int MG>
+__global__ __launch_bounds__(D *MG) void flash_attn_decode_merge_kernel(void *__restrict__ o_ptr,
+                                                                        const float *__restrict__ part, int n_splits,
+                                                                        uint8_t *__restrict__ q8_out) {
   // (q8_out, fp32 output only: the output row is also written as Q8_0 blocks, the bytes the Q8_0 quantizer makes of
   // it; a block is 32 neighbouring columns, one half of a wave)
-  const int    head = blockIdx.x, d = threadIdx.x, lane = threadIdx.x & (kWave - 1);
+  extern __shared__ float merge_lds[];  // MG > 1 only: the groups' columns [MG][D], then their (max, sum) [MG][2]
+  static_assert(D % kWave == 0, "a wave lies in one group");
+  const int    head = blockIdx.x, d = threadIdx.x % D, lane = threadIdx.x & (kWave - 1);
+  // (the same for the whole wave, and known to be: the bounds below then stay in scalar registers and the 64 loads of a
+  // chunk are switched by scalar branches instead of one lane mask each)
+  const int    grp  = __builtin_amdgcn_readfirstlane((int) threadIdx.x / D);
   const float *rec0 = part + (size_t) head * n_splits * (D + 2);
+  const int    per  = (n_splits + MG - 1) / MG;  // splits of a group
+  const int    s_begin = grp * per, s_end = min(n_splits, s_begin + per);
   float        m_run = -INFINITY, l_run = 0.0f, v_run = 0.0f;
-  for (int s0 = 0; s0 < n_splits; s0 += kMergeChunk) {
-    const int  left = n_splits - s0;  // >= 1
+  for (int s0 = s_begin; s0 < s_end; s0 += kMergeChunk) {
+    const int  left = s_end - s0;  // >= 1
     const bool mine = lane < kMergeChunk && lane < left;
     float      m_s = -INFINITY, l_s = 0.0f;
     if (mine) {
@@ -693,6 +740,30 @@ __global__ __launch_bounds__(D) void flash_attn_decode_merge_kernel(void *__rest
     }
     v_run = v_run * keep + v;
     m_run = m_new;
+  }
+  if (MG > 1) {
+    float *grp_v = merge_lds, *grp_ml = merge_lds + MG * D;
+    grp_v[grp * D + d] = v_run;
+    if (d == 0) {
+      grp_ml[2 * grp] = m_run, grp_ml[2 * grp + 1] = l_run;
+    }
+    __syncthreads();
+    if (grp != 0) {
+      return;
+    }
+    float m_all = grp_ml[0];
+#pragma unroll
+    for (int j = 1; j < MG; ++j) {
+      m_all = fmaxf(m_all, grp_ml[2 * j]);
+    }
+    const float m_safe = (m_all == -INFINITY) ? 0.0f : m_all;
+    l_run = 0.0f, v_run = 0.0f;
+#pragma unroll
+    for (int j = 0; j < MG; ++j) {  // (a group without splits has m = -inf, l = v = 0)
+      const float f = fast_exp2(grp_ml[2 * j] - m_safe);
+      l_run += grp_ml[2 * j + 1] * f;
+      v_run += grp_v[j * D + d] * f;
+    }
   }
   const float out = v_run * (1.0f / l_run);
   if (QO_F32) {
@@ -900,8 +971,9 @@ template <int D, int GH, bool QO_F32, int SPLIT, int THREADS>
 hipError_t launch_decode_pass(hipStream_t stream, dim3 grid, float *workspace, const void *q, const void *k, const void *v,
                               const void *mask, int kv_len, int n_heads, int n_kv_heads, int h0, int n_splits,
                               bool mask_threshold) {
-  constexpr int    kSlots = (THREADS / kWave) * (kWave / (D / 8));
-  constexpr size_t kLds   = ((size_t) kSlots * GH * D + (size_t) kSlots * GH + (size_t) (THREADS / kWave) * GH) * sizeof(float);
+  constexpr int    kWaves = THREADS / kWave, kSlots = kWaves * (kWave / (D / 8));
+  // (the waves' O, their sums and maxima, the probabilities: a dword per pair of keys and head)
+  constexpr size_t kLds = ((size_t) kSlots * GH * D + 2 * (size_t) kWaves * GH + (size_t) (SPLIT / 2) * GH) * sizeof(float);
   static_assert(kLds <= 160 * 1024, "LDS of one compute unit");
   auto *kernel = flash_attn_decode_kernel<D, GH, QO_F32, SPLIT, THREADS>;
   if (kLds > 64 * 1024) {
@@ -918,7 +990,8 @@ hipError_t launch_decode_pass(hipStream_t stream, dim3 grid, float *workspace, c
 
 template <int D, bool QO_F32>
 hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void *k, const void *v, const void *mask,
-                         int kv_len, int n_heads, int n_kv_heads, float *workspace, void *q8_out, bool mask_threshold) {
+                         int kv_len, int n_heads, int n_kv_heads, float *workspace, void *q8_out, bool mask_threshold,
+                         int parts = 3) {  // (bit 0: the split-KV launch, bit 1: the merge launch)
   const int  group    = n_heads / n_kv_heads;
   // 64-key chunks while 128-key ones would give fewer than 128 workgroups (measured at 8 KV heads: kv = 512 8.8 -> 7.1 us;
   // kv = 4096 and 16384 are 1 and 6 us slower with 64)
@@ -926,7 +999,7 @@ hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void 
   const int  split    = short_kv ? kDecSplitShort : kDecSplit;
   const int  n_splits = (kv_len + split - 1) / split;
   const dim3 grid((unsigned) n_splits, (unsigned) n_kv_heads);
-  for (int h0 = 0; h0 < group; h0 += kDecMaxGroup) {
+  for (int h0 = 0; h0 < group && (parts & 1); h0 += kDecMaxGroup) {
     const int  gh = group - h0;
     hipError_t e;
 #define HTPOPS_DECODE(GH)                                                                                              \
@@ -950,8 +1023,18 @@ hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void 
       return e;
     }
   }
-  hipLaunchKernelGGL((flash_attn_decode_merge_kernel<D, QO_F32>), dim3((unsigned) n_heads), dim3(D), 0, stream, o,
-                     workspace, n_splits, QO_F32 ? static_cast<uint8_t *>(q8_out) : nullptr);
+  if (!(parts & 2)) {
+    return hipGetLastError();
+  }
+  uint8_t *q8 = QO_F32 ? static_cast<uint8_t *>(q8_out) : nullptr;
+  if (n_splits > kMergeChunk) {
+    hipLaunchKernelGGL((flash_attn_decode_merge_kernel<D, QO_F32, kMergeGroups>), dim3((unsigned) n_heads),
+                       dim3(D * kMergeGroups), (size_t) kMergeGroups * (D + 2) * sizeof(float), stream, o, workspace,
+                       n_splits, q8);
+  } else {
+    hipLaunchKernelGGL((flash_attn_decode_merge_kernel<D, QO_F32, 1>), dim3((unsigned) n_heads), dim3(D), 0, stream, o,
+                       workspace, n_splits, q8);
+  }
   return hipGetLastError();
 }
 
@@ -967,6 +1050,21 @@ size_t flash_attn_workspace_bytes(int qo_len, int kv_len, int n_heads, int head_
   }
   const size_t n_splits = ((size_t) kv_len + kDecSplitShort - 1) / kDecSplitShort;  // the most there can be
   return (size_t) n_heads * n_splits * ((size_t) head_dim + 2) * sizeof(float);
+}
+
+hipError_t launch_flash_attn_decode_part(hipStream_t stream, int part, void *o, const void *q, const void *k,
+                                         const void *v, int kv_len, int n_heads, int n_kv_heads, int head_dim,
+                                         bool qo_is_f32, void *workspace) {
+  if ((head_dim != 64 && head_dim != 128) || (part != 1 && part != 2) || !workspace) {
+    return hipErrorNotSupported;
+  }
+  float *ws = static_cast<float *>(workspace);
+  if (head_dim == 128) {
+    return qo_is_f32 ? launch_decode<128, true>(stream, o, q, k, v, nullptr, kv_len, n_heads, n_kv_heads, ws, nullptr, false, part) :
+                       launch_decode<128, false>(stream, o, q, k, v, nullptr, kv_len, n_heads, n_kv_heads, ws, nullptr, false, part);
+  }
+  return qo_is_f32 ? launch_decode<64, true>(stream, o, q, k, v, nullptr, kv_len, n_heads, n_kv_heads, ws, nullptr, false, part) :
+                     launch_decode<64, false>(stream, o, q, k, v, nullptr, kv_len, n_heads, n_kv_heads, ws, nullptr, false, part);
 }
 
 hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const void *k, const void *v,

@@ -151,6 +151,11 @@ hipError_t launch_flash_attn(hipStream_t stream, void *o, const void *q, const v
                              const void *mask, int qo_len, int kv_len, int n_heads, int n_kv_heads, int head_dim,
                              bool qo_is_f32, bool causal, void *workspace, void *q8_out, int forced_key_groups,
                              bool mask_threshold);
+// One of the two launches of one-token attention by itself, for timing: part 1 = the split-KV launch (writes the
+// partial records into `workspace`), part 2 = the merge launch (reads them). Same arguments as above otherwise.
+hipError_t launch_flash_attn_decode_part(hipStream_t stream, int part, void *o, const void *q, const void *k,
+                                         const void *v, int kv_len, int n_heads, int n_kv_heads, int head_dim,
+                                         bool qo_is_f32, void *workspace);
 bool       flash_attn_writes_q8_0(int qo_len, int head_dim, bool qo_is_f32);
 
 // What the calling thread's most recent launch of the one-row matmul kernel was: kernel instance and geometry. The bench

@@ -59,6 +59,7 @@ EXPORTED_SYMBOLS = [
     "htpops_flash_attn_ptr", "htpops_flash_attn_noalloc_ptr", "htpops_timer_start", "htpops_timer_stop", "htpops_timer_elapsed_ms",
     "htpops_measure_mfma_peak", "htpops_measure_copy_bandwidth", "htpops_measure_read_us", "htpops_last_gemv_launch",
     "htpops_measure_host_walk_us",
+    "htpops_measure_decode_attention_parts",
 ]
 
 
@@ -126,6 +127,9 @@ def load_library(path=None):
         "htpops_measure_read_us": (ci, [vp, sz, ci, ci, ctypes.POINTER(ctypes.c_double)]),
         "htpops_last_gemv_launch": (ci, [vp, ctypes.c_char_p, sz]),
         "htpops_measure_host_walk_us": (ci, [vp, vp, sz, ci, ctypes.POINTER(ctypes.c_double)]),
+        "htpops_measure_decode_attention_parts": (ci, [vp, vp, vp, ctypes.POINTER(vp), ctypes.POINTER(vp), ci, ci, ci, ci, ci,
+                                                       ci, ci, ctypes.POINTER(ctypes.c_double),
+                                                       ctypes.POINTER(ctypes.c_double)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -380,6 +384,18 @@ class Context:
         self._check(self.lib.htpops_measure_host_walk_us(self._ctx, ctypes.cast(buf, ctypes.c_void_p), len(msg), iters,
                                                          ctypes.byref(v)))
         return float(v.value)
+
+    def measure_decode_attention_parts(self, o, q, ks, vs, kv_len, n_heads, n_kv_heads, head_dim, qo_is_f32, iters=100):
+        """(split-KV launch, merge launch) of one-token attention in microseconds per launch; o, q, ks[i], vs[i] are
+        buffer handles."""
+        n = len(ks)
+        kp = (ctypes.c_void_p * n)(*[self.device_ptr(h) for h in ks])
+        vpp = (ctypes.c_void_p * n)(*[self.device_ptr(h) for h in vs])
+        a, b = ctypes.c_double(), ctypes.c_double()
+        self._check(self.lib.htpops_measure_decode_attention_parts(
+            self._ctx, ctypes.c_void_p(self.device_ptr(o)), ctypes.c_void_p(self.device_ptr(q)), kp, vpp, n, kv_len,
+            n_heads, n_kv_heads, head_dim, int(qo_is_f32), iters, ctypes.byref(a), ctypes.byref(b)))
+        return float(a.value), float(b.value)
 
     def measure_copy_bandwidth(self, nbytes, iters=20):
         v = ctypes.c_double()

@@ -44,6 +44,14 @@ int htpops_last_gemv_launch(htpops_context *ctx, char *text, size_t cap);
 int htpops_measure_host_walk_us(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes, int iters,
                                 double *us_per_message);
 
+/* The two launches of one-token attention (head_dim 64 or 128, no mask) timed by themselves: `iters` launches of the
+ * split-KV kernel in a row, then `iters` of the merge kernel, each between two events on the context's stream, in
+ * microseconds per launch. o, q and the `sets` K/V pairs (ks[i], vs[i], read in turn) are device pointers laid out as
+ * for htpops_flash_attn_ptr; the partial records go to the context's workspace. */
+int htpops_measure_decode_attention_parts(htpops_context *ctx, void *o, const void *q, const void *const *ks,
+                                          const void *const *vs, int sets, int kv_len, int n_heads, int n_kv_heads,
+                                          int head_dim, int qo_is_f32, int iters, double *split_us, double *merge_us);
+
 #ifdef __cplusplus
 }
 #endif

@@ -38,6 +38,10 @@ CASES = [
     # decode on both sides of the switch between 64- and 128-key chunks (128 workgroups of 128 keys)
     (1, 64, 8, 8, 128), (1, 65, 8, 2, 64), (1, 2048, 32, 8, 128), (1, 1920, 32, 8, 128), (1, 1900, 16, 4, 64),
     (1, 2100, 16, 16, 64),
+    # decode long enough for a workgroup to walk several chunks of keys (about one workgroup per compute unit): ragged
+    # last workgroup, odd and even chunk counts, every group width, both head dims
+    (1, 4100, 32, 32, 128), (1, 9000, 16, 8, 64), (1, 6000, 12, 12, 128), (1, 20000, 12, 4, 128), (1, 9000, 48, 8, 64),
+    (1, 12500, 32, 8, 128),
     # head dims other than 64 and 128 (the reference's flash_attn_sp_hdim.c domain: any even head_dim)
     (1, 300, 8, 2, 80), (7, 133, 4, 2, 96), (33, 70, 6, 3, 40), (1, 1, 2, 1, 2), (20, 517, 4, 1, 256), (3, 64, 2, 2, 112),
     (1, 1000, 4, 4, 192), (65, 65, 2, 1, 30),
