@@ -441,88 +441,82 @@ __global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(
 
 // ------------------------------------------------------------------------------------------------ decode
 
-constexpr int kDecThreads  = 256;
+constexpr int kDecWaveKeys = 32;  // keys of one wave: two 16-key score tiles = one k step of P V
 constexpr int kDecMaxGroup = 8;   // query heads scored per pass against one K/V stream
-constexpr int kDecSplit    = 128; // keys per workgroup ...
-constexpr int kDecSplitShort = 64;  // ... and for short contexts, where 128 would leave most CUs without a workgroup
-
-// sum over the 16 (or 8) consecutive lanes of a key group with DPP row operations; every lane gets the sum
-template <int LPK>
-__device__ __forceinline__ float key_group_sum(float v) {
-#define HTPOPS_DPP_ADD(ctrl) v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, 0xf, 0xf, false))
-  HTPOPS_DPP_ADD(0xB1);   // quad_perm [1,0,3,2]
-  HTPOPS_DPP_ADD(0x4E);   // quad_perm [2,3,0,1]
-  HTPOPS_DPP_ADD(0x141);  // row_half_mirror: 8 lanes
-  if (LPK == 16) {
-    HTPOPS_DPP_ADD(0x140);  // row_mirror: 16 lanes
-  }
-#undef HTPOPS_DPP_ADD
-  return v;
-}
+constexpr int kDecSplit    = 128; // keys per workgroup (four waves) ...
+constexpr int kDecSplitShort = 64;  // ... and for short contexts (two waves), where 128 would leave most CUs without a workgroup
 
 // partial record per (head, split): m, l, then D floats of un-normalised O.
-// A workgroup of THREADS threads owns SPLIT consecutive keys of one KV head; each wave owns SPLIT / WAVES of them and
-// works without the others until the end. Every K and V load of the wave is issued before the first use.
-//  * scores: S = K Q^T on the matrix cores (v_mfma_f32_16x16x32_f16: 16 keys x up to 16 heads of the GQA group, the
-//    head dimension as k), K in the A operand as it lies in memory (a lane loads 16 bytes of a key row per k step), the
-//    queries of the group, scaled and rounded to fp16 like the prefill kernel's, in the B operand. A lane then holds the
-//    scores of 4 keys for one head per tile.
-//  * softmax against the wave's own maximum; the probabilities go through LDS (fp16, pairs of keys in a dword) to
-//  * O += P V on the vector ALU with v_dot2_f32_f16 (two keys per instruction, exact products, fp32 sums): LPK = D / 8
-//    lanes share a key, each with 16 bytes of its V row, all heads of the group against the same V registers.
+// A workgroup owns SPLIT consecutive keys of one KV head; each of its SPLIT / 32 waves owns 32 of them and works
+// without the others until the end. Both products run on the matrix cores (v_mfma_f32_16x16x32_f16), with up to 16
+// query heads of the GQA group as the 16 rows (columns) of a tile:
+//  * scores S = K Q^T: K in the A operand as it lies in memory (a lane loads 16 bytes of a key row per k step, all of
+//    a wave's K loads issued before the first use); the queries in the B operand, fp32 queries scaled and split into an
+//    fp16 pair (two instructions per k step: the scores are those of the fp32 queries to about 2^-22), fp16 queries as
+//    they are with the scale applied to the score. A lane then holds, for one head, the scores of 4 keys per tile.
+//  * softmax against the wave's own maximum, in those registers; rounded to fp16 they ARE the A operand of
+//  * O = P V: the contraction runs over the wave's 32 keys, key 16 t + 4 g + i (tile t, lane group g, register i)
+//    in k slot 8 g + 4 t + i. V is the B operand: a lane needs 8 keys at one column. The V rows come into LDS as they
+//    are by DMA (global_load_lds, no registers), and ds_read_b64_tr_b16 hands each lane of a 16-lane group one column
+//    of the 4 rows x 16 columns that the group's lanes point at (lanes 4 j .. 4 j + 3 at the four 8-byte pieces of
+//    row j). Within a row the 32-byte pieces are stored exclusive-or'ed with the row number's low bits (the DMA
+//    chooses what each lane fetches, not where it lands), so the four rows of a read lie in different banks.
 // The waves' (max, sum, O) are put together through LDS with the factor exp2(m_wave - m_all) per wave and head.
-// Measured on MI355X (32 query / 8 KV heads of 128, cold K/V) against the earlier all-vector-ALU version of this kernel
-// (8 multiply-adds, 4 lane exchanges and an exponential per key, head and lane: about 1000 vector instructions per
-// wave, which at kv_len 16384 kept the vector ALUs busy for longer than the K/V stream takes): see the table in the
-// launcher. Merging inside this launch -- records written through, a ticket per KV head, the last workgroup merges
-// -- was slower (18-19 us, 47 us at kv_len 16384).
-// (A variant in which a workgroup walks several chunks of SPLIT keys, the next chunk's K and V on their way while one is
-// worked on, about one workgroup per compute unit, was slower at kv_len 16384: 17.0 against 15.1 us.)
-template <int D, int GH, bool QO_F32, int SPLIT, int THREADS>
-__global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__restrict__ part,
-                                                                    const void *__restrict__ q_ptr,
-                                                                    const _Float16 *__restrict__ k_ptr,
-                                                                    const _Float16 *__restrict__ v_ptr,
-                                                                    const _Float16 *__restrict__ mask, int kv_len,
-                                                                    int n_heads, int n_kv_heads, int head0_in_group,
-                                                                    int n_splits, int mask_threshold) {
-  constexpr int LPK    = D / 8;        // lanes per key in the P V part (8 halfs = 16 bytes of the V row each)
-  constexpr int KPW    = kWave / LPK;  // keys per wave per pass
-  constexpr int WAVES  = THREADS / kWave;
-  constexpr int SLOTS  = WAVES * KPW;  // independent partial streams in the workgroup
-  constexpr int PASSES = SPLIT / SLOTS;
-  constexpr int TILE_PASSES = 16 / KPW;            // passes that make a 16-key score tile
-  constexpr int TILES       = PASSES / TILE_PASSES;  // score tiles of a wave
-  constexpr int KSTEPS      = D / 32;              // k steps of a score tile
-  static_assert(SPLIT % SLOTS == 0 && PASSES >= 2 && PASSES % 2 == 0 && PASSES % TILE_PASSES == 0, "whole tiles, pairs of passes");
-  static_assert(GH <= 16, "the heads of a pass are the columns of one score tile");
+// Measured on MI355X (32 query / 8 KV heads of 128, cold K/V; the split-KV launch alone, kv_len 4096 / 16384): all on
+// the vector ALU (8 multiply-adds, 4 lane exchanges and an exponential per key, head and lane) 7.5 / 17.0 us; scores on
+// the matrix cores and P V with v_dot2_f32_f16 6.3 / 15.3 us; this version: see the launcher. A variant in which a
+// workgroup walks several chunks of keys with the next chunk on its way, about one workgroup per compute unit, was
+// slower (17.0 us at 16384), and so was merging inside this launch behind a ticket per KV head (18-19 us at 4096).
+template <int D, int GH, bool QO_F32, int SPLIT>
+__global__ __launch_bounds__(SPLIT / kDecWaveKeys * kWave) void flash_attn_decode_kernel(
+  float *__restrict__ part, const void *__restrict__ q_ptr, const _Float16 *__restrict__ k_ptr,
+  const _Float16 *__restrict__ v_ptr, const _Float16 *__restrict__ mask, int kv_len, int n_heads, int n_kv_heads,
+  int head0_in_group, int n_splits, int mask_threshold) {
+  constexpr int WAVES   = SPLIT / kDecWaveKeys;
+  constexpr int THREADS = WAVES * kWave;
+  constexpr int KSTEPS  = D / 32;  // k steps of a score tile
+  constexpr int CT      = D / 16;  // 16-column tiles of O
+  constexpr int ROWB    = D * 2;   // bytes of a K or V row
+  constexpr int CHUNKS  = ROWB / 16;            // 16-byte pieces of a row
+  constexpr int DMA_ROWS = 1024 / ROWB;         // rows per DMA instruction (1 KiB)
+  constexpr int DMAS    = kDecWaveKeys / DMA_ROWS;
+  static_assert(GH <= 16 && (D == 64 || D == 128), "heads are the 16 rows of a tile");
   typedef float v4f __attribute__((ext_vector_type(4)));
-  // red_o[SLOTS][GH][D], red_l[WAVES][GH], red_m[WAVES][GH], then per wave the probabilities [PASSES / 2][KPW][GH] dwords
-  extern __shared__ float dec_lds[];
-  float    *red_o = dec_lds, *red_l = dec_lds + SLOTS * GH * D, *red_m = red_l + WAVES * GH;
-  uint32_t *p_sh  = reinterpret_cast<uint32_t *>(red_m + WAVES * GH);
+  typedef short v4s __attribute__((ext_vector_type(4)));
+  // LDS: V rows [SPLIT][D] halfs (wave w: rows 32 w ..), then o_w[WAVES][GH][D], red_l[WAVES][GH], red_m[WAVES][GH]
+  extern __shared__ __align__(1024) uint8_t dec_lds[];
+  float *o_sh  = reinterpret_cast<float *>(dec_lds + SPLIT * ROWB);
+  float *red_l = o_sh + WAVES * GH * D, *red_m = red_l + WAVES * GH;
 
   const int group = n_heads / n_kv_heads;
   const int h_kv  = blockIdx.y;
   const int split = blockIdx.x;
-  const int lane  = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int sub   = lane % LPK;  // P V part: which 8 dims
-  const int kslot = lane / LPK;  // P V part: which key of the pass
-  const int slot  = wave * KPW + kslot;
-  const int col   = lane & 15;   // score part: which head of the pass
-  const int kg    = lane >> 4;   // score part: which 8 of a k step's 32 dims; rows 4 kg .. 4 kg + 3 of the result
+  const int lane  = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int col   = lane & 15;   // head of the pass (scores, P), column of the tile (V, O)
+  const int kg    = lane >> 4;   // lane group: which 8 of a k step's 32 slots; rows 4 kg .. 4 kg + 3 of a result
   const float scale = (1.0f / sqrtf((float) D)) * kLog2e;
   const size_t kv_stride = (size_t) n_kv_heads * D;
 
-  const int k_begin = split * SPLIT;
-  const int k_end   = min(kv_len, k_begin + SPLIT);
-  // key of (pass, key slot of this wave); keys from k_end on are read as key k_end - 1 and score -inf
-  auto key_of = [&](int pass, int ks) { return k_begin + pass * SLOTS + wave * KPW + ks; };
+  const int k_end  = min(kv_len, (split + 1) * SPLIT);
+  const int k_wave = split * SPLIT + wave * kDecWaveKeys;  // this wave's keys: k_wave + 0 .. 31; keys from k_end on are
+                                                           // read as key k_end - 1 and score -inf
 
-  // the queries first (loads return in order): head `col` of the pass, dims 32 s + 8 kg .. + 7; fp32 queries are scaled
-  // before they are rounded, and what the rounding leaves over goes into a second operand (a second matrix
-  // instruction per k step: the scores are those of the fp32 queries to about 2^-22); fp16 queries stay as they are
-  // and the scale is applied to the score
+  // V first (loads return in order: the K loads the compiler counts are then the youngest, and its waits for them
+  // also cover these). DMA instruction i brings rows DMA_ROWS i .. of the wave's 32; lane L lands at byte 16 L of
+  // that KiB = row L / CHUNKS, piece L % CHUNKS, and fetches the piece that belongs there.
+  uint8_t *v_wave = dec_lds + wave * kDecWaveKeys * ROWB;
+  {
+    const uint32_t to = (uint32_t) (uintptr_t) v_wave;
+#pragma unroll
+    for (int i = 0; i < DMAS; ++i) {
+      const int row   = i * DMA_ROWS + lane / CHUNKS;
+      const int piece = (lane % CHUNKS) ^ (2 * (row & 3));  // (32-byte pieces exclusive-or'ed with the row's low bits)
+      const int key   = min(k_wave + row, k_end - 1);
+      const _Float16 *src = v_ptr + (size_t) key * kv_stride + (size_t) h_kv * D + 8 * piece;
+      asm volatile("s_mov_b32 m0, %1\n s_nop 0\n global_load_lds_dwordx4 %0, off" ::"v"(src), "s"(to + (uint32_t) (i * 1024)) : "memory");
+    }
+  }
+  // the queries: head `col` of the pass, dims 32 s + 8 kg .. + 7
   v8h qf[KSTEPS], qf_lo[KSTEPS];
   {
     const bool   q_on = col < GH && head0_in_group + col < group;
@@ -546,30 +540,33 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
       }
     }
   }
-  // all K (score layout: row `col` of tile t is key slot col % KPW of pass t TILE_PASSES + col / KPW) and all V (P V
-  // layout) of this lane, requested up front
-  v8h kf[TILES][KSTEPS], vreg[PASSES];
+  // K: row `col` of tile t is key 16 t + col of the wave
+  v8h kf[2][KSTEPS];
 #pragma unroll
-  for (int t = 0; t < TILES; ++t) {
-    const int    key = min(key_of(t * TILE_PASSES + col / KPW, col % KPW), k_end - 1);
+  for (int t = 0; t < 2; ++t) {
+    const int    key = min(k_wave + 16 * t + col, k_end - 1);
     const size_t off = (size_t) key * kv_stride + (size_t) h_kv * D + 8 * kg;
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
       kf[t][s] = *reinterpret_cast<const v8h *>(k_ptr + off + 32 * s);
     }
   }
+  // row 0 of the mask (qo_len == 1) for the 8 keys of this lane, requested with the rest
+  float mk[2][4];
 #pragma unroll
-  for (int p = 0; p < PASSES; ++p) {
-    const int    key = min(key_of(p, kslot), k_end - 1);
-    const size_t off = (size_t) key * kv_stride + (size_t) h_kv * D + sub * 8;
-    vreg[p]          = *reinterpret_cast<const v8h *>(v_ptr + off);
+  for (int t = 0; t < 2; ++t) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int key = k_wave + 16 * t + 4 * kg + i;
+      mk[t][i] = (mask && key < k_end) ? mask_term(mask[key], mask_threshold != 0) : 0.0f;
+    }
   }
 
-  // scores of this lane: head `col`, rows 4 kg + i of every tile
-  float sc[TILES][4];
-  float m_run = -INFINITY;
+  // scores of head `col` for keys 16 t + 4 kg + i
+  float sc[2][4];
+  float m_w = -INFINITY;
 #pragma unroll
-  for (int t = 0; t < TILES; ++t) {
+  for (int t = 0; t < 2; ++t) {
     v4f acc = { 0.0f, 0.0f, 0.0f, 0.0f };
 #pragma unroll
     for (int s = 0; s < KSTEPS; ++s) {
@@ -580,82 +577,70 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int  row  = 4 * kg + i;
-      const int  key  = key_of(t * TILE_PASSES + row / KPW, row % KPW);
-      const bool live = key < k_end;
-      const float mk  = (mask && live) ? mask_term(mask[key], mask_threshold != 0) : 0.0f;  // row 0 of the mask (qo_len == 1)
-      const float v   = (QO_F32 ? acc[i] : acc[i] * scale) + mk;
-      sc[t][i]        = live ? v : -INFINITY;
-      m_run           = fmaxf(m_run, sc[t][i]);
+      const bool  live = k_wave + 16 * t + 4 * kg + i < k_end;
+      const float v    = (QO_F32 ? acc[i] : acc[i] * scale) + mk[t][i];
+      sc[t][i]         = live ? v : -INFINITY;
+      m_w              = fmaxf(m_w, sc[t][i]);
     }
   }
-  // the wave's maximum of head `col`: over the four row groups
-  m_run = fmaxf(m_run, __shfl_xor(m_run, 16, kWave));
-  m_run = fmaxf(m_run, __shfl_xor(m_run, 32, kWave));
-  const float m_safe = (m_run == -INFINITY) ? 0.0f : m_run;
-  float       l_run  = 0.0f;  // (the sum of head `col`, still spread over the four row groups)
-  uint32_t   *p_wave = p_sh + wave * (PASSES / 2) * KPW * GH;
+  // the wave's maximum of head `col`: over the four lane groups
+  m_w = fmaxf(m_w, __shfl_xor(m_w, 16, kWave));
+  m_w = fmaxf(m_w, __shfl_xor(m_w, 32, kWave));
+  const float m_safe = (m_w == -INFINITY) ? 0.0f : m_w;
+  float       l_w    = 0.0f;
+  v8h         pf;  // A operand of P V: k slot 8 kg + 4 t + i
 #pragma unroll
-  for (int t = 0; t < TILES; ++t) {
+  for (int t = 0; t < 2; ++t) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const float pr = fast_exp2(sc[t][i] - m_safe);
-      l_run += pr;
-      const int row = 4 * kg + i, pass = t * TILE_PASSES + row / KPW, ks = row % KPW;
-      if (col < GH) {
-        reinterpret_cast<_Float16 *>(p_wave + ((pass >> 1) * KPW + ks) * GH + col)[pass & 1] = (_Float16) pr;
-      }
+      l_w += pr;
+      pf[4 * t + i] = (_Float16) pr;
     }
   }
-  // (LDS serves a wave's accesses in order: the reads below see the wave's own writes above; no other wave touches
-  // this part of LDS)
-  __builtin_amdgcn_wave_barrier();
-
-  // O += P V for the key slot and the 8 dims of this lane, all heads, two passes (keys) per instruction
-  float o[GH][8];
-#pragma unroll
-  for (int g = 0; g < GH; ++g) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      o[g][e] = 0.0f;
-    }
-  }
-#pragma unroll
-  for (int pp = 0; pp < PASSES / 2; ++pp) {
-    uint32_t pk[GH];
-#pragma unroll
-    for (int g = 0; g < GH; ++g) {
-      pk[g] = p_wave[(pp * KPW + kslot) * GH + g];
-    }
-    const uint4 va = __builtin_bit_cast(uint4, vreg[2 * pp]), vb = __builtin_bit_cast(uint4, vreg[2 * pp + 1]);
-    const uint32_t a4[4] = { va.x, va.y, va.z, va.w }, b4[4] = { vb.x, vb.y, vb.z, vb.w };
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      // (dim 2 e of both keys, dim 2 e + 1 of both keys)
-      const v2h lo = __builtin_bit_cast(v2h, __builtin_amdgcn_perm(b4[e], a4[e], 0x05040100u));
-      const v2h hi = __builtin_bit_cast(v2h, __builtin_amdgcn_perm(b4[e], a4[e], 0x07060302u));
-#pragma unroll
-      for (int g = 0; g < GH; ++g) {
-        const v2h p2  = __builtin_bit_cast(v2h, pk[g]);
-        o[g][2 * e]     = __builtin_amdgcn_fdot2(p2, lo, o[g][2 * e], false);
-        o[g][2 * e + 1] = __builtin_amdgcn_fdot2(p2, hi, o[g][2 * e + 1], false);
-      }
-    }
-  }
-  float l_w = l_run + __shfl_xor(l_run, 16, kWave);
+  l_w += __shfl_xor(l_w, 16, kWave);
   l_w += __shfl_xor(l_w, 32, kWave);
   if (kg == 0 && col < GH) {
-    red_m[wave * GH + col] = m_run;
+    red_m[wave * GH + col] = m_w;
     red_l[wave * GH + col] = l_w;
   }
+
+  // O = P V. (Every load of this wave has returned by now: the K loads were the youngest. The wait is written out
+  // because the compiler knows nothing of the DMA.) Read h of tile c: lane (group kg, col = 4 j + q) points at row
+  // 16 h + 4 kg + j, halfs 16 c + 4 q .. + 3, and receives column 16 c + col of rows 16 h + 4 kg + 0 .. 3.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  v4f oacc[CT];
+  {
+    const int j = col >> 2, q = col & 3;
 #pragma unroll
-  for (int g = 0; g < GH; ++g) {
-    float4 *dst = reinterpret_cast<float4 *>(red_o + ((size_t) slot * GH + g) * D + sub * 8);
-    dst[0]      = make_float4(o[g][0], o[g][1], o[g][2], o[g][3]);
-    dst[1]      = make_float4(o[g][4], o[g][5], o[g][6], o[g][7]);
+    for (int c = 0; c < CT; ++c) {
+      v4s b[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int row   = 16 * h + 4 * kg + j;
+        const int piece = (2 * c + (q >> 1)) ^ (2 * (row & 3));
+        const uint8_t *at = v_wave + row * ROWB + piece * 16 + 8 * (q & 1);
+        b[h] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3))) *) at);
+      }
+      const v8h bf = __builtin_bit_cast(v8h, (short __attribute__((ext_vector_type(8)))){ b[0][0], b[0][1], b[0][2], b[0][3],
+                                                                                           b[1][0], b[1][1], b[1][2], b[1][3] });
+      const v4f zero = { 0.0f, 0.0f, 0.0f, 0.0f };
+      oacc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pf, bf, zero, 0, 0, 0);
+    }
+  }
+  // rows 4 kg + i of the result are heads: this lane's column 16 c + col of each
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int g = 4 * kg + i;
+    if (g < GH) {
+#pragma unroll
+      for (int c = 0; c < CT; ++c) {
+        o_sh[((size_t) wave * GH + g) * D + 16 * c + col] = oacc[c][i];
+      }
+    }
   }
   __syncthreads();
-  // add the slots up, each wave's with its factor: two neighbouring columns per thread
+  // put the waves together, each with its factor: two neighbouring columns per thread
   for (int i = threadIdx.x * 2; i < GH * D; i += THREADS * 2) {
     const int g = i / D, d = i % D;
     if (head0_in_group + g >= group) {
@@ -670,15 +655,10 @@ __global__ __launch_bounds__(THREADS) void flash_attn_decode_kernel(float *__res
     float       v0 = 0.0f, v1 = 0.0f, l = 0.0f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) {
-      const float f = fast_exp2(red_m[w * GH + g] - m_ref);
+      const float  f = fast_exp2(red_m[w * GH + g] - m_ref);
+      const float2 x = *reinterpret_cast<const float2 *>(o_sh + ((size_t) w * GH + g) * D + d);
       l += red_l[w * GH + g] * f;
-      float x0 = 0.0f, x1 = 0.0f;
-#pragma unroll
-      for (int ks = 0; ks < KPW; ++ks) {
-        const float2 x = *reinterpret_cast<const float2 *>(red_o + ((size_t) (w * KPW + ks) * GH + g) * D + d);
-        x0 += x.x, x1 += x.y;
-      }
-      v0 += x0 * f, v1 += x1 * f;
+      v0 += x.x * f, v1 += x.y * f;
     }
     const int head = h_kv * group + head0_in_group + g;
     float    *rec  = part + ((size_t) head * n_splits + split) * (D + 2);
@@ -967,24 +947,17 @@ hipError_t launch_prefill(hipStream_t stream, void *o, const void *q, const void
   return hipGetLastError();
 }
 
-template <int D, int GH, bool QO_F32, int SPLIT, int THREADS>
+template <int D, int GH, bool QO_F32, int SPLIT>
 hipError_t launch_decode_pass(hipStream_t stream, dim3 grid, float *workspace, const void *q, const void *k, const void *v,
                               const void *mask, int kv_len, int n_heads, int n_kv_heads, int h0, int n_splits,
                               bool mask_threshold) {
-  constexpr int    kWaves = THREADS / kWave, kSlots = kWaves * (kWave / (D / 8));
-  // (the waves' O, their sums and maxima, the probabilities: a dword per pair of keys and head)
-  constexpr size_t kLds = ((size_t) kSlots * GH * D + 2 * (size_t) kWaves * GH + (size_t) (SPLIT / 2) * GH) * sizeof(float);
-  static_assert(kLds <= 160 * 1024, "LDS of one compute unit");
-  auto *kernel = flash_attn_decode_kernel<D, GH, QO_F32, SPLIT, THREADS>;
-  if (kLds > 64 * 1024) {
-    static const hipError_t raised =
-      hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int) kLds);
-    if (raised != hipSuccess) {
-      return raised;
-    }
-  }
-  hipLaunchKernelGGL(kernel, grid, dim3(THREADS), kLds, stream, workspace, q, (const _Float16 *) k, (const _Float16 *) v,
-                     (const _Float16 *) mask, kv_len, n_heads, n_kv_heads, h0, n_splits, mask_threshold ? 1 : 0);
+  constexpr int    kWaves = SPLIT / kDecWaveKeys;
+  // (the V rows; the waves' O, their sums and maxima)
+  constexpr size_t kLds = (size_t) SPLIT * D * 2 + ((size_t) kWaves * GH * D + 2 * (size_t) kWaves * GH) * sizeof(float);
+  static_assert(kLds <= 64 * 1024, "dynamic LDS without raising the limit");
+  hipLaunchKernelGGL((flash_attn_decode_kernel<D, GH, QO_F32, SPLIT>), grid, dim3(kWaves * kWave), kLds, stream, workspace,
+                     q, (const _Float16 *) k, (const _Float16 *) v, (const _Float16 *) mask, kv_len, n_heads, n_kv_heads,
+                     h0, n_splits, mask_threshold ? 1 : 0);
   return hipGetLastError();
 }
 
@@ -1002,13 +975,11 @@ hipError_t launch_decode(hipStream_t stream, void *o, const void *q, const void 
   for (int h0 = 0; h0 < group && (parts & 1); h0 += kDecMaxGroup) {
     const int  gh = group - h0;
     hipError_t e;
-#define HTPOPS_DECODE(GH)                                                                                              \
-  e = short_kv ? launch_decode_pass<D, GH, QO_F32, kDecSplitShort, kDecThreads>(stream, grid, workspace, q, k, v, mask, \
-                                                                               kv_len, n_heads, n_kv_heads, h0,        \
-                                                                               n_splits, mask_threshold) :             \
-                 launch_decode_pass<D, GH, QO_F32, kDecSplit, kDecThreads>(stream, grid, workspace, q, k, v, mask,  \
-                                                                              kv_len, n_heads, n_kv_heads, h0, n_splits, \
-                                                                              mask_threshold)
+#define HTPOPS_DECODE(GH)                                                                                           \
+  e = short_kv ? launch_decode_pass<D, GH, QO_F32, kDecSplitShort>(stream, grid, workspace, q, k, v, mask, kv_len, n_heads, \
+                                                                  n_kv_heads, h0, n_splits, mask_threshold) :      \
+                 launch_decode_pass<D, GH, QO_F32, kDecSplit>(stream, grid, workspace, q, k, v, mask, kv_len, n_heads,  \
+                                                              n_kv_heads, h0, n_splits, mask_threshold)
     if (gh > 4) {
       HTPOPS_DECODE(8);
     } else if (gh > 2) {
