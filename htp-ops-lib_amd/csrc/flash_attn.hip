@@ -10,14 +10,19 @@
 //  * prefill (any qo_len, head_dim 64 or 128): one workgroup = 32 query rows x up to 4 query heads of one KV head (one
 //    wave per head, so a K/V tile staged in LDS serves the whole GQA group). Scores are computed transposed,
 //    S^T = K Q^T with v_mfma_f32_32x32x16_f16, which puts one query per lane: row max / row sum are register
-//    reductions plus one exchange between the two lane halves. O^T += V^T P^T uses V transposed on its way into LDS;
-//    P goes from the score registers straight into the MFMA B operand. The next K/V block is fetched into registers
-//    while the current one is used; scores are accumulated on top of minus the running maximum, so most blocks need
-//    no rescaling. Under `causal`, KV blocks above the diagonal are skipped and the longest query blocks start first.
+//    reductions plus one exchange between the two lane halves. K and V blocks come into LDS as they lie in memory, by
+//    DMA (global_load_lds) into two buffers that take turns: the next block is on its way while one is used. V^T for
+//    O^T += V^T P^T is read out of the row-major tile with the transposing LDS read (ds_read_b64_tr_b16); P goes from
+//    the score registers straight into the MFMA B operand. Scores are accumulated on top of minus the running
+//    maximum, so most blocks need no rescaling. Under `causal`, KV blocks above the diagonal are skipped and the
+//    longest query blocks start first. Timing-only builds on the 256-CU device (2048 x 2048 causal, 32 / 8 heads of
+//    128: 59 us) put the kernel without any matrix instruction and without the exponentials at 39 us, without the DMA
+//    at 51 us: every wave reads the whole K and V tile out of LDS for its 32 queries (1 KiB per matrix instruction:
+//    LDS bandwidth would be exhausted at the matrix cores' full rate), and that traffic, not the arithmetic, sets the
+//    pace.
 //  * decode (qo_len == 1, head_dim 64 or 128): bandwidth bound. The KV range is split across workgroups (n_kv_heads
-//    alone would leave the GPU idle); 16 lanes share a key (16 bytes of K and V each), all heads of the GQA group are
-//    scored against the same K/V registers, and a second tiny kernel merges the per-split (max, sum, O) partials in
-//    one trip to memory.
+//    alone would leave the GPU idle); both products run on the matrix cores with the heads of the GQA group as one
+//    operand, and a second tiny kernel merges the per-split (max, sum, O) partials in one trip to memory.
 //  * any other even head_dim up to 256 (the reference's flash_attn_sp_hdim.c domain): a plain kernel without MFMA.
 #include "device_utils.h"
 #include "kernels.h"
@@ -55,16 +60,18 @@ constexpr int kBK        = 64;  // keys per KV block
 
 template <int D>
 struct PrefillSmem {
-  // K tile: [key][D] halfs, rows padded by 16 bytes (conflict-free 16-byte fragment reads)
-  _Float16 k[kBK][D + 8];
-  // V^T tile: [d][key] halfs, rows padded by 8 bytes; row d stores key j at column (j + 8 (d / 32)) % 64 so that the
-  // transposing stores of one wave hit 64 different banks
-  _Float16 vt[D][kBK + 4];
+  // K and V tiles of a block of keys, rows as they lie in memory ([key][D] halfs), two buffers each: the next block
+  // arrives by DMA while one is used. The 16-byte pieces of a row are stored exclusive-or'ed with low bits of the row
+  // number (the DMA chooses what each lane fetches, not where it lands): K rows with key % 8, so that the 16-byte
+  // fragment reads of 8 neighbouring keys fall into different banks; V rows with 2 (key % 4), which keeps 32-byte
+  // pieces whole for the transposing reads and puts the four rows of such a read into different banks.
+  uint8_t k[2][kBK * D * 2];
+  uint8_t v[2][kBK * D * 2];
 };
 
 // GROUPS = 1 or 2 key groups per workgroup (4 waves each); with 2 they take alternate KV blocks of the same queries
 template <int D, bool QO_F32, int GROUPS>
-__global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(void *__restrict__ o_ptr,
+__global__ __launch_bounds__(kPfThreads *GROUPS, 2) void flash_attn_prefill_kernel(void *__restrict__ o_ptr,
                                                                         const void *__restrict__ q_ptr,
                                                                         const _Float16 *__restrict__ k_ptr,
                                                                         const _Float16 *__restrict__ v_ptr,
@@ -72,14 +79,14 @@ __global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(
                                                                         int kv_len, int n_heads, int n_kv_heads,
                                                                         int flags) {
   const bool causal = (flags & 1) != 0, mask_threshold = (flags & 2) != 0;
-  __shared__ PrefillSmem<D> sm_all[GROUPS];
+  __shared__ __align__(1024) PrefillSmem<D> sm_all[GROUPS];
   constexpr int KSTEPS = D / 16;  // MFMA k-steps over the head dimension
   constexpr int DT     = D / 32;  // 32-row tiles of O^T
   // With GROUPS = 2, two groups of 4 waves work on the same queries and heads: group g takes KV blocks g, g + 2, ...
   // with its own K/V tiles in LDS and its own running (max, sum, O); the two states are merged through LDS at the
   // end. The longest workgroup then walks half as many iterations, which pays when the grid is too small to keep two
   // independent workgroups on every CU busy to the end (few query blocks, or the uneven lengths under `causal`).
-  const int           grp = threadIdx.x / kPfThreads;
+  const int           grp = __builtin_amdgcn_readfirstlane((int) threadIdx.x / kPfThreads);  // (the same for a wave)
   PrefillSmem<D>     &sm  = sm_all[grp];
 
   const int group = n_heads / n_kv_heads;
@@ -154,100 +161,125 @@ __global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(
   // last key this lane's query may see, relative to the first key this lane holds in a block (key0 = 4 * half)
   const int vis_last = (causal ? min(kv_len - 1, q_row + q_shift) : kv_len - 1) - 4 * half;
 
-  // The next K/V block travels global memory -> registers while the current one is being used from LDS.
-  constexpr int K_PIECES = kBK * D / 8 / kPfThreads;         // 16-byte pieces of K per thread
-  constexpr int V_TASKS  = (kBK / 2) * (D / 8) / kPfThreads;  // (key pair, 8-wide d chunk) tasks of V per thread
-  v8h kreg[K_PIECES], vreg[V_TASKS][2];
-  // thread-constant element offsets inside a block; everything that changes per block is uniform (scalar registers)
-  const unsigned k_off = (unsigned) (tid / (D / 8)) * (unsigned) kv_stride + (unsigned) (tid % (D / 8)) * 8u;
-  const unsigned v_off = (unsigned) (tid / (D / 8)) * 2u * (unsigned) kv_stride + (unsigned) (tid % (D / 8)) * 8u;
-  constexpr int  ROWS  = kPfThreads / (D / 8);  // keys (K) or key pairs (V) covered by one pass of the workgroup
-  auto fetch = [&](int k0) {
+  // The next K/V block travels global memory -> LDS by DMA (global_load_lds, 1 KiB per instruction: no registers, no
+  // stores) while the current one is being used. A tile is TILE_B / 1024 instructions, the four waves take every
+  // fourth; lane L of an instruction lands at byte 16 L of its KiB = row L / CHUNKS, piece L % CHUNKS, and fetches the
+  // piece that belongs there. Per lane the source offsets inside a block never change (kept in registers); what
+  // changes per block is a base address the same for all lanes.
+  constexpr int ROWB     = D * 2;          // bytes of a K or V row
+  constexpr int CHUNKS   = ROWB / 16;      // 16-byte pieces of a row
+  constexpr int DMA_ROWS = 1024 / ROWB;    // rows per DMA instruction
+  constexpr int TILE_B   = kBK * ROWB;
+  constexpr int NDMA     = TILE_B / 1024 / 4;  // instructions per wave and tile
+  const int     wave_u   = __builtin_amdgcn_readfirstlane(wave);
+  uint32_t      src_off[2][NDMA];  // [K, V]: byte offset of this lane's piece from the block's first row of this KV head
+#pragma unroll
+  for (int j = 0; j < NDMA; ++j) {
+    const int row = (wave_u + 4 * j) * DMA_ROWS + lane / CHUNKS, piece = lane % CHUNKS;
+    src_off[0][j] = (uint32_t) row * (uint32_t) (kv_stride * 2) + 16u * (uint32_t) (piece ^ (row & 7));
+    src_off[1][j] = (uint32_t) row * (uint32_t) (kv_stride * 2) + 16u * (uint32_t) (piece ^ (2 * (row & 3)));
+  }
+  auto fetch = [&](int k0, int buf) {
+    const uint32_t to_k = (uint32_t) (uintptr_t) sm.k[buf], to_v = (uint32_t) (uintptr_t) sm.v[buf];
+    const uint8_t *kb = reinterpret_cast<const uint8_t *>(k_ptr + (size_t) h_kv * D + (size_t) k0 * kv_stride);
+    const uint8_t *vb = reinterpret_cast<const uint8_t *>(v_ptr + (size_t) h_kv * D + (size_t) k0 * kv_stride);
     if (k0 + kBK <= kv_len) {
 #pragma unroll
-      for (int j = 0; j < K_PIECES; ++j) {
-        const _Float16 *base = k_ptr + (size_t) h_kv * D + (size_t) (k0 + ROWS * j) * kv_stride;
-        kreg[j]              = *reinterpret_cast<const v8h *>(base + k_off);
+      for (int j = 0; j < NDMA; ++j) {
+        asm volatile("s_mov_b32 m0, %2\n s_nop 0\n global_load_lds_dwordx4 %0, %1" ::"v"(src_off[0][j]), "s"(kb),
+                     "s"(to_k + (uint32_t) ((wave_u + 4 * j) * 1024))
+                     : "memory");
       }
 #pragma unroll
-      for (int j = 0; j < V_TASKS; ++j) {
-        const _Float16 *base = v_ptr + (size_t) h_kv * D + (size_t) (k0 + 2 * ROWS * j) * kv_stride;
-        vreg[j][0]           = *reinterpret_cast<const v8h *>(base + v_off);
-        vreg[j][1]           = *reinterpret_cast<const v8h *>(base + kv_stride + v_off);
+      for (int j = 0; j < NDMA; ++j) {
+        asm volatile("s_mov_b32 m0, %2\n s_nop 0\n global_load_lds_dwordx4 %0, %1" ::"v"(src_off[1][j]), "s"(vb),
+                     "s"(to_v + (uint32_t) ((wave_u + 4 * j) * 1024))
+                     : "memory");
       }
       return;
     }
     // last, partial block: rows past the end repeat the last key (their scores are hidden below)
 #pragma unroll
-    for (int j = 0; j < K_PIECES; ++j) {
-      const int i   = tid + j * kPfThreads;
-      const int key = i / (D / 8), part = i % (D / 8);
-      const int kg  = min(k0 + key, kv_len - 1);
-      kreg[j] = *reinterpret_cast<const v8h *>(k_ptr + (size_t) kg * kv_stride + (size_t) h_kv * D + part * 8);
-    }
-#pragma unroll
-    for (int j = 0; j < V_TASKS; ++j) {
-      const int i = tid + j * kPfThreads;
-      const int c = i % (D / 8), kp = i / (D / 8);
-      const int kg0 = min(k0 + 2 * kp, kv_len - 1), kg1 = min(k0 + 2 * kp + 1, kv_len - 1);
-      vreg[j][0] = *reinterpret_cast<const v8h *>(v_ptr + (size_t) kg0 * kv_stride + (size_t) h_kv * D + c * 8);
-      vreg[j][1] = *reinterpret_cast<const v8h *>(v_ptr + (size_t) kg1 * kv_stride + (size_t) h_kv * D + c * 8);
+    for (int j = 0; j < 2 * NDMA; ++j) {
+      const int  jj  = j % NDMA;
+      const bool isv = j >= NDMA;
+      const int  row = (wave_u + 4 * jj) * DMA_ROWS + lane / CHUNKS, piece = lane % CHUNKS;
+      const int  key = min(k0 + row, kv_len - 1);
+      const int  log = isv ? piece ^ (2 * (row & 3)) : piece ^ (row & 7);
+      const _Float16 *src = (isv ? v_ptr : k_ptr) + (size_t) key * kv_stride + (size_t) h_kv * D + 8 * log;
+      asm volatile("s_mov_b32 m0, %1\n s_nop 0\n global_load_lds_dwordx4 %0, off" ::"v"(src),
+                   "s"((isv ? to_v : to_k) + (uint32_t) ((wave_u + 4 * jj) * 1024))
+                   : "memory");
     }
   };
+  // additive mask values of this lane's 2 x 16 keys of a block: requested a block ahead, like the tiles
+  auto fetch_mask = [&](v4h (&m)[2][4], int k0) {
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        // four consecutive keys: one 8-byte load (rows are padded to a multiple of 64 keys)
+        m[kt][rg] = *reinterpret_cast<const v4h *>(mask + (size_t) q_clamp * mask_ld + k0 + 32 * kt + 8 * rg + 4 * half);
+      }
+    }
+  };
+  // where this lane's fragments lie in a tile (bytes): K row `col` (+ 32 per tile), piece 2 s + half; V: the lane
+  // (16-lane group g = lane / 16, i = lane % 16 = 4 j + q) points at row 4 half + j (+ 16 u + 8 per read), the 8-byte
+  // piece q of columns 32 t + 16 (g & 1) .. + 15, and receives column 32 t + 16 (g & 1) + i of four rows
+  uint32_t k_at[KSTEPS], v_at[DT];
+  {
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+      k_at[s] = (uint32_t) (col * ROWB + 16 * ((2 * s + half) ^ (col & 7)));
+    }
+    const int g = lane >> 4, j = (lane >> 2) & 3, q = lane & 3;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+      v_at[t] = (uint32_t) ((4 * half + j) * ROWB + 16 * ((4 * t + 2 * (g & 1) + (q >> 1)) ^ (2 * j)) + 8 * (q & 1));
+    }
+  }
+  typedef short v4s __attribute__((ext_vector_type(4)));
+
+  v4h mreg[2][4], mnext[2][4];
   if (grp * kBK < kv_limit) {
-    fetch(grp * kBK);
+    fetch(grp * kBK, 0);
+    if (mask) {
+      fetch_mask(mnext, grp * kBK);
+    }
   }
 
-  for (int kk = 0; kk < kv_limit; kk += GROUPS * kBK) {
+  int it = 0;
+  for (int kk = 0; kk < kv_limit; kk += GROUPS * kBK, ++it) {
     const int  k0   = kk + grp * kBK;  // this key group's block of the iteration
     const bool live = k0 < kv_limit;   // (the last iteration may have a block for the first group only)
-    __syncthreads();  // previous block's fragments are no longer needed
-    // ---- stage K [key][D] and V^T [d][key] from the registers ----
-    if (live) {
-#pragma unroll
-      for (int j = 0; j < K_PIECES; ++j) {
-        const int i   = tid + j * kPfThreads;
-        const int key = i / (D / 8), part = i % (D / 8);
-        *reinterpret_cast<v8h *>(&sm.k[key][part * 8]) = kreg[j];
-      }
-#pragma unroll
-      for (int j = 0; j < V_TASKS; ++j) {
-        // two keys of one 8-wide d chunk: eight 4-byte transposed stores
-        const int i = tid + j * kPfThreads;
-        const int c = i % (D / 8), kp = i / (D / 8);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const int d   = c * 8 + e;
-          const int pos = (2 * kp + 8 * (d / 32)) % kBK;
-          v2h       pr  = { vreg[j][0][e], vreg[j][1][e] };
-          *reinterpret_cast<v2h *>(&sm.vt[d][pos]) = pr;
-        }
-      }
-    }
+    const int  buf  = it & 1;
+    // this wave's share of the block has landed; behind the barrier everybody's has, and nobody reads the other
+    // buffer (the previous block) any more
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (k0 + GROUPS * kBK < kv_limit) {
-      fetch(k0 + GROUPS * kBK);
-    }
-    if (!live) {
-      continue;
-    }
-
-    // ---- S^T - m = K Q^T - m: two 32-key tiles, accumulated on top of minus the running maximum ----
-    // Scores come out of the MFMA already relative to the maximum seen so far, so a block that brings no new maximum
-    // to any query of the wave (the usual case after the first few blocks) needs no subtraction and no rescaling.
-    // additive mask values of this lane's 2 x 16 keys, requested before the products so that they arrive meanwhile
-    v4h mreg[2][4];
     if (mask) {
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
         for (int rg = 0; rg < 4; ++rg) {
-          // four consecutive keys: one 8-byte load (rows are padded to a multiple of 64 keys)
-          mreg[kt][rg] = *reinterpret_cast<const v4h *>(mask + (size_t) q_clamp * mask_ld + k0 + 32 * kt + 8 * rg +
-                                                        4 * half);
+          mreg[kt][rg] = mnext[kt][rg];
         }
       }
     }
+    if (k0 + GROUPS * kBK < kv_limit) {
+      fetch(k0 + GROUPS * kBK, buf ^ 1);
+      if (mask) {
+        fetch_mask(mnext, k0 + GROUPS * kBK);
+      }
+    }
+    if (!live) {
+      continue;
+    }
+    const uint8_t *k_tile = sm.k[buf], *v_tile = sm.v[buf];
+
+    // ---- S^T - m = K Q^T - m: two 32-key tiles, accumulated on top of minus the running maximum ----
+    // Scores come out of the MFMA already relative to the maximum seen so far, so a block that brings no new maximum
+    // to any query of the wave (the usual case after the first few blocks) needs no subtraction and no rescaling.
     const bool  fresh = m_run == -INFINITY;  // nothing visible yet for this query
     const float m_ref = fresh ? 0.0f : m_run;
     v16f st[2];
@@ -258,25 +290,29 @@ __global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(
         st[kt][r] = -m_ref;
       }
     }
-    // the two key tiles advance side by side (independent accumulators), and the fragments of step s + 1 are
+    // the two key tiles advance side by side (independent accumulators), and the fragments of step s + PF are
     // requested before the products of step s
     {
-      v8h kf[2][2];
+      constexpr int PF = 3;  // steps ahead (an LDS read takes longer to return than two steps' products to issue)
+      v8h kf[PF + 1][2];
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
-        kf[0][kt] = *reinterpret_cast<const v8h *>(&sm.k[32 * kt + col][8 * half]);
+      for (int s = 0; s < PF && s < KSTEPS; ++s) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt) {
+          kf[s][kt] = *reinterpret_cast<const v8h *>(k_tile + k_at[s] + 32 * kt * ROWB);
+        }
       }
 #pragma unroll
       for (int s = 0; s < KSTEPS; ++s) {
-        if (s + 1 < KSTEPS) {
+        if (s + PF < KSTEPS) {
 #pragma unroll
           for (int kt = 0; kt < 2; ++kt) {
-            kf[(s + 1) & 1][kt] = *reinterpret_cast<const v8h *>(&sm.k[32 * kt + col][16 * (s + 1) + 8 * half]);
+            kf[(s + PF) % (PF + 1)][kt] = *reinterpret_cast<const v8h *>(k_tile + k_at[s + PF] + 32 * kt * ROWB);
           }
         }
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt) {
-          st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s & 1][kt], qf[s], st[kt], 0, 0, 0);
+          st[kt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[s % (PF + 1)][kt], qf[s], st[kt], 0, 0, 0);
         }
       }
     }
@@ -322,6 +358,9 @@ __global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(
     // the first visible block of a query sets its maximum (either sign), later blocks only raise it
     const bool move = fresh ? (mx != -INFINITY) : (mx > 0.0f);
     if (__builtin_amdgcn_ballot_w64(move) != 0) {
+      // (a statement the compiler cannot run ahead of the test: without it the 97 instructions below are turned into
+      // selects and run for every block)
+      asm volatile("" ::: "memory");
       const float delta = move ? mx : 0.0f;
       const float alpha = fresh ? 0.0f : fast_exp2(-delta);  // O and l of a fresh query are still zero
 #pragma unroll
@@ -341,14 +380,20 @@ __global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(
       l_run *= alpha;
       m_run = move ? m_ref + mx : m_run;
     }
-    float psum[4] = { 0.0f, 0.0f, 0.0f, 0.0f };  // (four chains: an addition waits for the one before it in its chain)
+    // the probabilities, rounded to fp16 in pairs as the matrix instruction takes them; the row sum adds up the
+    // rounded values (v_dot2_f32_f16 with ones: two per instruction, fp32 sums), so O and l see the same numbers
+    uint32_t pk[2][8];
+    float    psum[4] = { 0.0f, 0.0f, 0.0f, 0.0f };  // (four chains: an addition waits for the one before it in its chain)
+    {
+      const v2h ones = { (_Float16) 1.0f, (_Float16) 1.0f };
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
+      for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float p = fast_exp2(st[kt][r]);
-        st[kt][r]     = p;
-        psum[r & 3] += p;
+        for (int r = 0; r < 16; r += 2) {
+          const v2h p2  = { (_Float16) fast_exp2(st[kt][r]), (_Float16) fast_exp2(st[kt][r + 1]) };
+          pk[kt][r / 2] = __builtin_bit_cast(uint32_t, p2);
+          psum[(r / 2) & 3] = __builtin_amdgcn_fdot2(p2, ones, psum[(r / 2) & 3], false);
+        }
       }
     }
     l_run += (psum[0] + psum[1]) + (psum[2] + psum[3]);
@@ -359,20 +404,16 @@ __global__ __launch_bounds__(kPfThreads *GROUPS) void flash_attn_prefill_kernel(
     for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        v8h pf;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          pf[e] = (_Float16) st[kt][8 * u + e];
-        }
+        const v8h pf = __builtin_bit_cast(v8h, make_uint4(pk[kt][4 * u], pk[kt][4 * u + 1], pk[kt][4 * u + 2], pk[kt][4 * u + 3]));
 #pragma unroll
         for (int t = 0; t < DT; ++t) {
-          const int d    = 32 * t + col;
-          const int key0 = (32 * kt + 16 * u + 4 * half + 8 * t) % kBK;  // rotated column of the first 4 keys
-          const int key1 = (key0 + 8) % kBK;
-          const v4h a0   = *reinterpret_cast<const v4h *>(&sm.vt[d][key0]);
-          const v4h a1   = *reinterpret_cast<const v4h *>(&sm.vt[d][key1]);
-          v8h       vf   = { a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3] };
-          oacc[t]        = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf, oacc[t], 0, 0, 0);
+          // (V^T fragment: column 32 t + lane % 32 of keys 32 kt + 16 u + 4 half + 0 .. 3 and + 8 .. 11)
+          const uint8_t *at = v_tile + v_at[t] + (32 * kt + 16 * u) * ROWB;
+          const v4s a0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3))) *) at);
+          const v4s a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4s __attribute__((address_space(3))) *) (at + 8 * ROWB));
+          const v8h vf = __builtin_bit_cast(v8h, (short __attribute__((ext_vector_type(8)))){ a0[0], a0[1], a0[2], a0[3],
+                                                                                             a1[0], a1[1], a1[2], a1[3] });
+          oacc[t]      = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf, oacc[t], 0, 0, 0);
         }
       }
     }
@@ -930,8 +971,8 @@ hipError_t launch_prefill(hipStream_t stream, void *o, const void *q, const void
   const dim3 grid((unsigned) (n_kv_heads * sub_groups), q_blocks);
   // Two key groups per workgroup when the grid leaves CUs without a second workgroup, or (causal) when the workgroups
   // all fit at once and their uneven lengths would leave the long ones running alone. Measured on the 256-CU device,
-  // 32 query / 8 KV heads of 128: 2048 x 2048 causal 67 us against 73 us, 1024 x 2048 65 against 72 us; but
-  // 2048 x 2048 without `causal` 117 against 107 us and 4096 x 4096 causal 242 against 214 us.
+  // 32 query / 8 KV heads of 128: 2048 x 2048 causal 59 us against 65 us, 1024 x 1024 without `causal` 30 against
+  // 33 us; but 2048 x 2048 without `causal` 101 against 92 us.
   constexpr unsigned kCus = 256;
   const unsigned     wgs  = grid.x * grid.y;
   const bool         two  = forced ? forced == 2 : (wgs <= kCus || (causal && wgs <= 2 * kCus));
