@@ -177,7 +177,7 @@ def test_threshold_mask_follows_the_dispatched_kernels_rule(oracle):
     want = np.array([0, 0, -np.inf, -np.inf, -np.inf, -np.inf, 0, 0, -np.inf, 0], np.float16)
     assert np.array_equal(got, want)
     assert vals[1] > np.float16(-16) and vals[3] < np.float16(-16)
-    # on a 0 / -inf mask the two conventions are the same function (the survey's "identical for 0 / -inf")
+    # on a 0 / -inf mask the two conventions are the same function
     rng = np.random.default_rng(5)
     q = rng.standard_normal((3, 2, 64)).astype(np.float32)
     k = rng.standard_normal((70, 1, 64)).astype(np.float16)
