@@ -16,7 +16,7 @@ The same run also measures, and reports inside the JSON line:
   launches      q+k+v, o, gate+up and down as launches of their own (cold weights), each with its share of HBM peak
   prefill_gemm  m = 512 Q4_0 GEMM, both shapes of config 2, in int8 Tera-ops/s (2 m n k per launch); the per-call
                 re-tiling of the activations and the one-time conversion of a weight buffer are reported separately
-  small_batch   the same layer at m = 2 and m = 8
+  small_batch   the same layer at m = 2, m = 3 and m = 8
   recorded_message_us_per_step   the m = 1 and m = 8 steps again, each layer's message recorded once into a HIP graph
                 and replayed (reported beside `value`, which is the ordinary message walk)
   q8_0_block    the Qwen2-1.5B-like Q8_0 block of config 4 at m = 1 and m = 128
@@ -126,7 +126,7 @@ def main():
     ACT_OF = {"q": 0, "k": 0, "v": 0, "o": 1, "gate": 2, "up": 2, "down": 3}
     ACT_K = {0: 4096, 1: 4096, 2: 4096, 3: 11008}
     act_q, h_act = {}, {}
-    for m in (1, 2, 8):
+    for m in (1, 2, 3, 8):
         for g, k in ACT_K.items():
             x = wl.make_activations(rng, m, k)
             act_q[(m, g)] = ctx.run_quantize_q8_0(x)                       # quantized on the GPU ...
@@ -135,7 +135,7 @@ def main():
     layers = []
     for _ in range(LAYERS):
         layers.append([ctx.upload(uniq[(n, k)]) for _, n, k in shapes])
-    h_out = {m: [ctx.alloc(m * n * 4) for _, n, _ in shapes] for m in (1, 2, 8)}
+    h_out = {m: [ctx.alloc(m * n * 4) for _, n, _ in shapes] for m in (1, 2, 3, 8)}
     log("setup: %d layers x %.1f MB of Q4_0 weights resident (%.1f s)" % (
         LAYERS, sum(uniq[(n, k)].nbytes for _, n, k in shapes) / 1e6, time.time() - t_setup))
 
@@ -169,10 +169,11 @@ def main():
         return worst, submissions
 
     (worst1, subs1), (worst2, subs2), (worst8, subs8) = check_layer(1), check_layer(2), check_layer(8)
-    log("parity m=1: worst |err|/sum|terms| = %.2e (%d launch per message); m=2: %.2e (%d); m=8: %.2e (%d launches)" % (
-        worst1, subs1, worst2, subs2, worst8, subs8))
+    worst3, subs3 = check_layer(3)
+    log("parity m=1: worst |err|/sum|terms| = %.2e (%d launch per message); m=2: %.2e (%d); m=3: %.2e (%d); m=8: %.2e (%d launches)" % (
+        worst1, subs1, worst2, subs2, worst3, subs3, worst8, subs8))
 
-    layer_bytes = {m: sum(wl.matmul_algorithmic_bytes(m, k, n, Q4) for _, n, k in shapes) for m in (1, 2, 8)}
+    layer_bytes = {m: sum(wl.matmul_algorithmic_bytes(m, k, n, Q4) for _, n, k in shapes) for m in (1, 2, 3, 8)}
 
     def time_layers(m, steps, warmup):
         msgs = [layer_message(l, m) for l in range(LAYERS)]
@@ -292,6 +293,8 @@ def main():
     ms_step2, _ = time_layers(2, max(20, min(args.steps // 4, 200)), LAYERS)
     log("layer m=2: %.2f us/step  %.0f GB/s" % (ms_step2 * 1e3, layer_bytes[2] / ms_step2 / 1e6))
     # (every layer is touched before the clock starts: the first few-row use of a weight buffer repacks it once)
+    ms_step3, _ = time_layers(3, max(20, min(args.steps // 4, 200)), LAYERS)
+    log("layer m=3: %.2f us/step  %.0f GB/s" % (ms_step3 * 1e3, layer_bytes[3] / ms_step3 / 1e6))
     ms_step8, _ = time_layers(8, max(20, min(args.steps // 4, 200)), LAYERS)
     log("layer m=8: %.2f us/step  %.0f GB/s" % (ms_step8 * 1e3, layer_bytes[8] / ms_step8 / 1e6))
     rec_step[8] = None if args.skip_recorded else time_recorded_layers(8, max(20, min(args.steps // 4, 200)), LAYERS)
@@ -765,6 +768,8 @@ def main():
         "prefill_gemm": prefill,
         "small_batch": [{"m": 2, "us_per_step": round(ms_step2 * 1e3, 2), "GBps": round(layer_bytes[2] / ms_step2 / 1e6, 1),
                          "launches_per_message": subs2},
+                        {"m": 3, "us_per_step": round(ms_step3 * 1e3, 2), "GBps": round(layer_bytes[3] / ms_step3 / 1e6, 1),
+                         "launches_per_message": subs3},
                         {"m": 8, "us_per_step": round(ms_step8 * 1e3, 2), "GBps": round(layer_bytes[8] / ms_step8 / 1e6, 1),
                          "launches_per_message": subs8}],
         "recorded_message_us_per_step": None if args.skip_recorded else

@@ -212,63 +212,79 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
     } else if (b.m == 1) {
       e = launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k, (WeightType) b.wt);
     } else {
-      // 2..16 rows. Two or three rows are one launch of the weight stream that keeps them in registers, each member
-      // with its own rows and row length. Otherwise members whose weights have (or get) a repacked copy go to the
-      // kernel that streams it, again each with its own activation rows (and, for the two-blocks-per-instruction
-      // kernel, its own k; the batch holds members of different k only where every one of them fits that kernel); the
-      // rest go to the K-sliced kernel, one launch per set of rows (it stages one). Which kernel a matrix gets depends
-      // on that matrix alone.
-      if (ctx->opt.gemv_rows_kernel != 0 && gemv_rows_fits(b.m, k0, (WeightType) b.wt)) {
-        e = launch_gemv_rows_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.m, b.k,
-                                                    (WeightType) b.wt);
-      } else {
-        float      *out_a[kGemvGroupMax];
-        const void *w_a[kGemvGroupMax], *act_a[kGemvGroupMax];
-        int         n_a[kGemvGroupMax], k_a[kGemvGroupMax], count_a = 0;
-        bool        sliced[kGemvGroupMax] = {};
-        bool        pairs = false;  // which repacked-weight kernel (the same for every member: it depends on m, k, type)
-        for (int i = 0; i < b.count; ++i) {
-          const void *lw = nullptr;
-          bool        member_pairs = false;
-          if (int r = lane_order_weights(ctx, b.w[i], b.act[i], b.m, b.k[i], b.n[i], b.wt, &lw, &member_pairs)) {
-            b.hdr[i]->state = r;
-          } else if (lw) {
-            pairs          = member_pairs;
-            out_a[count_a] = b.out[i], w_a[count_a] = lw, act_a[count_a] = b.act[i], k_a[count_a] = b.k[i];
-            n_a[count_a++] = b.n[i];
-          } else if (b.m <= kSkinnyGroupMaxM) {
-            sliced[i] = true;
-          } else {
-            // more rows than the K-sliced group launch takes: on its own
-            b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act[i], b.w[i], b.m, b.k[i], b.n[i], b.wt);
+      // 2..16 rows. Which kernel a matrix gets depends on that matrix alone, in the order of the single request
+      // (run_few_rows): three rows of Q4_0 that fit the two-blocks-per-instruction kernel and have, or get, their
+      // repacked copy go there; other two- and three-row members to the weight stream that keeps the rows in
+      // registers; the others to the kernel that streams their repacked copy (lane order), and what has no copy to
+      // the K-sliced kernel. Every kind is one launch for all its members, each with its own activation rows (and
+      // its own k, except in the lane-order kernel: a batch holds members of different k only where each of them fits
+      // the two- and three-row kernel or the two-blocks-per-instruction kernel); the K-sliced kernel stages one set
+      // of rows per launch.
+      struct Group {
+        float      *out[kGemvGroupMax];
+        const void *w[kGemvGroupMax], *act[kGemvGroupMax];
+        int         n[kGemvGroupMax], k[kGemvGroupMax], count = 0;
+        void add(float *o, const void *ww, const void *a, int nn, int kk) {
+          out[count] = o, w[count] = ww, act[count] = a, n[count] = nn, k[count++] = kk;
+        }
+      } pairs_g, lane_g, rows_g;
+      bool sliced[kGemvGroupMax] = {};
+      for (int i = 0; i < b.count; ++i) {
+        const void *lw = nullptr;
+        bool        member_pairs = false;
+        int         r = HTPOPS_OK;
+        if (prefers_block_pairs(ctx, b.m, b.k[i], b.n[i], b.wt)) {
+          r = lane_order_weights(ctx, b.w[i], b.act[i], b.m, b.k[i], b.n[i], b.wt, &lw, &member_pairs);
+        }
+        const bool rows = !lw && ctx->opt.gemv_rows_kernel != 0 && gemv_rows_fits(b.m, b.k[i], (WeightType) b.wt);
+        if (r == HTPOPS_OK && !lw && !rows) {
+          r = lane_order_weights(ctx, b.w[i], b.act[i], b.m, b.k[i], b.n[i], b.wt, &lw, &member_pairs);
+        }
+        if (r != HTPOPS_OK) {
+          b.hdr[i]->state = r;
+        } else if (lw) {
+          (member_pairs ? pairs_g : lane_g).add(b.out[i], lw, b.act[i], b.n[i], b.k[i]);
+        } else if (rows) {
+          rows_g.add(b.out[i], b.w[i], b.act[i], b.n[i], b.k[i]);
+        } else if (b.m <= kSkinnyGroupMaxM) {
+          sliced[i] = true;
+        } else {
+          // more rows than the K-sliced group launch takes: on its own
+          b.hdr[i]->state = op_mat_mul_q8(ctx, b.out[i], b.act[i], b.w[i], b.m, b.k[i], b.n[i], b.wt);
+        }
+      }
+      e = hipSuccess;
+      if (pairs_g.count > 0) {
+        e = launch_matmul_block_pairs_group(ctx->stream, pairs_g.count, pairs_g.out, pairs_g.act, pairs_g.w, pairs_g.n, b.m,
+                                            pairs_g.k);
+      }
+      if (e == hipSuccess && lane_g.count > 0) {
+        e = launch_matmul_lane_order_group(ctx->stream, lane_g.count, lane_g.out, lane_g.act, lane_g.w, lane_g.n, b.m, k0,
+                                           (WeightType) b.wt, ctx->opt.lane_order);
+      }
+      if (e == hipSuccess && rows_g.count > 0) {
+        e = launch_gemv_rows_group_q8_0_act(ctx->stream, rows_g.count, rows_g.out, rows_g.act, rows_g.w, rows_g.n, b.m,
+                                            rows_g.k, (WeightType) b.wt);
+      }
+      for (int first = 0; first < b.count && e == hipSuccess && ret == HTPOPS_OK; ++first) {
+        if (!sliced[first]) {
+          continue;
+        }
+        float      *out_b[kGemvGroupMax];
+        const void *w_b[kGemvGroupMax];
+        int         n_b[kGemvGroupMax], count_b = 0;
+        for (int i = first; i < b.count; ++i) {  // everybody left that reads the rows of `first`
+          if (sliced[i] && b.act[i] == b.act[first] && b.k[i] == b.k[first]) {
+            out_b[count_b] = b.out[i], w_b[count_b] = b.w[i], n_b[count_b++] = b.n[i];
+            sliced[i] = false;
           }
         }
-        e = hipSuccess;
-        if (count_a > 0) {
-          e = pairs ? launch_matmul_block_pairs_group(ctx->stream, count_a, out_a, act_a, w_a, n_a, b.m, k_a) :
-                      launch_matmul_lane_order_group(ctx->stream, count_a, out_a, act_a, w_a, n_a, b.m, k0,
-                                                     (WeightType) b.wt, ctx->opt.lane_order);
-        }
-        for (int first = 0; first < b.count && e == hipSuccess && ret == HTPOPS_OK; ++first) {
-          if (!sliced[first]) {
-            continue;
-          }
-          float      *out_b[kGemvGroupMax];
-          const void *w_b[kGemvGroupMax];
-          int         n_b[kGemvGroupMax], count_b = 0;
-          for (int i = first; i < b.count; ++i) {  // everybody left that reads the rows of `first`
-            if (sliced[i] && b.act[i] == b.act[first] && b.k[i] == b.k[first]) {
-              out_b[count_b] = b.out[i], w_b[count_b] = b.w[i], n_b[count_b++] = b.n[i];
-              sliced[i] = false;
-            }
-          }
-          const size_t ws = matmul_skinny_group_workspace_bytes(count_b, n_b, b.m, b.k[first]);
-          if (int r = ensure_workspace(ctx, ws)) {
-            ret = r;
-          } else {
-            e = launch_matmul_skinny_group(ctx->stream, count_b, out_b, b.act[first], w_b, n_b, b.m, b.k[first],
-                                                   (WeightType) b.wt, ctx->workspace, ctx->tickets, kTicketSlots);
-          }
+        const size_t ws = matmul_skinny_group_workspace_bytes(count_b, n_b, b.m, b.k[first]);
+        if (int r = ensure_workspace(ctx, ws)) {
+          ret = r;
+        } else {
+          e = launch_matmul_skinny_group(ctx->stream, count_b, out_b, b.act[first], w_b, n_b, b.m, b.k[first],
+                                                 (WeightType) b.wt, ctx->workspace, ctx->tickets, kTicketSlots);
         }
       }
     }

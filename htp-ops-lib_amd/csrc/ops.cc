@@ -97,6 +97,10 @@ int check_mat_mul(htpops_context *ctx, const void *dst, const void *act, const v
 // 16-byte aligned for the DMA into LDS, weights in memory whose copies may not be kept; the caller then uses the
 // kernels that read the weights as they are. A failed allocation or conversion launch is an error, not a reason to
 // switch kernels.)
+bool prefers_block_pairs(const htpops_context *ctx, int m, int k, int n, int wt) {
+  return m == 3 && wt == kQ4_0 && ctx->opt.lane_order == 1 && matmul_block_pairs_fits(n, m, k, (WeightType) wt);
+}
+
 int lane_order_weights(htpops_context *ctx, const void *weight, const void *act, int m, int k, int n, int wt,
                        const void **out, bool *block_pairs) {
   *out         = nullptr;
@@ -190,7 +194,14 @@ int run_few_rows(htpops_context *ctx, float *dst, const void *act, const void *w
                  uint8_t *ws) {
   // hipErrorNotSupported from a launcher means "this kernel does not take the shape": try the next one. Any other
   // failure is reported.
-  if (ctx->opt.gemv_rows_kernel != 0 && gemv_rows_fits(m, k, (WeightType) wt) && aligned(act, 4) && aligned(weight, 4)) {
+  const void *lw    = nullptr;
+  bool        pairs = false;
+  if (prefers_block_pairs(ctx, m, k, n, wt)) {
+    if (int r = lane_order_weights(ctx, weight, act, m, k, n, wt, &lw, &pairs)) {
+      return r;
+    }
+  }
+  if (!lw && ctx->opt.gemv_rows_kernel != 0 && gemv_rows_fits(m, k, (WeightType) wt) && aligned(act, 4) && aligned(weight, 4)) {
     const hipError_t e = launch_gemv_rows_group_q8_0_act(ctx->stream, 1, &dst, &act, &weight, &n, m, &k,
                                                                  (WeightType) wt);
     if (e == hipSuccess) {
@@ -201,10 +212,10 @@ int run_few_rows(htpops_context *ctx, float *dst, const void *act, const void *w
     }
     (void) hipGetLastError();
   }
-  const void *lw    = nullptr;
-  bool        pairs = false;
-  if (int r = lane_order_weights(ctx, weight, act, m, k, n, wt, &lw, &pairs)) {
-    return r;
+  if (!lw) {
+    if (int r = lane_order_weights(ctx, weight, act, m, k, n, wt, &lw, &pairs)) {
+      return r;
+    }
   }
   if (lw) {
     const hipError_t e = pairs ? launch_matmul_block_pairs_group(ctx->stream, 1, &dst, &act, &lw, &n, m, &k) :

@@ -344,7 +344,8 @@ extern "C" int htpops_buffer_prepare_weights(htpops_context *ctx, int handle, si
     if (int r = plan_weight_copy(ctx, plan, w, k, n, weight_type, &copy)) {
       return r;
     }
-  } else if (m_hint >= 2 && !(ctx->opt.gemv_rows_kernel != 0 && gemv_rows_fits(m_hint, k, (WeightType) weight_type))) {
+  } else if (m_hint >= 2 && (prefers_block_pairs(ctx, m_hint, k, n, weight_type) ||
+                             !(ctx->opt.gemv_rows_kernel != 0 && gemv_rows_fits(m_hint, k, (WeightType) weight_type)))) {
     // (the two- and three-row kernel reads the weights as they are: nothing to make for it)
     const void *copy  = nullptr;
     bool        pairs = false;

@@ -76,8 +76,8 @@ def test_llama7b_layer_message_at_full_size(ctx, oracle, llama_weights, m):
     # config 1: q/k/v/o 4096x4096, gate/up 11008x4096, down 4096x11008, seven requests in one message
     rng = wl.rng_for(1, 100 + m)
     acts = {g: oracle.quantize_q8_0(wl.make_activations(rng, m, k)) for g, k in {0: 4096, 1: 4096, 2: 4096, 3: 11008}.items()}
-    # the seven requests are one launch: up to three rows in the kernel that keeps the rows in registers, eight rows in
-    # the two-blocks-per-instruction kernel, whose members may differ in k
+    # the seven requests are one launch: two rows in the kernel that keeps the rows in registers, three and eight rows
+    # in the two-blocks-per-instruction kernel, whose members may differ in k
     run_layer_message(ctx, oracle, wl.LLAMA7B_LAYER, llama_weights, acts, m, Q4, launches=1)
 
 
