@@ -399,19 +399,56 @@ hipError_t launch_matmul_block_pairs_group(hipStream_t stream, int count, float 
   // workgroups take its tiles in turn.
   const int  per_cu   = alone ? 1 : (int) std::min<size_t>(3, kBpLdsLimit / lds);
   const long resident = 256L * per_cu;
-  long       tiles = 0;
-  double     work  = 0.0;
+  long       tiles    = 0;
   for (int i = 0; i < count; ++i) {
     tiles += ns[i] / kBpRows;
-    work += (double) (ns[i] / kBpRows) * ks[i];
   }
-  grp.count       = count;
+  grp.count = count;
+  long wgs[kGemvGroupMax];
+  if (tiles <= resident) {
+    for (int i = 0; i < count; ++i) {
+      wgs[i] = ns[i] / kBpRows;
+    }
+  } else {
+    // The launch ends with its busiest workgroup. A workgroup of member i that walks t tiles carries t k_i (weight
+    // bytes, up to a factor): find the smallest such load T for which ceil(tiles_i / floor(T / k_i)) workgroups per
+    // member fit the device, trying every load some member can produce (tiles-per-workgroup counts are small).
+    auto needed = [&](double T, long *out) {
+      long sum = 0;
+      for (int i = 0; i < count; ++i) {
+        const long per = (long) (T / ks[i]);
+        if (per < 1) {
+          return -1L;
+        }
+        const long mine = ns[i] / kBpRows;
+        out[i] = (mine + per - 1) / per;
+        sum += out[i];
+      }
+      return sum;
+    };
+    double best_T = 0.0;
+    for (int i = 0; i < count; ++i) {
+      const long mine = ns[i] / kBpRows;
+      for (long t = 1; t <= mine; ++t) {
+        const double T = (double) t * ks[i];
+        if (best_T > 0.0 && T >= best_T) {
+          break;
+        }
+        long       tmp[kGemvGroupMax];
+        const long sum = needed(T, tmp);
+        if (sum > 0 && sum <= resident) {
+          best_T = T;
+          break;  // (larger t of this member only raise T)
+        }
+      }
+    }
+    if (best_T <= 0.0 || needed(best_T, wgs) < 0) {
+      return hipErrorNotSupported;  // (more members than workgroups: cannot happen with at most 8 members)
+    }
+  }
   grp.wg_begin[0] = 0;
   for (int i = 0; i < count; ++i) {
-    const long mine = ns[i] / kBpRows;
-    const long wgs  = tiles <= resident ? mine :
-                                          std::max(1L, std::min(mine, (long) ((double) mine * ks[i] * resident / work + 0.5)));
-    grp.wg_begin[i + 1] = grp.wg_begin[i] + (int) wgs;
+    grp.wg_begin[i + 1] = grp.wg_begin[i] + (int) wgs[i];
   }
   const dim3 grid((unsigned) grp.wg_begin[count]), block(kBpThreads);
   if (alone) {
