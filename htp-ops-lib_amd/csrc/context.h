@@ -247,9 +247,9 @@ int plan_weight_copy(htpops_context *ctx, MatMulPlan &plan, const void *weight, 
 // when this matmul takes neither of them. *block_pairs: which of the two operand orders the copy is in (the kernel
 // with two blocks per matrix instruction for up to 8 rows of Q4_0, the one-block kernel otherwise); the choice depends
 // on (m, k, weight type) and the context's switches only, so the members of a grouped launch agree on it.
-// Three rows of Q4_0: the two-blocks-per-instruction kernel over a repacked copy where the shape fits it and a copy is
-// there or may be kept (a Llama-7B layer: 27 against 32 us); the kernel that holds the rows in registers and reads the
-// weights as they are otherwise, and always for two rows (level: no reason to hold a copy).
+// Two and three rows of Q4_0: the two-blocks-per-instruction kernel over a repacked copy where the shape fits it and a
+// copy is there or may be kept (a Llama-7B layer: 25 against 28 us at two rows, 25 against 32 us at three); the kernel
+// that holds the rows in registers and reads the weights as they are otherwise.
 bool prefers_block_pairs(const htpops_context *ctx, int m, int k, int n, int wt);
 int lane_order_weights(htpops_context *ctx, const void *weight, const void *act, int m, int k, int n, int wt,
                        const void **out, bool *block_pairs);

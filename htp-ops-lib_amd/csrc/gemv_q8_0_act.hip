@@ -981,8 +981,8 @@ bool gemv_rows_fits(int m, int k, WeightType wt) {
   // measured on Llama-7B (Q4_0) and Qwen2-1.5B (Q8_0) layers: up to three rows the kernel beats the repacked-weight and
   // K-sliced kernels (28.2 / 31.8 against 38.9 / 39.3 us and 13.3 / 14.8 against 18.3 / 18.5 us), at four rows they
   // are level (39.0 against 38.2, 18.4 against 18.6 us); every further row costs it as much again while theirs come
-  // free up to eight. (Three rows of Q4_0 go to the two-blocks-per-instruction kernel instead where a repacked copy of
-  // the weights is there or may be kept, 27 against 32 us; the caller decides that.)
+  // free up to eight. (Two and three rows of Q4_0 go to the two-blocks-per-instruction kernel instead where a repacked
+  // copy of the weights is there or may be kept, 25 against 28 and 32 us; the caller decides that.)
   (void) wt;
   const int nblk = k / kQK;
   return m >= 2 && m <= 3 && k % (2 * kQK) == 0 && nblk / 2 <= kSharedActMaxPairs;

@@ -213,7 +213,7 @@ void flush_batch(htpops_context *ctx, GemvBatch &b) {
       e = launch_gemv_group_q8_0_act(ctx->stream, b.count, b.out, b.act, b.w, b.n, b.k, (WeightType) b.wt);
     } else {
       // 2..16 rows. Which kernel a matrix gets depends on that matrix alone, in the order of the single request
-      // (run_few_rows): three rows of Q4_0 that fit the two-blocks-per-instruction kernel and have, or get, their
+      // (run_few_rows): two and three rows of Q4_0 that fit the two-blocks-per-instruction kernel and have, or get, their
       // repacked copy go there; other two- and three-row members to the weight stream that keeps the rows in
       // registers; the others to the kernel that streams their repacked copy (lane order), and what has no copy to
       // the K-sliced kernel. Every kind is one launch for all its members, each with its own activation rows (and

@@ -98,7 +98,7 @@ int check_mat_mul(htpops_context *ctx, const void *dst, const void *act, const v
 // kernels that read the weights as they are. A failed allocation or conversion launch is an error, not a reason to
 // switch kernels.)
 bool prefers_block_pairs(const htpops_context *ctx, int m, int k, int n, int wt) {
-  return m == 3 && wt == kQ4_0 && ctx->opt.lane_order == 1 && matmul_block_pairs_fits(n, m, k, (WeightType) wt);
+  return (m == 2 || m == 3) && wt == kQ4_0 && ctx->opt.lane_order == 1 && matmul_block_pairs_fits(n, m, k, (WeightType) wt);
 }
 
 int lane_order_weights(htpops_context *ctx, const void *weight, const void *act, int m, int k, int n, int wt,

@@ -142,9 +142,11 @@ int htpops_process_message(htpops_context *ctx, struct MessageHeader *msg, size_
 int htpops_enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes);
 int htpops_finish_message(htpops_context *ctx, struct MessageHeader *msg);
 
-/* How many separately launched units the most recent walk of a message on this context issued: compute requests that
- * were grouped into one kernel launch count once (diagnostic; the reference runs one op per request,
- * src/dsp/commu.c:91-100). Grouping never changes a result: a request joins a group only if it neither reads nor
+/* How many separately submitted units the most recent walk of a message on this context issued: compute requests that
+ * were grouped count once (diagnostic; the reference runs one op per request, src/dsp/commu.c:91-100). A group is one
+ * kernel launch where all its members take the same kernel (the projections of a decoder layer do); a group of
+ * many-row matmuls adds one launch that converts the activations, and a few-row group whose members take different
+ * kernels (by shape and weight type) issues one launch per kernel. Grouping never changes a result: a request joins a group only if it neither reads nor
  * overwrites what an earlier member writes and writes nothing an earlier member reads. */
 int htpops_last_message_submissions(htpops_context *ctx);
 

@@ -313,10 +313,13 @@ def test_small_batch_repeated_launches_are_bit_identical(ctx):
 def test_two_and_three_rows_on_the_decode_kernels_weight_stream(ctx, oracle, wt, m, k, n):
     # 2 and 3 rows run the decode kernel's stream over the weights with the rows held in registers: one, two or three
     # waves per weight row (k <= 4096, <= 8192, <= 12288), rows past the last whole walk of a workgroup, one lane of a
-    # chunk only (k = 4096 + 64). Against the oracle, against the kernels they replace (HTPOPS_GEMV_ROWS_KERNEL=0), bit for bit on a repeat, and
+    # chunk only (k = 4096 + 64). HTPOPS_LANE_ORDER=0 pins that kernel (by default Q4_0 with n % 16 == 0 and
+    # k % 256 == 0 goes to the kernel over repacked weights instead). Against the oracle, bit for bit on a repeat,
     # every row against the one-row kernel (same block sums and lane mapping; the compiler is free to fuse the scale
-    # multiplications differently in the two kernels, so to rounding).
+    # multiplications differently in the two kernels, so to rounding), and against what the default switches and
+    # HTPOPS_GEMV_ROWS_KERNEL=0 choose for the same matmul.
     rng = wl.rng_for(69, wt * 1000 + m * 100 + k + n)
+    ctx.set_option("lane_order", 0)
     got, x, w = check_mat_mul(ctx, oracle, rng, m, k, n, wt)
     a = oracle.quantize_q8_0(x)
     assert np.array_equal(ctx.run_mat_mul(a, w, m, k, n, wt), got)
@@ -324,6 +327,9 @@ def test_two_and_three_rows_on_the_decode_kernels_weight_stream(ctx, oracle, wt,
     for r in range(m):
         one = ctx.run_mat_mul(a[r:r + 1], w, 1, k, n, wt)[0]
         assert np.all(np.abs(one - got[r]) <= 1e-6 * mag[r]), "row %d differs from the one-row kernel" % r
+    ctx.set_option("lane_order", 1)
+    default = ctx.run_mat_mul(a, w, m, k, n, wt)
+    assert np.all(np.abs(default - got) <= 2 * MATMUL_RTOL * mag)
     ctx.set_option("gemv_rows_kernel", 0)
     other = ctx.run_mat_mul(a, w, m, k, n, wt)
     assert np.all(np.abs(other - got) <= 2 * MATMUL_RTOL * mag)
@@ -769,8 +775,9 @@ def test_message_groups_independent_many_row_matmuls(ctx, oracle, wt):
 @pytest.mark.parametrize("m", [2, 3, 8])
 def test_message_groups_independent_few_row_matmuls(ctx, oracle, wt, m):
     # Few-row matmuls of the same k that nothing orders share a launch although they read different activation rows
-    # (2, 3 rows: the weight stream with the rows in registers; 8: the kernel over repacked weights for Q4_0, one
-    # launch per set of rows otherwise). Every request must equal its own launch bit for bit.
+    # (2, 3 rows: the weight stream with the rows in registers, or for Q4_0 members that fit it the kernel over
+    # repacked weights, one launch of each kind; 8: the kernel over repacked weights for Q4_0, one launch per set of
+    # rows otherwise). Every request must equal its own launch bit for bit.
     # With two and three rows the members may also differ in k (one, two and three waves per weight row here).
     rng = wl.rng_for(76, wt * 10 + m)
     op = api.HTP_OPS_MAT_MUL_Q4_0_Q8_0 if wt == wl.GGML_TYPE_Q4_0 else api.HTP_OPS_MAT_MUL_Q8_0_Q8_0
