@@ -450,7 +450,40 @@ struct RequestHeader *attention_output_quantizer(htpops_context *ctx, const stru
 
 }  // namespace
 
+// How many bytes of parameters the op of a compute request reads behind its OpComputeRequest; 0 for an op the
+// dispatcher does not know (it reports that itself). The reference casts without looking (op_executor.cc:52-204): a
+// request shorter than its op's parameters would make the dispatcher read past it, past the end of the message for
+// the last one.
+static size_t op_payload_bytes(uint32_t op) {
+  switch (op) {
+    case HTP_OPS_RMS_NORM_F32:
+    case HTP_OPS_QUANTIZE_Q8_0:
+      return sizeof(RmsNormF32Params);
+    case HTP_OPS_RMS_NORM_F32_EX:
+    case HTP_OPS_RMS_NORM_QUANTIZE_Q8_0:
+      return sizeof(RmsNormExParams);
+    case HTP_OPS_MAT_MUL_PERMUTED_W16A32:
+    case HTP_OPS_MAT_MUL_PERMUTED_W4D16A32:
+    case HTP_OPS_MAT_MUL_PERMUTED_W8D16A32:
+    case HTP_OPS_MAT_MUL_PERMUTED_W4D16A32_IQ4_NL:
+    case HTP_OPS_MAT_MUL_Q4_0_Q8_0:
+    case HTP_OPS_MAT_MUL_Q8_0_Q8_0:
+    case HTP_OPS_MAT_MUL_Q4_0_A32:
+    case HTP_OPS_MAT_MUL_Q8_0_A32:
+      return sizeof(MatMulParams);
+    case HTP_OPS_FLASH_ATTN_QO_F32_KV_F16:
+      return sizeof(FlashAttnParams);
+    case HTP_OPS_FLASH_ATTN_F16:
+      return sizeof(FlashAttnExParams);
+    default:
+      return 0;
+  }
+}
+
 int check_message_framing(htpops_context *ctx, const struct MessageHeader *msg, size_t msg_bytes) {
+  if (msg_bytes && msg_bytes < sizeof(struct MessageHeader)) {
+    return fail(ctx, HTPOPS_ERR_REJECTED, "message: %zu bytes do not hold a header", msg_bytes);
+  }
   const int n_reqs = msg->n_reqs;
   if (n_reqs < 0 || n_reqs > (1 << 20)) {
     return fail(ctx, HTPOPS_ERR_REJECTED, "message: n_reqs=%d", n_reqs);
@@ -492,6 +525,12 @@ int enqueue_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_b
           hdr->state = HTPOPS_ERR_REJECTED;
         } else {
           const auto *req = reinterpret_cast<const struct OpComputeRequest *>(hdr->data);
+          if (size < sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest) + op_payload_bytes(req->op)) {
+            flush_batch(ctx, batch);
+            hdr->state = fail(ctx, HTPOPS_ERR_REJECTED, "message: request %d is shorter than the parameters of op %u", i,
+                              req->op);
+            break;
+          }
           const bool  matmul_payload =
             size >= sizeof(struct RequestHeader) + sizeof(struct OpComputeRequest) + sizeof(MatMulParams);
           const bool  norm_payload =

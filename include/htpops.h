@@ -131,8 +131,9 @@ int htpops_execute_op(htpops_context *ctx, const struct OpComputeRequest *req);
  * request in order, stores each op's return code in RequestHeader.state, honours
  * RPCMEM_MAP.n_puts as handle releases, waits for the stream, then publishes completion by
  * storing state.d = v[0] | (1 << 8). Returns 0, or a negative error if the message is malformed
- * (offsets outside `msg_bytes`; pass 0 to skip the bound check). The go byte v[0] is not
- * required to be set. */
+ * (offsets outside `msg_bytes`; pass 0 to skip the bound check). A compute request that ends before
+ * the parameter struct of its op does gets HTPOPS_ERR_REJECTED as its state and is not run (the
+ * reference casts without looking at the request's size). The go byte v[0] is not required to be set. */
 int htpops_process_message(htpops_context *ctx, struct MessageHeader *msg, size_t msg_bytes);
 
 /* The two halves of htpops_process_message, for producers that keep several messages in flight:

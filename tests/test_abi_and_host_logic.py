@@ -136,6 +136,34 @@ def test_process_message_rejects_malformed_framing(ctx):
     broken = bytearray(msg)
     struct.pack_into("<i", broken, 12, -1)
     assert ctx.process_message(broken) == api.HTPOPS_ERR_REJECTED
+    assert ctx.process_message(bytearray(msg[:12])) == api.HTPOPS_ERR_REJECTED  # not even a header
+
+
+def test_process_message_rejects_requests_shorter_than_their_parameters(ctx):
+    # The reference casts a request's bytes to its op's parameter struct without looking at the request's size
+    # (op_executor.cc:52-204); here a compute request that ends before its op's parameters do is refused with its own
+    # state, the requests around it run, and nothing behind the request is read (for the last request that would be
+    # memory behind the message).
+    src, dst = ctx.alloc(256), ctx.alloc(256)
+    good = api.op_compute_request(api.HTP_OPS_RMS_NORM_F32, api.rms_norm_params((dst, 0), (src, 0), 64, 1))
+    bodies = {
+        api.HTP_OPS_RMS_NORM_F32: good,
+        api.HTP_OPS_MAT_MUL_Q4_0_Q8_0: api.op_compute_request(api.HTP_OPS_MAT_MUL_Q4_0_Q8_0, api.mat_mul_params((dst, 0), (src, 0), (src, 0), 1, 32, 1)),
+        api.HTP_OPS_MAT_MUL_PERMUTED_W16A32: api.op_compute_request(api.HTP_OPS_MAT_MUL_PERMUTED_W16A32, api.mat_mul_params((dst, 0), (src, 0), (src, 0), 1, 32, 32)),
+        api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16: api.op_compute_request(api.HTP_OPS_FLASH_ATTN_QO_F32_KV_F16, b"\0" * 60),
+        api.HTP_OPS_FLASH_ATTN_F16: api.op_compute_request(api.HTP_OPS_FLASH_ATTN_F16, b"\0" * 64),
+        api.HTP_OPS_RMS_NORM_QUANTIZE_Q8_0: api.op_compute_request(api.HTP_OPS_RMS_NORM_QUANTIZE_Q8_0, b"\0" * 36),
+    }
+    for op, body in bodies.items():
+        for cut in (1, 4, len(body) - 4):  # one byte short, one field short, the op word alone
+            msg = api.build_message([(api.REQUEST_TYPE_OP_COMPUTE, good), (api.REQUEST_TYPE_OP_COMPUTE, body[:len(body) - cut])])
+            assert ctx.process_message(msg) == 0
+            states = api.message_request_states(msg)
+            assert states == [api.HTPOPS_ERR_NO_DEVICE, api.HTPOPS_ERR_REJECTED], (op, cut, states)
+            assert "shorter than the parameters" in ctx.last_error()
+        whole = api.build_message([(api.REQUEST_TYPE_OP_COMPUTE, body)])
+        assert ctx.process_message(whole) == 0
+        assert "shorter than the parameters" not in ctx.last_error()
 
 
 def test_channel_poller_follows_the_state_byte_protocol(ctx, lib):
