@@ -1030,7 +1030,7 @@ def test_message_decode_chain_keeps_its_own_launch_when_it_must(ctx, oracle):
 def test_message_batching_equals_one_request_at_a_time(ctx, seed):
     # Random programs over a small pool of buffers, so that requests read what earlier ones wrote, overwrite what earlier
     # ones read, and write the same bytes twice: RMSNorm -> Q8_0 (op 13), Q8_0 quantization (op 14) and matmuls of 1, 2,
-    # 8 and 64 rows whose outputs feed later norms -- or land on Q8_0 rows that later matmuls read as they are (whatever
+    # 3, 5, 8 and 64 rows whose outputs feed later norms -- or land on Q8_0 rows that later matmuls read as they are (whatever
     # those bytes mean as blocks: both walks must agree on every byte, NaNs included). The walk of ONE message (which
     # shares launches where it may) must leave every buffer exactly as one message per request does, where nothing can
     # share.
@@ -1050,7 +1050,7 @@ def test_message_batching_equals_one_request_at_a_time(ctx, seed):
         reqs = []
         for _ in range(16):
             kind = rng.integers(0, 10)
-            m = int(rng.choice([1, 1, 1, 1, 2, 8, 64]))
+            m = int(rng.choice([1, 1, 1, 1, 2, 3, 5, 8, 64]))
             row = int(rng.integers(0, rows - m + 1))          # requests work on rows row .. row + m - 1 of their buffers
             f, q = int(rng.integers(0, len(hf))), int(rng.integers(0, len(hq)))
             if kind < 3:
