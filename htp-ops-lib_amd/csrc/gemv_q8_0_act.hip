@@ -21,6 +21,8 @@
 
 #include <stdlib.h>
 
+#include <algorithm>
+
 namespace htpops {
 
 namespace {
@@ -939,14 +941,27 @@ hipError_t launch_gemv_group_q8_0_act(hipStream_t stream, int count, float *cons
   }
   GemvMembers grp = {};
   grp.count       = count;
+  // The members are laid out over the workgroups in order of their size, largest first:
+  // workgroups start in index order, and a launch that ends with the workgroups of its small matrices ends sooner
+  // than one that ends with those of a large one (a 7B layer's seven projections: 19.9 us as gate, up, down, q, k, v, o
+  // against 20.2 us as q, k, v, o, gate, up, down). A member's own workgroups and sums do not depend on its place.
+  int order[kGemvGroupMax];
   for (int i = 0; i < count; ++i) {
+    order[i] = i;
+  }
+  std::stable_sort(order, order + count, [&](int a, int b) {
+    const long sa = (long) ns[a] * ks[a], sb = (long) ns[b] * ks[b];
+    return sa != sb ? sa > sb : ks[a] < ks[b];  // (equal sizes: the shorter rows first -- gate, down, up measured 20.5 us)
+  });
+  for (int j = 0; j < count; ++j) {
+    const int i    = order[j];
     const int nblk = ks[i] / kQK;
     if (ks[i] % (2 * kQK) != 0 || nblk / 2 > kSharedActMaxPairs ||
         ((reinterpret_cast<uintptr_t>(weights[i]) | reinterpret_cast<uintptr_t>(acts[i])) & 3) != 0) {
       return hipErrorNotSupported;
     }
-    grp.m[i].w = static_cast<const uint32_t *>(weights[i]), grp.m[i].act = static_cast<const uint32_t *>(acts[i]);
-    grp.m[i].out = outs[i], grp.m[i].n = ns[i], grp.m[i].pairs = nblk / 2;
+    grp.m[j].w = static_cast<const uint32_t *>(weights[i]), grp.m[j].act = static_cast<const uint32_t *>(acts[i]);
+    grp.m[j].out = outs[i], grp.m[j].n = ns[i], grp.m[j].pairs = nblk / 2;
   }
   return wt == kQ4_0 ? launch_gemv_members<kQ4_0>(stream, grp) : launch_gemv_members<kQ8_0>(stream, grp);
 }
